@@ -1,0 +1,60 @@
+"""Builds libcascmm.so (HIP, gfx950 only) in-tree with hipcc.
+
+    python -m basedxl_amd.build
+
+Every .hip file under csrc/ is one translation unit; they are compiled in parallel and
+linked into basedxl_amd/libcascmm.so, which the ctypes loader in _lib.py opens.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
+LIB = os.path.join(HERE, "libcascmm.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
+    # packed fp32 VALU ops are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def sources():
+    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _compile(src: str) -> str:
+    obj = os.path.join(OBJ, src[:-4] + ".o")
+    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "warning generated" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(verbose: bool = True, jobs: int = 8) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=min(jobs, len(srcs))) as ex:
+        objs = list(ex.map(_compile, srcs))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print(f"built {LIB} from {len(srcs)} translation units")
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,161 @@
+"""cascaded_lowp_matmul for MI355X: same call surface as the reference operator
+(basedxl/triton/cascaded_lowp_matmul.py:139-173), arithmetic done by hand-written gfx950
+kernels behind the C ABI of include/cascmm.h.
+
+The operands are split on the fly into ``terms`` low-precision terms (``lowp``), the kept
+partial products run on MFMA with fp32 accumulation and are summed in registers.
+
+Differences from the reference wrapper, all behind keyword-only arguments with defaults:
+  * ``lowp`` / ``terms`` / ``products`` choose the cascade (default: two bf16 terms, the
+    three products hi.hi + hi.lo + lo.hi);
+  * ``bias`` fuses the ``x + bias`` that basedxl/modules/lowp_linear.py:17-19 does separately;
+  * there is no torch.matmul fallback for small shapes (:155-156): every shape, including
+    M = 154 text tokens, runs the HIP kernels, and a batched ``b`` loops over its batch.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.DT_F32, torch.float16: _lib.DT_F16, torch.bfloat16: _lib.DT_BF16}
+
+#: persistent zero-initialised split-K workspaces, one per (device index, stream handle)
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, stream: int, nbytes: int) -> Optional[torch.Tensor]:
+    if nbytes == 0:
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _check_device_tensor(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"cascaded_lowp_matmul: {name} is on {t.device}; the operator only runs on an AMD GPU "
+            "(there is no CPU fallback)")
+
+
+def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optional[torch.Tensor],
+             fmt: int, terms: int, products: int, variant: int) -> None:
+    M, K = a2.shape
+    N = b2.shape[1]
+    dt = _DTYPES[a2.dtype]
+    l = _lib.lib()
+    stream = torch.cuda.current_stream(a2.device).cuda_stream
+    ws_bytes = l.cascmm_workspace_bytes(M, N, K, dt, fmt, terms, products)
+    ws = _workspace(a2.device, stream, ws_bytes)
+    exps = None
+    if fmt == _lib.FMT_FP8:
+        exps = torch.empty(2, dtype=torch.int32, device=a2.device)
+        _lib.check(l.cascmm_tensor_exp(a2.data_ptr(), M, K, a2.stride(0), dt, exps.data_ptr(), stream),
+                   "cascmm_tensor_exp(A)")
+        _lib.check(l.cascmm_tensor_exp(b2.data_ptr(), K, N, b2.stride(0), dt, exps.data_ptr() + 4, stream),
+                   "cascmm_tensor_exp(B)")
+    st = l.cascmm_gemm_variant(
+        a2.data_ptr(), b2.data_ptr(), out2.data_ptr(), bias.data_ptr() if bias is not None else None,
+        M, N, K, a2.stride(0) if M > 1 else max(K, 1), b2.stride(0) if K > 1 else max(N, 1),
+        out2.stride(0) if M > 1 else max(N, 1),
+        dt, fmt, terms, products,
+        exps.data_ptr() if exps is not None else None,
+        ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+        stream, variant)
+    _lib.check(st, "cascmm_gemm")
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """2-D view whose rows are contiguous (row stride free); copies only when it must."""
+    if t.stride(-1) != 1 and t.shape[-1] > 1:
+        return t.contiguous()
+    if t.shape[0] > 1 and t.stride(0) < t.shape[1]:
+        return t.contiguous()
+    return t
+
+
+def cascaded_lowp_matmul(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    *,
+    out: Optional[torch.Tensor] = None,
+    dump_ptx: bool = False,
+    lowp: str = "bf16",
+    terms: int = 2,
+    products: str = "tri",
+    bias: Optional[torch.Tensor] = None,
+    variant: int = -1,
+) -> torch.Tensor:
+    assert a.shape[-1] == b.shape[-2], "Incompatible dimensions"
+    # assert a.is_contiguous(), "Matrix A must be contiguous"
+    assert b.is_contiguous(), "Matrix B must be contiguous"
+    _check_device_tensor(a, "a")
+    _check_device_tensor(b, "b")
+    if a.dtype not in _DTYPES:
+        raise TypeError(f"cascaded_lowp_matmul: unsupported dtype {a.dtype}")
+    if b.dtype != a.dtype:
+        raise TypeError(f"cascaded_lowp_matmul: a is {a.dtype} but b is {b.dtype}")
+    if lowp not in _lib.FMT_BY_NAME:
+        raise ValueError(f"lowp must be one of {sorted(_lib.FMT_BY_NAME)}, got {lowp!r}")
+    if products not in _lib.PROD_BY_NAME:
+        raise ValueError(f"products must be 'tri' or 'full', got {products!r}")
+    fmt, prod = _lib.FMT_BY_NAME[lowp], _lib.PROD_BY_NAME[products]
+    if bias is not None:
+        _check_device_tensor(bias, "bias")
+        if bias.dtype != a.dtype or bias.dim() != 1 or bias.shape[0] != b.shape[-1]:
+            raise ValueError("bias must be a 1-D tensor of length N with the dtype of a")
+        bias = bias.contiguous()
+
+    K, N = b.shape[-2], b.shape[-1]
+
+    if b.dim() > 2:
+        # batched right operand: torch.matmul broadcasting, one GEMM per batch entry
+        if a.dim() < 2:
+            raise ValueError("a must have at least 2 dims when b is batched")
+        batch = torch.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+        rows = a.shape[-2]
+        a_b = a.expand(*batch, rows, K).reshape(-1, rows, K)
+        b_b = b.expand(*batch, K, N).reshape(-1, K, N)
+        res = out if out is not None else torch.empty((*batch, rows, N), device=a.device, dtype=a.dtype)
+        if tuple(res.shape) != (*batch, rows, N) or not res.is_contiguous():
+            raise ValueError("out must be a contiguous tensor of the broadcast result shape")
+        res_b = res.view(-1, rows, N)
+        for i in range(a_b.shape[0]):
+            _gemm_2d(_rows(a_b[i]), b_b[i].contiguous(), res_b[i], bias, fmt, terms, prod, variant)
+        return res
+
+    batch_dims = a.shape[:-1]
+    M = batch_dims.numel()
+    a2 = _rows(a.reshape(M, K))
+
+    if out is None:
+        out = torch.empty((M, N), device=a.device, dtype=a.dtype)
+    else:
+        _check_device_tensor(out, "out")
+        if out.dtype != a.dtype:
+            raise TypeError("out must have the dtype of a")
+        if out.numel() != M * N:
+            raise ValueError(f"out has {out.numel()} elements, expected {M * N}")
+    out2 = out if out.dim() == 2 and out.shape == (M, N) else out.view(M, N)
+    if N > 1 and out2.stride(1) != 1:
+        raise ValueError("out must have unit stride along N")
+
+    _gemm_2d(a2, b, out2, bias, fmt, terms, prod, variant)
+
+    if dump_ptx:
+        # the reference writes the kernel's PTX (cascaded_lowp_matmul.py:170-171); there is no
+        # PTX here, so the file names the gfx950 kernel variant that ran instead
+        l = _lib.lib()
+        v = variant if variant >= 0 else l.cascmm_select_variant(
+            M, N, K, a2.stride(0), b.stride(0), out2.stride(0), _DTYPES[a.dtype], fmt, terms, prod)
+        name = l.cascmm_variant_name(v)
+        with open("dump.ptx", "w") as f:
+            f.write(f"// gfx950 kernel variant: {name.decode() if name else v}\n")
+
+    return out.reshape(*batch_dims, N)

@@ -1,0 +1,246 @@
+// extern "C" entry points: argument checks, kernel selection, small utility kernels.
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "cascmm_variants.h"
+
+namespace cascmm {
+
+// ---------------------------------------------------------------------------------------
+// variant table (immutable after first use)
+// ---------------------------------------------------------------------------------------
+static const std::vector<VariantDesc>& table() {
+  static const std::vector<VariantDesc> t = [] {
+    std::vector<VariantDesc> v;
+    int n = 0;
+    const VariantDesc* p = variants_bf16(&n);
+    v.insert(v.end(), p, p + n);
+    p = variants_fp16(&n);
+    v.insert(v.end(), p, p + n);
+    return v;
+  }();
+  return t;
+}
+
+static bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+static size_t dtype_size(int dt) { return dt == CASCMM_DT_F32 ? 4 : 2; }
+
+struct Problem {
+  int64_t M, N, K, lda, ldb, ldc;
+  int dtype, fmt, terms, products;
+};
+
+static int check_problem(const Problem& q) {
+  if (q.dtype != CASCMM_DT_F32 && q.dtype != CASCMM_DT_F16 && q.dtype != CASCMM_DT_BF16) return CASCMM_ERR_BAD_DTYPE;
+  if (q.fmt != CASCMM_FMT_BF16 && q.fmt != CASCMM_FMT_FP16 && q.fmt != CASCMM_FMT_FP8) return CASCMM_ERR_BAD_FORMAT;
+  if (q.terms < 1 || q.terms > 3) return CASCMM_ERR_BAD_FORMAT;
+  if (q.products != CASCMM_PROD_TRI && q.products != CASCMM_PROD_FULL) return CASCMM_ERR_BAD_FORMAT;
+  if (q.M < 0 || q.N < 0 || q.K < 0) return CASCMM_ERR_BAD_SHAPE;
+  if (q.M > INT32_MAX || q.N > INT32_MAX || q.K > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (q.lda < q.K || q.ldb < q.N || q.ldc < q.N) return CASCMM_ERR_BAD_SHAPE;
+  return CASCMM_OK;
+}
+
+// what the fast (buffer-load, no K tail) kernels need apart from K % BK == 0
+static bool fast_ok(const Problem& q, const void* A) {
+  return q.dtype == CASCMM_DT_F32 && q.lda % 4 == 0 && (A == nullptr || aligned_to(A, 16)) &&
+         q.lda * 4 * 512 < INT32_MAX && q.ldb * 4 * 136 < INT32_MAX;  // 32-bit byte offsets inside a tile
+}
+
+static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
+  const int full = (q.products == CASCMM_PROD_FULL && q.terms > 1) ? 1 : 0;
+  if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full) return false;
+  if (v.fast && (!fast || q.K % v.BK != 0)) return false;
+  return true;
+}
+
+// Cost model: time ~ rounds over the 256 CUs x per-tile time, where a tile costs its MFMA
+// work (BM*BN) plus a staging term proportional to the operand rows it has to load, split
+// and write to LDS per k (BM+BN).  Constants fitted on MI355X measurements.
+static double variant_cost(const VariantDesc& v, const Problem& q) {
+  const double tiles = (double)((q.M + v.BM - 1) / v.BM) * (double)((q.N + v.BN - 1) / v.BN);
+  const double slots = 256.0;
+  const double rounds = (double)(int64_t)((tiles + slots - 1) / slots);
+  const double per_tile = (double)v.BM * v.BN + 64.0 * (v.BM + v.BN);
+  return rounds * per_tile + (v.fast ? 0.0 : 1e-3);
+}
+
+static int select_variant(const Problem& q, const void* A) {
+  const bool fast = fast_ok(q, A);
+  const auto& t = table();
+  int best = -1;
+  double best_cost = 0;
+  for (int i = 0; i < (int)t.size(); ++i) {
+    if (!variant_matches(t[i], q, fast)) continue;
+    const double c = variant_cost(t[i], q);
+    if (best < 0 || c < best_cost) { best = i; best_cost = c; }
+  }
+  return best < 0 ? (int)CASCMM_ERR_BAD_FORMAT : best;
+}
+
+// ---------------------------------------------------------------------------------------
+// utility kernels
+// ---------------------------------------------------------------------------------------
+template <int IODT>
+__global__ void fill_bias_kernel(void* C, const void* bias, int M, int N, int64_t ldc) {
+  typedef typename IoType<IODT>::T T;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)M * N) return;
+  const int r = (int)(i / N), c = (int)(i % N);
+  IoType<IODT>::store((T*)C + (int64_t)r * ldc + c, bias ? IoType<IODT>::load((const T*)bias + c) : 0.f);
+}
+
+template <int IODT, int FMT, int TERMS>
+__global__ void split_terms_kernel(const void* x, float* out, int64_t n, int tensor_exp) {
+  typedef typename IoType<IODT>::T T;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float r[8];
+  r[0] = IoType<IODT>::load((const T*)x + i) * __builtin_ldexpf(1.0f, tensor_exp);
+#pragma unroll
+  for (int e = 1; e < 8; ++e) r[e] = 0.f;
+  u32x4 t[TERMS];
+  split8<FMT, TERMS>(r, t);
+#pragma unroll
+  for (int k = 0; k < TERMS; ++k) {
+    typename Lowp<FMT>::Vec v = __builtin_bit_cast(typename Lowp<FMT>::Vec, t[k]);
+    out[(int64_t)k * n + i] = (float)v[0];
+  }
+}
+
+template <int IODT, int FMT>
+static int launch_split(const void* x, float* out, int64_t n, int terms, int tensor_exp, hipStream_t s) {
+  const unsigned grid = (unsigned)((n + 255) / 256);
+  switch (terms) {
+    case 1: hipLaunchKernelGGL((split_terms_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
+    case 2: hipLaunchKernelGGL((split_terms_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
+    case 3: hipLaunchKernelGGL((split_terms_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
+    default: return CASCMM_ERR_BAD_FORMAT;
+  }
+  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+}
+
+static int gemm_impl(const void* A, const void* B, void* C, const void* bias, const Problem& q,
+                     const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream, int variant) {
+  int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  if (q.M == 0 || q.N == 0) return CASCMM_OK;
+  if (!C) return CASCMM_ERR_NULL_POINTER;
+  const size_t es = dtype_size(q.dtype);
+  if (!aligned_to(C, es) || !aligned_to(bias, es)) return CASCMM_ERR_ALIGNMENT;
+  if (q.K == 0) {
+    const int64_t total = q.M * q.N;
+    const unsigned grid = (unsigned)((total + 255) / 256);
+    if (q.dtype == CASCMM_DT_F32)
+      hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, stream, C, bias, (int)q.M, (int)q.N, q.ldc);
+    else if (q.dtype == CASCMM_DT_F16)
+      hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, stream, C, bias, (int)q.M, (int)q.N, q.ldc);
+    else
+      hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, stream, C, bias, (int)q.M, (int)q.N, q.ldc);
+    return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  }
+  if (!A || !B) return CASCMM_ERR_NULL_POINTER;
+  if (!aligned_to(A, es) || !aligned_to(B, es)) return CASCMM_ERR_ALIGNMENT;
+
+  const auto& t = table();
+  if (variant < 0) {
+    variant = select_variant(q, A);
+    if (variant < 0) return variant;
+  } else {
+    if (variant >= (int)t.size()) return CASCMM_ERR_BAD_VARIANT;
+    if (!variant_matches(t[variant], q, fast_ok(q, A))) return CASCMM_ERR_BAD_VARIANT;
+  }
+  const VariantDesc& v = t[variant];
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = A; p.B = B; p.C = C; p.bias = bias;
+  p.M = (int)q.M; p.N = (int)q.N; p.K = (int)q.K;
+  p.lda = q.lda; p.ldb = q.ldb; p.ldc = q.ldc;
+  const int64_t tm = (q.M + v.BM - 1) / v.BM, tn = (q.N + v.BN - 1) / v.BN;
+  if (tm * tn > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  p.tiles_m = (int)tm; p.tiles_n = (int)tn;
+  p.tensor_exps = tensor_exps;
+  (void)workspace; (void)workspace_bytes;
+  return v.launch(p, stream);
+}
+
+}  // namespace cascmm
+
+using namespace cascmm;
+
+extern "C" {
+
+int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt, int terms, int products,
+                        const int32_t* tensor_exps, void* workspace, size_t workspace_bytes, void* stream,
+                        int variant) {
+  const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  return gemm_impl(A, B, C, bias, q, tensor_exps, workspace, workspace_bytes, (hipStream_t)stream, variant);
+}
+
+int cascmm_gemm(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K, int64_t lda,
+                int64_t ldb, int64_t ldc, int dtype, int fmt, int terms, int products, const int32_t* tensor_exps,
+                void* workspace, size_t workspace_bytes, void* stream) {
+  return cascmm_gemm_variant(A, B, C, bias, M, N, K, lda, ldb, ldc, dtype, fmt, terms, products, tensor_exps,
+                             workspace, workspace_bytes, stream, -1);
+}
+
+size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms, int products) {
+  (void)M; (void)N; (void)K; (void)dtype; (void)fmt; (void)terms; (void)products;
+  return 0;
+}
+
+int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt,
+                          int terms, int products) {
+  const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  return select_variant(q, nullptr);
+}
+
+int cascmm_variant_count(void) { return (int)table().size(); }
+
+const char* cascmm_variant_name(int variant) {
+  if (variant < 0 || variant >= (int)table().size()) return nullptr;
+  return table()[variant].name;
+}
+
+int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, int32_t* exp_out,
+                      void* stream) {
+  (void)x; (void)rows; (void)cols; (void)ld; (void)dtype; (void)exp_out; (void)stream;
+  return CASCMM_ERR_BAD_FORMAT;
+}
+
+int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms, int tensor_exp,
+                       void* stream) {
+  if (n < 0) return CASCMM_ERR_BAD_SHAPE;
+  if (n == 0) return CASCMM_OK;
+  if (!x || !out) return CASCMM_ERR_NULL_POINTER;
+  if (dtype != CASCMM_DT_F32) return CASCMM_ERR_BAD_DTYPE;
+  hipStream_t s = (hipStream_t)stream;
+  if (fmt == CASCMM_FMT_BF16) return launch_split<CASCMM_DT_F32, CASCMM_FMT_BF16>(x, out, n, terms, tensor_exp, s);
+  if (fmt == CASCMM_FMT_FP16) return launch_split<CASCMM_DT_F32, CASCMM_FMT_FP16>(x, out, n, terms, tensor_exp, s);
+  return CASCMM_ERR_BAD_FORMAT;
+}
+
+const char* cascmm_strerror(int status) {
+  switch (status) {
+    case CASCMM_OK: return "ok";
+    case CASCMM_ERR_NULL_POINTER: return "null pointer argument";
+    case CASCMM_ERR_BAD_SHAPE: return "bad shape or leading dimension";
+    case CASCMM_ERR_BAD_DTYPE: return "unsupported element type";
+    case CASCMM_ERR_BAD_FORMAT: return "unsupported format / terms / products combination";
+    case CASCMM_ERR_WORKSPACE: return "workspace missing or too small";
+    case CASCMM_ERR_ALIGNMENT: return "pointer not aligned to its element size";
+    case CASCMM_ERR_LAUNCH: return "HIP launch failed";
+    case CASCMM_ERR_BAD_VARIANT: return "kernel variant unknown or unable to run this problem";
+    case CASCMM_ERR_TOO_LARGE: return "dimension too large";
+    default: return "unknown status";
+  }
+}
+
+int cascmm_version(void) { return CASCMM_VERSION; }
+
+}  // extern "C"

@@ -1,0 +1,135 @@
+// Shared device/host helpers of the cascaded low-precision matmul kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/cascmm.h"
+
+namespace cascmm {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------------------
+// memory element types (what A, B, C, bias are stored as)
+// ---------------------------------------------------------------------------------------
+template <int DT> struct IoType;
+template <> struct IoType<CASCMM_DT_F32> {
+  typedef float T;
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct IoType<CASCMM_DT_F16> {
+  typedef _Float16 T;
+  static __device__ __forceinline__ float load(const _Float16* p) { return (float)*p; }
+  static __device__ __forceinline__ void store(_Float16* p, float v) { *p = (_Float16)v; }
+};
+template <> struct IoType<CASCMM_DT_BF16> {
+  typedef __bf16 T;
+  static __device__ __forceinline__ float load(const __bf16* p) { return (float)*p; }
+  static __device__ __forceinline__ void store(__bf16* p, float v) { *p = (__bf16)v; }
+};
+
+// ---------------------------------------------------------------------------------------
+// low-precision term formats: rounding, term scaling, packing of 8 values into one 16-byte
+// LDS slot (bf16 / fp16) and the MFMA that consumes two such slots.
+//   r_0 = x;  t_i = lowp(r_i * 2^(shift*i));  r_{i+1} = r_i - t_i * 2^(-shift*i)
+// Both the scaling and the residual are exact in fp32 (power-of-two scale, and the
+// residual of a round-to-nearest needs fewer significand bits than fp32 has).
+// ---------------------------------------------------------------------------------------
+template <int FMT> struct Lowp;
+
+template <> struct Lowp<CASCMM_FMT_BF16> {
+  static constexpr int kShift = 0;
+  typedef bf16x8 Vec;
+  static __device__ __forceinline__ f32x16 mfma(Vec a, Vec b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  // round 8 residuals to the format, update the residuals, return the packed slot
+  template <int TERM, bool LAST>
+  static __device__ __forceinline__ u32x4 peel(float (&r)[8]) {
+    Vec v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      __bf16 t = (__bf16)r[e];
+      v[e] = t;
+      if (!LAST) r[e] = r[e] - (float)t;
+    }
+    return __builtin_bit_cast(u32x4, v);
+  }
+};
+
+template <> struct Lowp<CASCMM_FMT_FP16> {
+  static constexpr int kShift = 11;
+  typedef f16x8 Vec;
+  static __device__ __forceinline__ f32x16 mfma(Vec a, Vec b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  template <int TERM, bool LAST>
+  static __device__ __forceinline__ u32x4 peel(float (&r)[8]) {
+    constexpr float s = (float)(1u << (kShift * TERM > 30 ? 30 : kShift * TERM));
+    constexpr float inv = 1.0f / s;
+    Vec v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      _Float16 t = (_Float16)(r[e] * s);
+      v[e] = t;
+      if (!LAST) r[e] = __builtin_fmaf(-(float)t, inv, r[e]);
+    }
+    return __builtin_bit_cast(u32x4, v);
+  }
+};
+
+template <int FMT, int TERMS>
+__device__ __forceinline__ void split8(float (&r)[8], u32x4 (&out)[TERMS]) {
+  out[0] = Lowp<FMT>::template peel<0, TERMS == 1>(r);
+  if constexpr (TERMS > 1) out[1] = Lowp<FMT>::template peel<1, TERMS == 2>(r);
+  if constexpr (TERMS > 2) out[2] = Lowp<FMT>::template peel<2, TERMS == 3>(r);
+}
+
+// scale class of product (i, j) is i + j; products kept: i + j <= TERMS-1 (tri) or all (full)
+template <int TERMS, bool FULL> struct ProductSet {
+  static constexpr int kClasses = FULL ? (2 * TERMS - 1) : TERMS;
+  static constexpr __host__ __device__ bool keep(int i, int j) { return FULL || (i + j <= TERMS - 1); }
+  static constexpr int count() {
+    int n = 0;
+    for (int i = 0; i < TERMS; ++i)
+      for (int j = 0; j < TERMS; ++j) n += keep(i, j) ? 1 : 0;
+    return n;
+  }
+};
+
+// Accumulators.  Products of scale class s = i + j carry the factor 2^(-shift*s), so formats
+// with a term shift need one accumulator per class.  bf16 terms are unscaled: one accumulator
+// serves two terms (the dropped lo.lo product dominates the error there), but with three
+// terms the result is at the fp32 rounding floor, and adding the small classes into the big
+// hi.hi sum would round it once per MFMA; the classes are kept apart and added once at the end.
+template <int FMT, int TERMS, bool FULL> struct AccClasses {
+  static constexpr bool kScaled = Lowp<FMT>::kShift != 0;
+  static constexpr int kCount = kScaled ? ProductSet<TERMS, FULL>::kClasses : (TERMS >= 3 ? 3 : 1);
+  static constexpr float kFoldScale = kScaled ? 1.0f / (float)(1 << Lowp<FMT>::kShift) : 1.0f;
+  static constexpr __host__ __device__ int index(int s) { return kCount == 1 ? 0 : (s < kCount ? s : kCount - 1); }
+};
+
+struct GemmParams {
+  const void* A;
+  const void* B;
+  void* C;
+  const void* bias;
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  int tiles_m, tiles_n;
+  int k_splits;          // split-K path only
+  int k_per_split;       // split-K path only (multiple of the kernel's BK)
+  float* partials;       // split-K workspace: [k_splits][M][N] fp32 after the counters
+  unsigned* counters;    // split-K arrival counters, one per output tile
+  const int32_t* tensor_exps;
+};
+
+}  // namespace cascmm

@@ -1,0 +1,401 @@
+// LDS-tiled MFMA kernel of the cascade GEMM (gfx950).
+//
+// One workgroup computes a BM x BN tile of C.  Per K step of BK:
+//   global (row-major)  --VGPR: split into TERMS low-precision terms-->  LDS  -->  MFMA
+// Both operands are staged in LDS already split, in "slot" form: one 16-byte slot holds 8
+// consecutive-k values of one row (A) or one column (B) of one term, i.e. exactly what one
+// lane feeds to v_mfma_f32_32x32x16 (lane l: row/col l%32, k-group l/32).  A plane is all
+// slots of one k-group, BM (or BN) slots long; 16 consecutive lanes of a fragment read
+// therefore fetch 256 contiguous bytes and planes start at multiples of 256 bytes, which is
+// what the 64-bank LDS needs for full-rate ds_read_b128.  A-side stores come from lanes
+// that walk k fastest (coalesced global loads), so rows are XOR-swizzled per k-group to keep
+// eight consecutive lanes on eight different 16-byte bank groups.
+//
+// The 32x32x16 MFMA is used rather than 16x16x32: it sustains a higher rate on this part and,
+// more important here, leaves room for about six other VALU instructions per MFMA (the
+// 16x16x32 form leaves two), which is what hides the three VALU operations per element that
+// the operand split costs.
+//
+// Global loads are raw buffer loads: the per-lane offset is fixed for the whole K loop and the
+// K position is a scalar offset, so the loop spends no VALU work on addresses.  Rows and
+// columns past the matrix edge are clamped to the last valid one (their results are never
+// stored).  Each thread keeps DEPTH K-steps of operands in flight in registers (a ring
+// indexed by compile-time constants), the LDS stage is double buffered, and there is one
+// barrier per K step.
+//
+// Waves are arranged WM x WN x WK.  With WK = 2 the two wave groups take alternate 16-wide
+// k slices of every stage and their accumulators are added through LDS at the end.
+//
+// All partial products of one (m-tile, n-tile) reuse the same fragments in registers; the
+// cross-term sum happens in the accumulator registers (one accumulator per scale class).
+#pragma once
+#include "cascmm_common.h"
+
+namespace cascmm {
+
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2>
+struct Tile {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, WK = WK_, DEPTH = DEPTH_;
+  static constexpr int NT = WM * WN * WK * kWave;
+  static constexpr int KG = BK / 8;          // k-groups (planes) per stage
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
+  static constexpr int MT = WTM / 32, NTL = WTN / 32;
+  static constexpr int KSUB = BK / 16;       // MFMA k slices per stage
+  static_assert(BK == 32 || BK == 64 || BK == 128, "BK");
+  static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile must be a multiple of 32");
+  static_assert(KSUB % WK == 0, "k slices must divide evenly among the wave groups");
+  static_assert(WK == 1 || WK == 2, "WK");
+  static_assert(DEPTH >= 1 && DEPTH <= 4, "DEPTH");
+};
+
+template <class TL, int TERMS>
+struct LdsLayout {
+  // in slots (16 bytes)
+  static constexpr int kAPlane = TL::BM;
+  static constexpr int kBPlane = TL::BN;
+  static constexpr int kATerm = TL::KG * kAPlane;
+  static constexpr int kBTerm = TL::KG * kBPlane;
+  static constexpr int kStage = TERMS * (kATerm + kBTerm);
+  static constexpr int kReduce = (TL::WK > 1) ? TL::BM * TL::BN / 4 : 0;  // fp32 tile, in slots
+  static constexpr int kSlots = (2 * kStage > kReduce) ? 2 * kStage : kReduce;
+  static constexpr int kBytes = kSlots * 16;
+  // XOR applied to the row index of an A slot in k-group kg: lanes walk k-groups fastest, so
+  // 8 consecutive lanes cover 8/KG' rows x KG' k-groups (KG' = min(KG, 8)); the XOR spreads
+  // them over 8 different 16-byte bank groups.
+  static __device__ __forceinline__ int swz(int kg) { return (kg * (TL::KG >= 8 ? 1 : 8 / TL::KG)) & 7; }
+};
+
+// XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs, each with its own
+// L2: give every XCD one contiguous range of tile ids.  Inside the range, tile ids walk
+// kGroupM rows of tiles down before moving one tile to the right, so the workgroups that are
+// resident together on one XCD cover a roughly square block and share both A and B tiles in
+// that L2.
+constexpr int kGroupM = 4;
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int total = tiles_m * tiles_n;
+  const int per = total >> 3;
+  int id = bid;
+  if (bid < (per << 3)) id = (bid & 7) * per + (bid >> 3);
+  const int group = kGroupM * tiles_n;
+  const int g = id / group;
+  const int first = g * kGroupM;
+  const int rows = (tiles_m - first) < kGroupM ? (tiles_m - first) : kGroupM;
+  const int in = id - g * group;
+  tm = first + in % rows;
+  tn = in / rows;
+}
+
+// Raw buffer loads through the LLVM intrinsics: address = base + voffset + soffset, voffset a
+// per-lane VGPR, soffset a wave-uniform SGPR.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+__device__ float llvm_raw_buffer_load_f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.f32");
+__device__ f32x4 llvm_raw_buffer_load_v4f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
+
+// gfx9-family raw buffer descriptor: 48-bit base, stride 0, byte count, 32-bit data format
+__device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
+  const uint64_t b = (uint64_t)base;
+  i32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)((b >> 32) & 0xFFFFu));
+  r[2] = __builtin_amdgcn_readfirstlane(bytes > 0x7FFFFFFF ? 0x7FFFFFFF : (int)bytes);
+  r[3] = 0x00020000;
+  return r;
+}
+
+template <class TL, int IODT, int FMT, int TERMS, bool FULL>
+struct TileGemm {
+  typedef Lowp<FMT> LP;
+  typedef typename LP::Vec Vec;
+  typedef LdsLayout<TL, TERMS> LL;
+  typedef ProductSet<TERMS, FULL> PS;
+  typedef AccClasses<FMT, TERMS, FULL> AC;
+  typedef typename IoType<IODT>::T IoT;
+  static constexpr int ES = sizeof(IoT);
+  static constexpr int NCLS = AC::kCount;
+  static constexpr int A_UNITS = TL::KG * TL::BM, B_UNITS = TL::KG * TL::BN;
+  static constexpr int A_IT = (A_UNITS + TL::NT - 1) / TL::NT, B_IT = (B_UNITS + TL::NT - 1) / TL::NT;
+  static constexpr int D = TL::DEPTH;
+
+  struct Regs {
+    float a[A_IT][8];
+    float b[B_IT][8];
+  };
+
+  struct Ctx {
+    i32x4 ra, rb;
+    int voff_a[A_IT];   // bytes: row * lda + kg * 8
+    int voff_b[B_IT];   // bytes: kg * 8 * ldb + col
+    int lds_a[A_IT];    // slot index inside a term plane set, -1 if this thread has no such unit
+    int lds_b[B_IT];
+    int ldb_bytes;
+  };
+
+  static __device__ __forceinline__ void init_ctx(Ctx& c, const GemmParams& p, int m0, int n0) {
+    const IoT* A = (const IoT*)p.A + (int64_t)m0 * p.lda;
+    const IoT* B = (const IoT*)p.B + n0;
+    // bytes from the tile origin to the end of the matrix; rows and columns are also clamped
+    // below, so no access relies on the hardware range check
+    c.ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
+    c.rb = make_rsrc(B, ((int64_t)(p.K - 1) * p.ldb + (p.N - n0)) * ES);
+    c.ldb_bytes = (int)(p.ldb * ES);
+    const int last_row = p.M - 1 - m0, last_col = p.N - 1 - n0;
+#pragma unroll
+    for (int it = 0; it < A_IT; ++it) {
+      int u = threadIdx.x + it * TL::NT;
+      const bool mine = u < A_UNITS;
+      u = mine ? u : A_UNITS - 1;
+      const int kg = u % TL::KG, r = u / TL::KG;
+      const int rc = r < last_row ? r : last_row;
+      c.voff_a[it] = (int)((rc * p.lda + kg * 8) * ES);
+      c.lds_a[it] = mine ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
+    }
+#pragma unroll
+    for (int it = 0; it < B_IT; ++it) {
+      int u = threadIdx.x + it * TL::NT;
+      const bool mine = u < B_UNITS;
+      u = mine ? u : B_UNITS - 1;
+      const int n = u % TL::BN, kg = u / TL::BN;
+      const int nc = n < last_col ? n : last_col;
+      c.voff_b[it] = (int)((kg * 8 * p.ldb + nc) * ES);
+      c.lds_b[it] = mine ? kg * LL::kBPlane + n : -1;
+    }
+  }
+
+  // ---- global -> registers (fast path: fp32, K % BK == 0, 16-byte aligned A rows) ---------
+  static __device__ __forceinline__ void load_fast(const Ctx& c, int k0, Regs& r) {
+    const int soff_a = k0 * ES;
+#pragma unroll
+    for (int it = 0; it < A_IT; ++it) {
+      const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
+      const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        r.a[it][e] = v0[e];
+        r.a[it][4 + e] = v1[e];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int soff_b = (k0 + e) * c.ldb_bytes;
+#pragma unroll
+      for (int it = 0; it < B_IT; ++it) r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], soff_b, 0);
+    }
+  }
+
+  // ---- global -> registers (generic: any dtype, any K, element-wise, bounds-checked) ------
+  static __device__ __forceinline__ void load_generic(const GemmParams& p, int m0, int n0, int k0, Regs& r) {
+    const IoT* A = (const IoT*)p.A;
+    const IoT* B = (const IoT*)p.B;
+#pragma unroll
+    for (int it = 0; it < A_IT; ++it) {
+      int u = threadIdx.x + it * TL::NT;
+      u = u < A_UNITS ? u : A_UNITS - 1;
+      const int kg = u % TL::KG;
+      int row = m0 + u / TL::KG;
+      row = row < p.M ? row : p.M - 1;
+      const int k = k0 + kg * 8;
+      const IoT* src = A + (int64_t)row * p.lda + k;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r.a[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + e) : 0.f;
+    }
+#pragma unroll
+    for (int it = 0; it < B_IT; ++it) {
+      int u = threadIdx.x + it * TL::NT;
+      u = u < B_UNITS ? u : B_UNITS - 1;
+      const int kg = u / TL::BN;
+      int col = n0 + u % TL::BN;
+      col = col < p.N ? col : p.N - 1;
+      const int k = k0 + kg * 8;
+      const IoT* src = B + (int64_t)k * p.ldb + col;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) r.b[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + (int64_t)e * p.ldb) : 0.f;
+    }
+  }
+
+  // ---- registers -> split -> LDS --------------------------------------------------------
+  static __device__ __forceinline__ void store(const Ctx& c, u32x4* stage, Regs& r) {
+    u32x4* sb = stage + TERMS * LL::kATerm;
+#pragma unroll
+    for (int it = 0; it < A_IT; ++it) {
+      if (A_UNITS % TL::NT != 0 && c.lds_a[it] < 0) continue;
+      u32x4 t[TERMS];
+      split8<FMT, TERMS>(r.a[it], t);
+#pragma unroll
+      for (int i = 0; i < TERMS; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+    }
+#pragma unroll
+    for (int it = 0; it < B_IT; ++it) {
+      if (B_UNITS % TL::NT != 0 && c.lds_b[it] < 0) continue;
+      u32x4 t[TERMS];
+      split8<FMT, TERMS>(r.b[it], t);
+#pragma unroll
+      for (int i = 0; i < TERMS; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+    }
+  }
+
+  // ---- LDS -> MFMA ----------------------------------------------------------------------
+  static __device__ __forceinline__ void compute(const u32x4* stage, int wm0, int wn0, int wk,
+                                                 f32x16 (&acc)[NCLS][TL::MT][TL::NTL]) {
+    const int lane = threadIdx.x & 63, l31 = lane & 31, g = lane >> 5;
+    const u32x4* sa = stage;
+    const u32x4* sb = stage + TERMS * LL::kATerm;
+#pragma unroll
+    for (int kk = 0; kk < TL::KSUB / TL::WK; ++kk) {
+      const int ks = kk * TL::WK + wk;
+      const int kg = ks * 2 + g;
+      Vec a[TERMS][TL::MT], b[TERMS][TL::NTL];
+#pragma unroll
+      for (int i = 0; i < TERMS; ++i) {
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+          a[i][mi] = __builtin_bit_cast(Vec, sa[i * LL::kATerm + kg * LL::kAPlane + wm0 + mi * 32 + (l31 ^ LL::swz(kg))]);
+#pragma unroll
+        for (int ni = 0; ni < TL::NTL; ++ni)
+          b[i][ni] = __builtin_bit_cast(Vec, sb[i * LL::kBTerm + kg * LL::kBPlane + wn0 + ni * 32 + l31]);
+      }
+      // smallest products first; consecutive MFMAs go to different accumulators
+#pragma unroll
+      for (int s = 2 * TERMS - 2; s >= 0; --s)
+#pragma unroll
+        for (int i = 0; i < TERMS; ++i) {
+          const int j = s - i;
+          if (j < 0 || j >= TERMS || !PS::keep(i, j)) continue;
+          const int cls = AC::index(s);
+#pragma unroll
+          for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < TL::NTL; ++ni) acc[cls][mi][ni] = LP::mfma(a[i][mi], b[j][ni], acc[cls][mi][ni]);
+        }
+    }
+  }
+
+  // ---- the kernel body ------------------------------------------------------------------
+  template <bool FAST>
+  static __device__ __forceinline__ void run(const GemmParams& p, u32x4* lds) {
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * TL::BM, n0 = tn * TL::BN;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wk = wave / (TL::WM * TL::WN);
+    const int wmn = wave - wk * (TL::WM * TL::WN);
+    const int wm0 = (wmn / TL::WN) * TL::WTM, wn0 = (wmn % TL::WN) * TL::WTN;
+
+    f32x16 acc[NCLS][TL::MT][TL::NTL];
+#pragma unroll
+    for (int c = 0; c < NCLS; ++c)
+#pragma unroll
+      for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < TL::NTL; ++ni)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[c][mi][ni][e] = 0.f;
+
+    Ctx ctx;
+    init_ctx(ctx, p, m0, n0);
+    Regs ring[D];
+    const int ktiles = (p.K + TL::BK - 1) / TL::BK;
+
+    // loads are only ever issued for k steps that exist (kt < ktiles)
+    auto issue = [&](int kt, Regs& r) {
+      if (FAST) load_fast(ctx, kt * TL::BK, r);
+      else load_generic(p, m0, n0, kt * TL::BK, r);
+    };
+
+    // prologue: up to DEPTH steps in flight, the first one staged
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+      if (d < ktiles) issue(d, ring[d]);
+    if (ktiles > 0) store(ctx, lds, ring[0]);
+    __syncthreads();
+
+    // step kt: refill the ring slot that step kt vacated, run the MFMAs of stage kt, stage kt+1
+    int kt = 0;
+    for (; kt + 2 * D <= ktiles; kt += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        issue(kt + d + D, ring[d]);
+        compute(lds + ((kt + d) & 1) * LL::kStage, wm0, wn0, wk, acc);
+        store(ctx, lds + ((kt + d + 1) & 1) * LL::kStage, ring[(d + 1) % D]);
+        __syncthreads();
+      }
+    }
+    // tail: fewer than 2*DEPTH steps left, nothing (or not everything) left to prefetch
+#pragma unroll
+    for (int dd = 0; dd < 2 * D; ++dd) {
+      const int d = dd % D;
+      if (kt + dd < ktiles) {
+        if (kt + dd + D < ktiles) issue(kt + dd + D, ring[d]);
+        compute(lds + ((kt + dd) & 1) * LL::kStage, wm0, wn0, wk, acc);
+        if (kt + dd + 1 < ktiles) store(ctx, lds + ((kt + dd + 1) & 1) * LL::kStage, ring[(d + 1) % D]);
+        __syncthreads();
+      }
+    }
+
+    // fold the scale classes (smallest first), then the cross-wave-group reduction (WK == 2):
+    // group 1 parks its tile in LDS, group 0 adds it
+    f32x16 res[TL::MT][TL::NTL];
+#pragma unroll
+    for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+      for (int ni = 0; ni < TL::NTL; ++ni) {
+        f32x16 v = acc[NCLS - 1][mi][ni];
+#pragma unroll
+        for (int c = NCLS - 2; c >= 0; --c) v = v * AC::kFoldScale + acc[c][mi][ni];
+        res[mi][ni] = v;
+      }
+    const int lane = threadIdx.x & 63, l31 = lane & 31, g = lane >> 5;
+    if (TL::WK > 1) {
+      f32x4* red = (f32x4*)lds + wmn * (TL::MT * TL::NTL * 4 * 64) + lane;
+      if (wk == 1) {
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < TL::NTL; ++ni)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              red[((mi * TL::NTL + ni) * 4 + q) * 64] =
+                  (f32x4){res[mi][ni][4 * q], res[mi][ni][4 * q + 1], res[mi][ni][4 * q + 2], res[mi][ni][4 * q + 3]};
+      }
+      __syncthreads();
+      if (wk == 1) return;
+#pragma unroll
+      for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < TL::NTL; ++ni)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4 o = red[((mi * TL::NTL + ni) * 4 + q) * 64];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) res[mi][ni][4 * q + e] += o[e];
+          }
+    }
+
+    // epilogue: of every 32x32 tile a lane holds column lane%32 and rows 8*q + 4*(lane/32) + e
+    IoT* C = (IoT*)p.C;
+    const IoT* bias = (const IoT*)p.bias;
+#pragma unroll
+    for (int ni = 0; ni < TL::NTL; ++ni) {
+      const int col = n0 + wn0 + ni * 32 + l31;
+      if (col >= p.N) continue;
+      const float bv = bias ? IoType<IODT>::load(bias + col) : 0.f;
+#pragma unroll
+      for (int mi = 0; mi < TL::MT; ++mi) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int row = m0 + wm0 + mi * 32 + q * 8 + g * 4 + e;
+            if (row < p.M) IoType<IODT>::store(C + (int64_t)row * p.ldc + col, res[mi][ni][4 * q + e] + bv);
+          }
+      }
+    }
+  }
+};
+
+template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
+__global__ __launch_bounds__(TL::NT) void cascmm_tile_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char cascmm_smem[];
+  TileGemm<TL, IODT, FMT, TERMS, FULL>::template run<FAST>(p, (u32x4*)cascmm_smem);
+}
+
+}  // namespace cascmm

@@ -1,0 +1,49 @@
+// Host-side table of compiled kernel variants and the launcher template that fills it.
+#pragma once
+#include <mutex>
+
+#include "cascmm_tile_kernel.h"
+
+namespace cascmm {
+
+enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1 };
+
+struct VariantDesc {
+  const char* name;
+  int kind;
+  int iodt, fmt, terms, full;
+  int BM, BN, BK, threads;
+  int lds_bytes;
+  bool fast;  // needs fp32 operands, K % BK == 0, 16-byte aligned A rows
+  int (*launch)(const GemmParams&, hipStream_t);
+};
+
+template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
+int launch_tile(const GemmParams& p, hipStream_t stream) {
+  auto kfn = cascmm_tile_kernel<TL, IODT, FMT, TERMS, FULL, FAST>;
+  constexpr int lds = LdsLayout<TL, TERMS>::kBytes;
+  static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
+  if (lds > 64 * 1024) {
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+      attr_err = hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    });
+    if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
+  }
+  const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n;
+  hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
+  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+}
+
+#define CASCMM_TILE_VARIANT(NAME, BM, BN, BK, WM, WN, WK, DEPTH, IODT, FMT, TERMS, FULL, FAST)         \
+  {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, WM * WN * WK * 64,                            \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, TERMS>::kBytes, FAST,                               \
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, IODT, FMT, TERMS, FULL, FAST>}
+
+// each instantiation unit exports its slice of the table
+const VariantDesc* variants_bf16(int* n);
+const VariantDesc* variants_fp16(int* n);
+const VariantDesc* variants_io16(int* n);
+
+}  // namespace cascmm

@@ -1,0 +1,35 @@
+"""Drop-in for the reference's BasedXLLowPLinear (basedxl/modules/lowp_linear.py:7-20)."""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from ..cascaded_lowp_matmul import cascaded_lowp_matmul
+
+
+class BasedXLLowPLinear(nn.Module):
+    """Wraps an ``nn.Linear``: the weight is stored transposed as ``[in, out]``
+    (lowp_linear.py:12) and the forward pass is one cascade GEMM with the bias add fused
+    into its store (the reference adds it in a second kernel, lowp_linear.py:17-19)."""
+
+    def __init__(self, submodule: nn.Linear, *, lowp: str = "bf16", terms: int = 2, products: str = "tri"):
+        super().__init__()
+        self.in_features = submodule.in_features
+        self.out_features = submodule.out_features
+        self.weight = submodule.weight.detach().T.contiguous().clone()
+        self.bias = submodule.bias.detach().clone() if submodule.bias is not None else None
+        self.lowp, self.terms, self.products = lowp, terms, products
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return cascaded_lowp_matmul(x, self.weight, bias=self.bias, lowp=self.lowp, terms=self.terms,
+                                    products=self.products)
+
+
+def patch_linear_layers(model: nn.Module, **cascade_kwargs) -> nn.Module:
+    """Replace every ``nn.Linear`` child with :class:`BasedXLLowPLinear`
+    (same walk as basedxl/unet.py:81-87)."""
+    for _name, module in model.named_modules():
+        for subname, submodule in module.named_children():
+            if isinstance(submodule, nn.Linear):
+                setattr(module, subname, BasedXLLowPLinear(submodule, **cascade_kwargs))
+    return model

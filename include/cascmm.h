@@ -1,0 +1,121 @@
+/*
+ * cascmm.h -- C ABI of the MI355X (gfx950) cascaded low-precision matmul library.
+ *
+ * The library computes  C[M,N] = A[M,K] . B[K,N] (+ bias[N])  where the fp32 operands are
+ * split on the fly into `terms` low-precision terms (bf16 / fp16 / fp8-e4m3), the kept
+ * partial products run on MFMA and are accumulated in fp32.
+ *
+ * It is the device side of the Python operator
+ *     cascaded_lowp_matmul(a, b, *, out=None, dump_ptx=False)
+ * of the reference (basedxl/triton/cascaded_lowp_matmul.py:139-173): the host wrapper
+ * does the shape checks / batch flattening / output allocation of :146-161,173 and calls
+ * cascmm_gemm() where the reference launches its Triton kernel (:163-168).
+ *
+ * Conventions
+ *  - every pointer named A, B, C, bias, x, out, workspace, tensor_exps is a DEVICE pointer;
+ *  - the library never allocates or frees device memory and never synchronises the host;
+ *  - all work is enqueued on `stream` (a hipStream_t passed as void*, NULL = default stream);
+ *  - every function returns 0 on success or a negative cascmm_status; nothing throws.
+ *  - row-major operands, leading dimensions in ELEMENTS.
+ */
+#ifndef CASCMM_H
+#define CASCMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CASCMM_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* element type of A, B, C and bias as stored in memory (C has the type of A, like
+ * `torch.empty((M, N), dtype=a.dtype)` at cascaded_lowp_matmul.py:161) */
+enum cascmm_dtype { CASCMM_DT_F32 = 0, CASCMM_DT_F16 = 1, CASCMM_DT_BF16 = 2 };
+
+/* low-precision format of the cascade terms */
+enum cascmm_fmt { CASCMM_FMT_BF16 = 0, CASCMM_FMT_FP16 = 1, CASCMM_FMT_FP8 = 2 };
+
+/* which partial products A_i.B_j are summed: TRI keeps i + j <= terms - 1, FULL keeps all */
+enum cascmm_products { CASCMM_PROD_TRI = 0, CASCMM_PROD_FULL = 1 };
+
+enum cascmm_status {
+  CASCMM_OK = 0,
+  CASCMM_ERR_NULL_POINTER = -1,
+  CASCMM_ERR_BAD_SHAPE = -2,     /* negative size, leading dimension smaller than the row */
+  CASCMM_ERR_BAD_DTYPE = -3,
+  CASCMM_ERR_BAD_FORMAT = -4,    /* unknown fmt / unsupported (fmt, terms, products) */
+  CASCMM_ERR_WORKSPACE = -5,     /* workspace missing or smaller than cascmm_workspace_bytes */
+  CASCMM_ERR_ALIGNMENT = -6,     /* pointer not aligned to its element size */
+  CASCMM_ERR_LAUNCH = -7,        /* the HIP runtime refused the launch */
+  CASCMM_ERR_BAD_VARIANT = -8,   /* forced kernel variant unknown or unable to run this problem */
+  CASCMM_ERR_TOO_LARGE = -9      /* a dimension exceeds 2^31 - 1 or a product overflows */
+};
+
+/*
+ * The matmul.  Replaces the `_matmul_kernel[grid](...)` launch of
+ * basedxl/triton/cascaded_lowp_matmul.py:166-168 and, when `bias` is non-NULL, the
+ * separate `x + bias` of basedxl/modules/lowp_linear.py:17-19.
+ *
+ *   A [M,K] lda>=K, B [K,N] ldb>=N, C [M,N] ldc>=N, bias [N] or NULL; all of `dtype`.
+ *   fmt/terms/products: supported combinations are
+ *       bf16: terms 1..3;  fp16: terms 1..3;  fp8: terms 1..3.
+ *   tensor_exps: fp8 only -- device pointer to two int32 {e_A, e_B}: the operands are
+ *       scaled by 2^e before rounding (see cascmm_tensor_exp); NULL means {0, 0}.
+ *   workspace: needed only when cascmm_workspace_bytes(...) > 0 (the split-K path for
+ *       skinny shapes); its first bytes must be zero on first use and are left zero.
+ *   M, N or K equal to 0 is valid (K == 0 writes bias or zeros).
+ */
+int cascmm_gemm(const void* A, const void* B, void* C, const void* bias,
+                int64_t M, int64_t N, int64_t K,
+                int64_t lda, int64_t ldb, int64_t ldc,
+                int dtype, int fmt, int terms, int products,
+                const int32_t* tensor_exps,
+                void* workspace, size_t workspace_bytes, void* stream);
+
+/* Same with the kernel variant forced (index into the variant table, see
+ * cascmm_variant_count / cascmm_variant_name); variant < 0 selects automatically.
+ * No counterpart in the reference, whose Triton autotuner picks among its two configs
+ * (cascaded_lowp_matmul.py:29-51); used by the tests and the tuning sweep. */
+int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,
+                        int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc,
+                        int dtype, int fmt, int terms, int products,
+                        const int32_t* tensor_exps,
+                        void* workspace, size_t workspace_bytes, void* stream, int variant);
+
+/* Bytes of device workspace cascmm_gemm needs for this problem (0 for most shapes).
+ * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,
+ * cascaded_lowp_matmul.py:155-156); the caller allocates, as it allocates `out` (:161). */
+size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms,
+                              int products);
+
+/* Variant the automatic selection would run for this problem (index), or a negative status. */
+int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                          int dtype, int fmt, int terms, int products);
+int cascmm_variant_count(void);
+/* Static string: the device function name of the variant's kernel is a template
+ * instantiation whose text contains this name (for filtering rocprof output), or NULL. */
+const char* cascmm_variant_name(int variant);
+
+/* fp8 tensor scale: writes to *exp_out (device int32) the exponent e with
+ * max|x| * 2^e in (224, 448] (0 for an all-zero tensor).  x is [rows, cols] with leading
+ * dimension ld.  *exp_out is overwritten; the call is stream-ordered. */
+int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype,
+                      int32_t* exp_out, void* stream);
+
+/* The operand split alone (a test hook for parity of the split with the CPU oracle):
+ * out is fp32 [terms][n]; term i holds lowp(r_i * 2^(tensor_exp + shift*i)) upcast to fp32
+ * with r_0 = x, r_{i+1} = r_i - t_i / 2^(tensor_exp + shift*i); shift = 0 / 11 / 4 for
+ * bf16 / fp16 / fp8.  x is `n` contiguous elements of `dtype`. */
+int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms,
+                       int tensor_exp, void* stream);
+
+const char* cascmm_strerror(int status);
+int cascmm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CASCMM_H */

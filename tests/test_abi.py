@@ -1,0 +1,94 @@
+"""CPU-only checks of the C ABI: the library loads, exports everything the header declares,
+and its argument validation (which runs before any GPU work) returns the documented codes."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from basedxl_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "cascmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cascmm_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared()
+    assert "cascmm_gemm" in names and len(names) >= 8
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f"{n} declared in include/cascmm.h but not exported"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_version_and_strerror():
+    l = _lib.lib()
+    assert l.cascmm_version() == 100
+    assert l.cascmm_strerror(0) == b"ok"
+    for code in range(-9, 0):
+        assert l.cascmm_strerror(code) not in (None, b"unknown status")
+    assert l.cascmm_strerror(-99) == b"unknown status"
+
+
+def test_variant_table():
+    names = _lib.variant_names()
+    assert len(names) == len(set(names)) > 10
+    assert any("bf16x2_tri" in n for n in names)
+    assert _lib.lib().cascmm_variant_name(-1) is None
+    assert _lib.lib().cascmm_variant_name(len(names)) is None
+
+
+def _gemm(M, N, K, lda=None, ldb=None, ldc=None, dtype=0, fmt=0, terms=2, products=0, A=8, B=8, C=8):
+    l = _lib.lib()
+    return l.cascmm_gemm(A, B, C, None, M, N, K, lda if lda is not None else K, ldb if ldb is not None else N,
+                         ldc if ldc is not None else N, dtype, fmt, terms, products, None, None, 0, None)
+
+
+def test_argument_validation_codes():
+    # all of these return before touching the device
+    assert _gemm(-1, 4, 4) == -2
+    assert _gemm(4, 4, 4, lda=3) == -2
+    assert _gemm(4, 4, 4, ldb=3) == -2
+    assert _gemm(4, 4, 4, ldc=3) == -2
+    assert _gemm(4, 4, 4, dtype=7) == -3
+    assert _gemm(4, 4, 4, fmt=9) == -4
+    assert _gemm(4, 4, 4, terms=0) == -4
+    assert _gemm(4, 4, 4, terms=4) == -4
+    assert _gemm(4, 4, 4, products=2) == -4
+    assert _gemm(2 ** 31, 4, 4) == -9
+    assert _gemm(4, 4, 4, C=None) == -1
+    assert _gemm(4, 4, 4, A=None) == -1
+    assert _gemm(4, 4, 4, A=6) == -6
+    # empty problems are fine and launch nothing
+    assert _gemm(0, 4, 4, A=None, B=None, C=None) == 0
+    assert _gemm(4, 0, 4, A=None, B=None, C=None) == 0
+
+
+def test_select_variant_prefers_sensible_tiles():
+    l = _lib.lib()
+    names = _lib.variant_names()
+    v = l.cascmm_select_variant(4096, 640, 640, 640, 640, 640, 0, 0, 2, 0)
+    assert v >= 0 and "bf16x2_tri" in names[v]
+    # K not a multiple of 8 must take a bounds-checked kernel
+    v = l.cascmm_select_variant(10, 30, 20, 20, 30, 30, 0, 0, 2, 0)
+    assert v >= 0 and "generic" in names[v]
+    v = l.cascmm_select_variant(128, 128, 128, 128, 128, 128, 0, 1, 3, 0)
+    assert v >= 0 and "fp16x3_tri" in names[v]
+    assert l.cascmm_select_variant(4, 4, 4, 4, 4, 4, 0, 5, 2, 0) == -4
+
+
+def test_cpu_tensors_are_rejected_without_fallback():
+    import torch
+    from basedxl_amd import cascaded_lowp_matmul
+
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        cascaded_lowp_matmul(torch.randn(4, 4), torch.randn(4, 4))
+    with pytest.raises(AssertionError, match="Incompatible dimensions"):
+        cascaded_lowp_matmul(torch.randn(4, 4), torch.randn(5, 4))
+    with pytest.raises(AssertionError, match="Matrix B must be contiguous"):
+        cascaded_lowp_matmul(torch.randn(4, 4), torch.randn(4, 4).t())

@@ -1,0 +1,231 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI via the Python operator,
+against the CPU oracle.
+
+Bars: bit-exact where the mathematics fixes the bits (the operand split; integer-valued
+operands whose partial sums stay below 2**24); for random fp32 operands the error versus an
+fp64 product must be no worse than 1.25x the oracle cascade's error (max-abs and relative
+Frobenius), same split and same product set.
+"""
+import numpy as np
+import pytest
+import torch
+
+from basedxl_amd import _lib, cascaded_lowp_matmul, BasedXLLowPLinear
+from oracle import cascade as oc
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1.25  # kernel error may be at most this multiple of the oracle cascade's error
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _gpu(t):
+    return t.to("cuda:0")
+
+
+def _variants_for(tag):
+    return [(i, n) for i, n in enumerate(_lib.variant_names()) if tag in n]
+
+
+# ---------------------------------------------------------------------------------------
+# the split alone
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fmt,terms", [("bf16", 1), ("bf16", 2), ("bf16", 3), ("fp16", 1), ("fp16", 2), ("fp16", 3)])
+def test_split_matches_oracle_bit_for_bit(gpu_device, fmt, terms):
+    _say("split", fmt, terms)
+    g = torch.Generator().manual_seed(0)
+    x = torch.cat([
+        torch.randn(100_000, generator=g), torch.randn(100_000, generator=g) * 0.02,
+        torch.randn(20_000, generator=g) * 1e-4, torch.randn(20_000, generator=g) * 300.0,
+        torch.tensor([0.0, -0.0, 1.0, 1.00390625, 1.005859375, 65504.0 if fmt == "fp16" else 3e38, 6e-8, 2 ** -24,
+                      2 ** -25, 1e-30, -1e-30, 2 ** -14, 1.0 + 2 ** -11, 1.0 + 3 * 2 ** -11]),
+    ]).float()
+    want, scales = oc.split_terms(x, fmt, terms, tensor_exp=0)
+    xd = _gpu(x)
+    out = torch.empty(terms, x.numel(), dtype=torch.float32, device=xd.device)
+    st = _lib.lib().cascmm_split_terms(xd.data_ptr(), out.data_ptr(), x.numel(), _lib.DT_F32, _lib.FMT_BY_NAME[fmt],
+                                       terms, 0, torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    got = out.cpu()
+    for i in range(terms):
+        # bit-exact, except that a zero term may carry either sign (it cannot change any sum)
+        both_zero = (got[i] == 0) & (want[i] == 0)
+        bad = ((got[i].view(torch.int32) != want[i].view(torch.int32)) & ~both_zero).nonzero().flatten()
+        assert bad.numel() == 0, (fmt, terms, i, [(float(x[j]), float(got[i][j]), float(want[i][j])) for j in bad[:8]])
+
+
+# ---------------------------------------------------------------------------------------
+# exact integer known-answer tests, every kernel variant, ragged shapes
+# ---------------------------------------------------------------------------------------
+def _int_case(M, K, N, hi, seed):
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-hi, hi + 1, size=(M, K))
+    b = rng.integers(-hi, hi + 1, size=(K, N))
+    return a, b, a @ b
+
+
+INT_SHAPES = [(16, 32, 16), (17, 33, 19), (154, 64, 48), (1, 7, 1), (130, 40, 81), (256, 192, 160), (300, 128, 200),
+              (257, 64, 161)]
+
+
+@pytest.mark.parametrize("shape", INT_SHAPES)
+def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
+    M, K, N = shape
+    a, b, want = _int_case(M, K, N, 100, seed=M + K + N)
+    assert np.abs(want).max() < 2 ** 24
+    at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
+    l = _lib.lib()
+    names = _lib.variant_names()
+    ran = 0
+    for vi, name in enumerate(names):
+        fmt = "bf16" if "bf16" in name else "fp16"
+        terms = int(name.split(fmt + "x")[1][0])
+        products = "full" if "_full" in name else "tri"
+        bk = int(name.split("_")[0].split("x")[2])
+        if "generic" not in name and (K % bk != 0):
+            continue  # fast variants need K % BK == 0 (rejected by the library otherwise)
+        _say("int-exact", shape, name)
+        out = cascaded_lowp_matmul(at, bt, lowp=fmt, terms=terms, products=products, variant=vi)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        assert np.array_equal(got.astype(np.int64), want), (name, shape)
+        ran += 1
+    assert ran >= 5
+
+
+def test_fast_variant_is_refused_for_unaligned_k(gpu_device):
+    a, b = _gpu(torch.randn(32, 20)), _gpu(torch.randn(20, 32))
+    vi = [i for i, n in enumerate(_lib.variant_names()) if "bf16x2_tri" in n and "generic" not in n][0]
+    with pytest.raises(_lib.CascmmError, match="variant"):
+        cascaded_lowp_matmul(a, b, variant=vi)
+
+
+def test_sixteen_bit_integers_full_product_set_is_exact(gpu_device):
+    """Operands need both bf16 terms; 'full' keeps lo.lo so the result is the exact integer
+    product, 'tri' differs from it by exactly the lo.lo part the oracle also drops."""
+    rng = np.random.default_rng(5)
+    a = rng.integers(-2000, 2001, size=(64, 16))
+    b = rng.integers(-2000, 2001, size=(16, 48))
+    want = a @ b
+    at, bt = torch.tensor(a, dtype=torch.float32), torch.tensor(b, dtype=torch.float32)
+    keep = np.abs(want) < 2 ** 24
+    full = cascaded_lowp_matmul(_gpu(at), _gpu(bt), products="full").cpu().numpy().astype(np.int64)
+    tri = cascaded_lowp_matmul(_gpu(at), _gpu(bt), products="tri").cpu()
+    assert np.array_equal(full[keep], want[keep])
+    assert torch.equal(tri, oc.cascade_matmul_ref(at, bt, "bf16", 2, "tri"))
+
+
+# ---------------------------------------------------------------------------------------
+# accuracy bound against the oracle on the baseline configurations
+# ---------------------------------------------------------------------------------------
+ACC_CASES = [
+    # name, M, K, N, w_std, seed
+    ("cfg1 1024^3", 1024, 1024, 1024, 1.0, 0),
+    ("cfg2 self-attn proj", 4096, 640, 640, 0.02, 1),
+    ("cfg3 geglu up (N/4)", 2048, 1280, 2560, 0.02, 2),
+    ("cfg3 ff down", 2048, 5120, 1280, 0.02, 3),
+    ("cfg4 cross-attn kv 1280", 154, 2048, 1280, 0.02, 4),
+    ("cfg4 cross-attn kv 640", 154, 2048, 640, 0.02, 5),
+    ("ragged", 333, 456, 211, 1.0, 6),
+]
+ACC_FORMATS = [("bf16", 2, "tri"), ("bf16", 2, "full"), ("bf16", 3, "tri"), ("fp16", 3, "tri"), ("fp16", 2, "tri"),
+               ("bf16", 1, "tri")]
+
+
+@pytest.mark.parametrize("case", ACC_CASES, ids=[c[0] for c in ACC_CASES])
+@pytest.mark.parametrize("fmt,terms,products", ACC_FORMATS)
+def test_error_vs_fp64_within_bound_of_oracle(gpu_device, case, fmt, terms, products):
+    name, M, K, N, w_std, seed = case
+    _say("accuracy", name, fmt, terms, products)
+    a, b = oc.make_operands(M, K, N, seed=seed, w_std=w_std)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, fmt, terms, products), exp)
+    out = cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp=fmt, terms=terms, products=products)
+    torch.cuda.synchronize()
+    got = oc.error_metrics(out.cpu(), exp)
+    _say(f"   rel_fro kernel {got['rel_fro']:.3e} oracle {ref['rel_fro']:.3e}  max_abs kernel {got['max_abs']:.3e} "
+         f"oracle {ref['max_abs']:.3e}")
+    assert got["rel_fro"] <= TOL * ref["rel_fro"], (got["rel_fro"], ref["rel_fro"])
+    assert got["max_abs"] <= TOL * ref["max_abs"], (got["max_abs"], ref["max_abs"])
+
+
+def test_every_headline_variant_meets_the_bound(gpu_device):
+    a, b = oc.make_operands(1024, 640, 640, seed=9, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exp)
+    ad, bd = _gpu(a), _gpu(b)
+    for vi, name in _variants_for("bf16x2_tri"):
+        _say("variant", name)
+        got = oc.error_metrics(cascaded_lowp_matmul(ad, bd, variant=vi).cpu(), exp)
+        assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"], name
+
+
+def test_repeated_launches_are_bit_identical(gpu_device):
+    a, b = oc.make_operands(1000, 648, 640, seed=10, w_std=0.02)
+    ad, bd = _gpu(a), _gpu(b)
+    first = cascaded_lowp_matmul(ad, bd).clone()
+    for _ in range(20):
+        assert torch.equal(cascaded_lowp_matmul(ad, bd), first)
+
+
+# ---------------------------------------------------------------------------------------
+# wrapper semantics (shape cases of the reference's own test, tests/test_cascaded_lowp_matmul.py:9-14)
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape_a,shape_b", [
+    ((10, 20), (20, 30)), ((5, 10, 20), (20, 30)), ((10, 20), (5, 20, 30)), ((5, 10, 20), (5, 20, 30)),
+    ((128, 512), (512, 128)), ((1024, 2048), (2048, 1024)),
+])
+def test_reference_shape_cases(gpu_device, shape_a, shape_b):
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn(*shape_a, generator=g)
+    b = torch.randn(*shape_b, generator=g)
+    out = cascaded_lowp_matmul(_gpu(a), _gpu(b))
+    want = oc.cascaded_lowp_matmul_ref(a, b)
+    exp = torch.matmul(a.double(), b.double())
+    assert out.shape == want.shape and out.dtype == a.dtype
+    got = oc.error_metrics(out.cpu(), exp)
+    ref = oc.error_metrics(want, exp)
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+    # and the reference's own acceptance criterion (tests/test_cascaded_lowp_matmul.py:26)
+    assert torch.allclose(out.cpu(), torch.matmul(a, b), rtol=0.001, atol=0.35)
+
+
+def test_out_argument_strided_input_and_bias(gpu_device):
+    g = torch.Generator().manual_seed(12)
+    big = _gpu(torch.randn(64, 200, generator=g))
+    a = big[:, 8:136]  # row stride 200, 128 columns: not contiguous, rows contiguous
+    b = _gpu(torch.randn(128, 96, generator=g))
+    bias = _gpu(torch.randn(96, generator=g))
+    out = torch.empty(64, 96, device="cuda:0")
+    r = cascaded_lowp_matmul(a, b, out=out, bias=bias)
+    assert r.data_ptr() == out.data_ptr()
+    want = oc.cascade_matmul_ref(a.cpu().contiguous(), b.cpu()) + bias.cpu()
+    assert torch.allclose(out.cpu(), want, rtol=0, atol=2e-5)
+    # transposed a (unit stride along M, not K) is made contiguous by the wrapper
+    at = _gpu(torch.randn(128, 64, generator=g)).t()
+    r2 = cascaded_lowp_matmul(at, b)
+    assert torch.allclose(r2.cpu(), oc.cascade_matmul_ref(at.cpu().contiguous(), b.cpu()), rtol=0, atol=2e-5)
+
+
+def test_k_zero_and_empty(gpu_device):
+    a = torch.empty(5, 0, device="cuda:0")
+    b = torch.empty(0, 7, device="cuda:0")
+    bias = torch.arange(7, dtype=torch.float32, device="cuda:0")
+    assert torch.equal(cascaded_lowp_matmul(a, b).cpu(), torch.zeros(5, 7))
+    assert torch.equal(cascaded_lowp_matmul(a, b, bias=bias).cpu(), bias.cpu().expand(5, 7))
+    assert cascaded_lowp_matmul(torch.empty(0, 8, device="cuda:0"), torch.empty(8, 4, device="cuda:0")).shape == (0, 4)
+
+
+def test_lowp_linear_module(gpu_device):
+    torch.manual_seed(13)
+    lin = torch.nn.Linear(640, 320).to("cuda:0")
+    mod = BasedXLLowPLinear(lin)
+    x = torch.randn(2, 77, 640, device="cuda:0")
+    y = mod(x)
+    want = oc.cascade_matmul_ref(x.cpu().reshape(-1, 640), lin.weight.detach().cpu().t().contiguous()) \
+        + lin.bias.detach().cpu()
+    assert y.shape == (2, 77, 320)
+    assert torch.allclose(y.cpu().reshape(-1, 320), want, rtol=0, atol=2e-5)
