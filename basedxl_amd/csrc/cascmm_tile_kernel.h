@@ -23,8 +23,13 @@
 // indexed by compile-time constants), the LDS stage is double buffered, and there is one
 // barrier per K step.
 //
-// Waves are arranged WM x WN x WK.  With WK = 2 the two wave groups take alternate 16-wide
-// k slices of every stage and their accumulators are added through LDS at the end.
+// The workgroup is specialised.  WM x WN x WK "consumer" waves only read fragments from LDS
+// and issue MFMAs; NP "producer" waves only load, split and write LDS.  With one wave of each
+// kind per SIMD, the producer's VALU work issues in the gaps the consumer's MFMAs leave on
+// the VALU port, and neither kind ever waits for the other except at the one barrier per K
+// step.  Producers hold no accumulators, so their registers go to a deep prefetch ring.
+// With WK = 2 the two consumer groups take alternate 16-wide k slices of every stage and
+// their accumulators are added through LDS at the end.
 //
 // All partial products of one (m-tile, n-tile) reuse the same fragments in registers; the
 // cross-term sum happens in the accumulator registers (one accumulator per scale class).
@@ -33,10 +38,12 @@
 
 namespace cascmm {
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2, int NP_ = 4>
 struct Tile {
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, WK = WK_, DEPTH = DEPTH_;
-  static constexpr int NT = WM * WN * WK * kWave;
+  static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, WK = WK_, DEPTH = DEPTH_, NP = NP_;
+  static constexpr int NCW = WM * WN * WK;   // consumer waves
+  static constexpr int NTP = NP * kWave;     // producer threads
+  static constexpr int NT = (NCW + NP) * kWave;
   static constexpr int KG = BK / 8;          // k-groups (planes) per stage
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int MT = WTM / 32, NTL = WTN / 32;
@@ -90,6 +97,7 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 __device__ float llvm_raw_buffer_load_f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.f32");
 __device__ f32x4 llvm_raw_buffer_load_v4f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
+__device__ void llvm_raw_buffer_store_f32(float v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.f32");
 
 // gfx9-family raw buffer descriptor: 48-bit base, stride 0, byte count, 32-bit data format
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
@@ -113,7 +121,7 @@ struct TileGemm {
   static constexpr int ES = sizeof(IoT);
   static constexpr int NCLS = AC::kCount;
   static constexpr int A_UNITS = TL::KG * TL::BM, B_UNITS = TL::KG * TL::BN;
-  static constexpr int A_IT = (A_UNITS + TL::NT - 1) / TL::NT, B_IT = (B_UNITS + TL::NT - 1) / TL::NT;
+  static constexpr int A_IT = (A_UNITS + TL::NTP - 1) / TL::NTP, B_IT = (B_UNITS + TL::NTP - 1) / TL::NTP;
   static constexpr int D = TL::DEPTH;
 
   struct Regs {
@@ -130,7 +138,7 @@ struct TileGemm {
     int ldb_bytes;
   };
 
-  static __device__ __forceinline__ void init_ctx(Ctx& c, const GemmParams& p, int m0, int n0) {
+  static __device__ __forceinline__ void init_ctx(Ctx& c, const GemmParams& p, int m0, int n0, int ptid) {
     const IoT* A = (const IoT*)p.A + (int64_t)m0 * p.lda;
     const IoT* B = (const IoT*)p.B + n0;
     // bytes from the tile origin to the end of the matrix; rows and columns are also clamped
@@ -141,7 +149,7 @@ struct TileGemm {
     const int last_row = p.M - 1 - m0, last_col = p.N - 1 - n0;
 #pragma unroll
     for (int it = 0; it < A_IT; ++it) {
-      int u = threadIdx.x + it * TL::NT;
+      int u = ptid + it * TL::NTP;
       const bool mine = u < A_UNITS;
       u = mine ? u : A_UNITS - 1;
       const int kg = u % TL::KG, r = u / TL::KG;
@@ -151,7 +159,7 @@ struct TileGemm {
     }
 #pragma unroll
     for (int it = 0; it < B_IT; ++it) {
-      int u = threadIdx.x + it * TL::NT;
+      int u = ptid + it * TL::NTP;
       const bool mine = u < B_UNITS;
       u = mine ? u : B_UNITS - 1;
       const int n = u % TL::BN, kg = u / TL::BN;
@@ -183,12 +191,12 @@ struct TileGemm {
   }
 
   // ---- global -> registers (generic: any dtype, any K, element-wise, bounds-checked) ------
-  static __device__ __forceinline__ void load_generic(const GemmParams& p, int m0, int n0, int k0, Regs& r) {
+  static __device__ __forceinline__ void load_generic(const GemmParams& p, int m0, int n0, int k0, int ptid, Regs& r) {
     const IoT* A = (const IoT*)p.A;
     const IoT* B = (const IoT*)p.B;
 #pragma unroll
     for (int it = 0; it < A_IT; ++it) {
-      int u = threadIdx.x + it * TL::NT;
+      int u = ptid + it * TL::NTP;
       u = u < A_UNITS ? u : A_UNITS - 1;
       const int kg = u % TL::KG;
       int row = m0 + u / TL::KG;
@@ -200,7 +208,7 @@ struct TileGemm {
     }
 #pragma unroll
     for (int it = 0; it < B_IT; ++it) {
-      int u = threadIdx.x + it * TL::NT;
+      int u = ptid + it * TL::NTP;
       u = u < B_UNITS ? u : B_UNITS - 1;
       const int kg = u / TL::BN;
       int col = n0 + u % TL::BN;
@@ -217,7 +225,7 @@ struct TileGemm {
     u32x4* sb = stage + TERMS * LL::kATerm;
 #pragma unroll
     for (int it = 0; it < A_IT; ++it) {
-      if (A_UNITS % TL::NT != 0 && c.lds_a[it] < 0) continue;
+      if (A_UNITS % TL::NTP != 0 && c.lds_a[it] < 0) continue;
       u32x4 t[TERMS];
       split8<FMT, TERMS>(r.a[it], t);
 #pragma unroll
@@ -225,7 +233,7 @@ struct TileGemm {
     }
 #pragma unroll
     for (int it = 0; it < B_IT; ++it) {
-      if (B_UNITS % TL::NT != 0 && c.lds_b[it] < 0) continue;
+      if (B_UNITS % TL::NTP != 0 && c.lds_b[it] < 0) continue;
       u32x4 t[TERMS];
       split8<FMT, TERMS>(r.b[it], t);
 #pragma unroll
@@ -269,13 +277,51 @@ struct TileGemm {
     }
   }
 
-  // ---- the kernel body ------------------------------------------------------------------
+  // ---- producer waves: global -> split -> LDS, one stage per barrier interval -----------------
+  // Barrier protocol (both kinds of wave execute exactly ktiles + 1 barriers, plus one more
+  // for the WK reduction):
+  //   producer:  store(0) B0 store(1) B1 ... store(kt-1) B(kt-1)            B(kt)
+  //   consumer:           B0 compute(0) B1 ... compute(kt-2) B(kt-1) compute(kt-1) B(kt)
+  // store(s) writes LDS buffer s&1 between B(s-1) and B(s); the last reader of that buffer,
+  // compute(s-2), finished before B(s-1), and its first reader, compute(s), starts after B(s).
   template <bool FAST>
-  static __device__ __forceinline__ void run(const GemmParams& p, u32x4* lds) {
-    int tm, tn;
-    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-    const int m0 = tm * TL::BM, n0 = tn * TL::BN;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  static __device__ __forceinline__ void producer(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles) {
+    const int ptid = threadIdx.x - TL::NCW * kWave;
+    Ctx ctx;
+    init_ctx(ctx, p, m0, n0, ptid);
+    Regs ring[D];
+    // loads are only ever issued for k steps that exist (s < ktiles)
+    auto issue = [&](int s, Regs& r) {
+      if (FAST) load_fast(ctx, s * TL::BK, r);
+      else load_generic(p, m0, n0, s * TL::BK, ptid, r);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+      if (d < ktiles) issue(d, ring[d]);
+    int s = 0;
+    for (; s + 2 * D <= ktiles; s += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        store(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d]);
+        issue(s + d + D, ring[d]);
+        __syncthreads();
+      }
+    }
+#pragma unroll
+    for (int dd = 0; dd < 2 * D; ++dd) {
+      const int d = dd % D;
+      if (s + dd < ktiles) {
+        store(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d]);
+        if (s + dd + D < ktiles) issue(s + dd + D, ring[d]);
+        __syncthreads();
+      }
+    }
+    __syncthreads();
+    if (TL::WK > 1) __syncthreads();
+  }
+
+  // ---- consumer waves: LDS -> MFMA, then the epilogue --------------------------------------
+  static __device__ __forceinline__ void consumer(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles, int wave) {
     const int wk = wave / (TL::WM * TL::WN);
     const int wmn = wave - wk * (TL::WM * TL::WN);
     const int wm0 = (wmn / TL::WN) * TL::WTM, wn0 = (wmn % TL::WN) * TL::WTN;
@@ -290,45 +336,10 @@ struct TileGemm {
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[c][mi][ni][e] = 0.f;
 
-    Ctx ctx;
-    init_ctx(ctx, p, m0, n0);
-    Regs ring[D];
-    const int ktiles = (p.K + TL::BK - 1) / TL::BK;
-
-    // loads are only ever issued for k steps that exist (kt < ktiles)
-    auto issue = [&](int kt, Regs& r) {
-      if (FAST) load_fast(ctx, kt * TL::BK, r);
-      else load_generic(p, m0, n0, kt * TL::BK, r);
-    };
-
-    // prologue: up to DEPTH steps in flight, the first one staged
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-      if (d < ktiles) issue(d, ring[d]);
-    if (ktiles > 0) store(ctx, lds, ring[0]);
     __syncthreads();
-
-    // step kt: refill the ring slot that step kt vacated, run the MFMAs of stage kt, stage kt+1
-    int kt = 0;
-    for (; kt + 2 * D <= ktiles; kt += D) {
-#pragma unroll
-      for (int d = 0; d < D; ++d) {
-        issue(kt + d + D, ring[d]);
-        compute(lds + ((kt + d) & 1) * LL::kStage, wm0, wn0, wk, acc);
-        store(ctx, lds + ((kt + d + 1) & 1) * LL::kStage, ring[(d + 1) % D]);
-        __syncthreads();
-      }
-    }
-    // tail: fewer than 2*DEPTH steps left, nothing (or not everything) left to prefetch
-#pragma unroll
-    for (int dd = 0; dd < 2 * D; ++dd) {
-      const int d = dd % D;
-      if (kt + dd < ktiles) {
-        if (kt + dd + D < ktiles) issue(kt + dd + D, ring[d]);
-        compute(lds + ((kt + dd) & 1) * LL::kStage, wm0, wn0, wk, acc);
-        if (kt + dd + 1 < ktiles) store(ctx, lds + ((kt + dd + 1) & 1) * LL::kStage, ring[(d + 1) % D]);
-        __syncthreads();
-      }
+    for (int kt = 0; kt < ktiles; ++kt) {
+      compute(lds + (kt & 1) * LL::kStage, wm0, wn0, wk, acc);
+      __syncthreads();
     }
 
     // fold the scale classes (smallest first), then the cross-wave-group reduction (WK == 2):
@@ -373,6 +384,27 @@ struct TileGemm {
     // epilogue: of every 32x32 tile a lane holds column lane%32 and rows 8*q + 4*(lane/32) + e
     IoT* C = (IoT*)p.C;
     const IoT* bias = (const IoT*)p.bias;
+    const bool interior = (m0 + TL::BM <= p.M) && (n0 + TL::BN <= p.N) && p.ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
+    if (IODT == CASCMM_DT_F32 && interior) {
+      // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask.
+      // A store instruction writes two full 128-byte row segments.
+      const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * p.ldc + n0 + wn0, 0x7FFFFFFF);
+      const int ldc_bytes = (int)p.ldc * ES;
+      const int voff = g * 4 * ldc_bytes + l31 * ES;
+#pragma unroll
+      for (int ni = 0; ni < TL::NTL; ++ni) {
+        const float bv = bias ? IoType<IODT>::load(bias + n0 + wn0 + ni * 32 + l31) : 0.f;
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              llvm_raw_buffer_store_f32(res[mi][ni][4 * q + e] + bv, rc, voff,
+                                        (mi * 32 + q * 8 + e) * ldc_bytes + ni * 32 * ES, 0);
+      }
+      return;
+    }
 #pragma unroll
     for (int ni = 0; ni < TL::NTL; ++ni) {
       const int col = n0 + wn0 + ni * 32 + l31;
@@ -380,15 +412,27 @@ struct TileGemm {
       const float bv = bias ? IoType<IODT>::load(bias + col) : 0.f;
 #pragma unroll
       for (int mi = 0; mi < TL::MT; ++mi) {
+        const int row0 = m0 + wm0 + mi * 32 + g * 4;
+        IoT* dst = C + (int64_t)row0 * p.ldc + col;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int row = m0 + wm0 + mi * 32 + q * 8 + g * 4 + e;
-            if (row < p.M) IoType<IODT>::store(C + (int64_t)row * p.ldc + col, res[mi][ni][4 * q + e] + bv);
+            if (row0 + q * 8 + e < p.M) IoType<IODT>::store(dst + (int64_t)(q * 8 + e) * p.ldc, res[mi][ni][4 * q + e] + bv);
           }
       }
     }
+  }
+
+  template <bool FAST>
+  static __device__ __forceinline__ void run(const GemmParams& p, u32x4* lds) {
+    int tm, tn;
+    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    const int m0 = tm * TL::BM, n0 = tn * TL::BN;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ktiles = (p.K + TL::BK - 1) / TL::BK;
+    if (wave >= TL::NCW) producer<FAST>(p, lds, m0, n0, ktiles);
+    else consumer(p, lds, m0, n0, ktiles, wave);
   }
 };
 

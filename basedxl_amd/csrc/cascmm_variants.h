@@ -37,7 +37,7 @@ int launch_tile(const GemmParams& p, hipStream_t stream) {
 }
 
 #define CASCMM_TILE_VARIANT(NAME, BM, BN, BK, WM, WN, WK, DEPTH, IODT, FMT, TERMS, FULL, FAST)         \
-  {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, WM * WN * WK * 64,                            \
+  {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH>::NT,       \
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, TERMS>::kBytes, FAST,                               \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, IODT, FMT, TERMS, FULL, FAST>}
 
