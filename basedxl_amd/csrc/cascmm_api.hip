@@ -42,9 +42,10 @@ static int check_problem(const Problem& q) {
   return CASCMM_OK;
 }
 
-// what the fast (buffer-load, no K tail) kernels need apart from K % BK == 0
-static bool fast_ok(const Problem& q, const void* A) {
+// what the fast (buffer-load, 16-byte accesses, no K tail) kernels need apart from K % BK == 0
+static bool fast_ok(const Problem& q, const void* A, const void* B) {
   return q.dtype == CASCMM_DT_F32 && q.lda % 4 == 0 && (A == nullptr || aligned_to(A, 16)) &&
+         q.ldb % 4 == 0 && q.N % 4 == 0 && (B == nullptr || aligned_to(B, 16)) &&
          q.lda * 4 * 512 < INT32_MAX && q.ldb * 4 * 136 < INT32_MAX;  // 32-bit byte offsets inside a tile
 }
 
@@ -66,8 +67,8 @@ static double variant_cost(const VariantDesc& v, const Problem& q) {
   return rounds * per_tile + (v.fast ? 0.0 : 1e-3);
 }
 
-static int select_variant(const Problem& q, const void* A) {
-  const bool fast = fast_ok(q, A);
+static int select_variant(const Problem& q, const void* A, const void* B) {
+  const bool fast = fast_ok(q, A, B);
   const auto& t = table();
   int best = -1;
   double best_cost = 0;
@@ -146,11 +147,11 @@ static int gemm_impl(const void* A, const void* B, void* C, const void* bias, co
 
   const auto& t = table();
   if (variant < 0) {
-    variant = select_variant(q, A);
+    variant = select_variant(q, A, B);
     if (variant < 0) return variant;
   } else {
     if (variant >= (int)t.size()) return CASCMM_ERR_BAD_VARIANT;
-    if (!variant_matches(t[variant], q, fast_ok(q, A))) return CASCMM_ERR_BAD_VARIANT;
+    if (!variant_matches(t[variant], q, fast_ok(q, A, B))) return CASCMM_ERR_BAD_VARIANT;
   }
   const VariantDesc& v = t[variant];
   GemmParams p;
@@ -197,7 +198,7 @@ int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
   const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
   const int st = check_problem(q);
   if (st != CASCMM_OK) return st;
-  return select_variant(q, nullptr);
+  return select_variant(q, nullptr, nullptr);
 }
 
 int cascmm_variant_count(void) { return (int)table().size(); }

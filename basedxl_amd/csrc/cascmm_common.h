@@ -51,17 +51,25 @@ template <> struct Lowp<CASCMM_FMT_BF16> {
   static __device__ __forceinline__ f32x16 mfma(Vec a, Vec b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
-  // round 8 residuals to the format, update the residuals, return the packed slot
+  // round 8 residuals to the format, update the residuals, return the packed slot.
+  // Pairwise: one packed convert gives two terms; their fp32 values are the two halves of
+  // the packed word moved to the top 16 bits (1 shift, 1 and), then two subtractions.
   template <int TERM, bool LAST>
   static __device__ __forceinline__ u32x4 peel(float (&r)[8]) {
-    Vec v;
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    u32x4 out;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      __bf16 t = (__bf16)r[e];
-      v[e] = t;
-      if (!LAST) r[e] = r[e] - (float)t;
+    for (int e = 0; e < 4; ++e) {
+      const f32x2 x = {r[2 * e], r[2 * e + 1]};
+      const unsigned hp = __builtin_bit_cast(unsigned, __builtin_convertvector(x, bf16x2));
+      out[e] = hp;
+      if (!LAST) {
+        r[2 * e] = r[2 * e] - __builtin_bit_cast(float, hp << 16);
+        r[2 * e + 1] = r[2 * e + 1] - __builtin_bit_cast(float, hp & 0xFFFF0000u);
+      }
     }
-    return __builtin_bit_cast(u32x4, v);
+    return out;
   }
 };
 

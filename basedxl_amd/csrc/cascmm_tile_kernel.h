@@ -11,6 +11,14 @@
 // that walk k fastest (coalesced global loads), so rows are XOR-swizzled per k-group to keep
 // eight consecutive lanes on eight different 16-byte bank groups.
 //
+// B columns come in groups of 128.  A producer lane loads a 8(k) x 4(n) block with eight
+// 16-byte loads and owns four slots; slot i*32 + j of the group holds column 4*j + i, so the
+// four slot writes of 64 lanes are contiguous (no bank conflicts) and, in the epilogue, lane
+// j of the four 32-column MFMA blocks of a group holds columns 4*j .. 4*j+3 of a row: one
+// 16-byte store.  Wide loads also keep the number of loads in flight under the 6-bit vmcnt
+// limit, without which the prefetch ring cannot be waited on selectively.  Columns left over
+// after the last whole group (a multiple of 32) are loaded one per lane, unpermuted.
+//
 // The 32x32x16 MFMA is used rather than 16x16x32: it sustains a higher rate on this part and,
 // more important here, leaves room for about six other VALU instructions per MFMA (the
 // 16x16x32 form leaves two), which is what hides the three VALU operations per element that
@@ -48,6 +56,10 @@ struct Tile {
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int MT = WTM / 32, NTL = WTN / 32;
   static constexpr int KSUB = BK / 16;       // MFMA k slices per stage
+  // B columns: the first BNQ (whole groups of 128) are loaded four at a time (16-byte loads)
+  // and stored permuted in LDS; the remaining BNS columns are loaded one at a time.
+  static constexpr int BNQ = (BN / 128) * 128, BNS = BN - BNQ;
+  static_assert(BNQ == 0 || WN == 1, "permuted B columns need one consumer wave column");
   static_assert(BK == 32 || BK == 64 || BK == 128, "BK");
   static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile must be a multiple of 32");
   static_assert(KSUB % WK == 0, "k slices must divide evenly among the wave groups");
@@ -98,6 +110,7 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 __device__ float llvm_raw_buffer_load_f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.f32");
 __device__ f32x4 llvm_raw_buffer_load_v4f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
 __device__ void llvm_raw_buffer_store_f32(float v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.f32");
+__device__ void llvm_raw_buffer_store_v4f32(f32x4 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v4f32");
 
 // gfx9-family raw buffer descriptor: 48-bit base, stride 0, byte count, 32-bit data format
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
@@ -120,21 +133,31 @@ struct TileGemm {
   typedef typename IoType<IODT>::T IoT;
   static constexpr int ES = sizeof(IoT);
   static constexpr int NCLS = AC::kCount;
-  static constexpr int A_UNITS = TL::KG * TL::BM, B_UNITS = TL::KG * TL::BN;
-  static constexpr int A_IT = (A_UNITS + TL::NTP - 1) / TL::NTP, B_IT = (B_UNITS + TL::NTP - 1) / TL::NTP;
+  static constexpr int A_UNITS = TL::KG * TL::BM;
+  static constexpr int Q_UNITS = TL::KG * (TL::BNQ / 4);   // 8(k) x 4(n) blocks of B
+  static constexpr int B_UNITS = TL::KG * TL::BNS;         // 8(k) x 1(n) columns of B
+  static constexpr int A_IT = (A_UNITS + TL::NTP - 1) / TL::NTP;
+  static constexpr int Q_IT = (Q_UNITS + TL::NTP - 1) / TL::NTP;
+  static constexpr int B_IT = (B_UNITS + TL::NTP - 1) / TL::NTP;
   static constexpr int D = TL::DEPTH;
+  static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // quads per row of the permuted part
+  static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
+  static_assert((A_IT * 2 + Q_IT * 8 + B_IT * 8) * D <= 60, "too many loads in flight for the vmcnt counter");
 
   struct Regs {
     float a[A_IT][8];
-    float b[B_IT][8];
+    float q[Q_IT > 0 ? Q_IT : 1][8][4];
+    float b[B_IT > 0 ? B_IT : 1][8];
   };
 
   struct Ctx {
     i32x4 ra, rb;
     int voff_a[A_IT];   // bytes: row * lda + kg * 8
-    int voff_b[B_IT];   // bytes: kg * 8 * ldb + col
+    int voff_q[Q_IT > 0 ? Q_IT : 1];   // bytes: kg * 8 * ldb + 4 * quad
+    int voff_b[B_IT > 0 ? B_IT : 1];   // bytes: kg * 8 * ldb + col
     int lds_a[A_IT];    // slot index inside a term plane set, -1 if this thread has no such unit
-    int lds_b[B_IT];
+    int lds_q[Q_IT > 0 ? Q_IT : 1];    // slot of column 4*quad (the other three follow at +32, +64, +96)
+    int lds_b[B_IT > 0 ? B_IT : 1];
     int ldb_bytes;
   };
 
@@ -158,11 +181,22 @@ struct TileGemm {
       c.lds_a[it] = mine ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
     }
 #pragma unroll
+    for (int it = 0; it < Q_IT; ++it) {
+      int u = ptid + it * TL::NTP;
+      const bool mine = u < Q_UNITS;
+      u = mine ? u : Q_UNITS - 1;
+      const int quad = u % QW, kg = u / QW;
+      const int last_quad = last_col >> 2;  // fast path: N % 4 == 0, a quad is wholly in or out
+      const int qc = quad < last_quad ? quad : last_quad;
+      c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc) * ES);
+      c.lds_q[it] = mine ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) : -1;
+    }
+#pragma unroll
     for (int it = 0; it < B_IT; ++it) {
       int u = ptid + it * TL::NTP;
       const bool mine = u < B_UNITS;
       u = mine ? u : B_UNITS - 1;
-      const int n = u % TL::BN, kg = u / TL::BN;
+      const int n = TL::BNQ + u % SW, kg = u / SW;
       const int nc = n < last_col ? n : last_col;
       c.voff_b[it] = (int)((kg * 8 * p.ldb + nc) * ES);
       c.lds_b[it] = mine ? kg * LL::kBPlane + n : -1;
@@ -186,6 +220,12 @@ struct TileGemm {
     for (int e = 0; e < 8; ++e) {
       const int soff_b = (k0 + e) * c.ldb_bytes;
 #pragma unroll
+      for (int it = 0; it < Q_IT; ++it) {
+        const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], soff_b, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
+      }
+#pragma unroll
       for (int it = 0; it < B_IT; ++it) r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], soff_b, 0);
     }
   }
@@ -207,11 +247,26 @@ struct TileGemm {
       for (int e = 0; e < 8; ++e) r.a[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + e) : 0.f;
     }
 #pragma unroll
+    for (int it = 0; it < Q_IT; ++it) {
+      int u = ptid + it * TL::NTP;
+      u = u < Q_UNITS ? u : Q_UNITS - 1;
+      const int quad = u % QW, kg = u / QW;
+      const int k = k0 + kg * 8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int col = n0 + 4 * quad + i;
+        col = col < p.N ? col : p.N - 1;
+        const IoT* src = B + (int64_t)k * p.ldb + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.q[it][e][i] = (k + e < p.K) ? IoType<IODT>::load(src + (int64_t)e * p.ldb) : 0.f;
+      }
+    }
+#pragma unroll
     for (int it = 0; it < B_IT; ++it) {
       int u = ptid + it * TL::NTP;
       u = u < B_UNITS ? u : B_UNITS - 1;
-      const int kg = u / TL::BN;
-      int col = n0 + u % TL::BN;
+      const int kg = u / SW;
+      int col = n0 + TL::BNQ + u % SW;
       col = col < p.N ? col : p.N - 1;
       const int k = k0 + kg * 8;
       const IoT* src = B + (int64_t)k * p.ldb + col;
@@ -220,24 +275,69 @@ struct TileGemm {
     }
   }
 
-  // ---- registers -> split -> LDS --------------------------------------------------------
-  static __device__ __forceinline__ void store(const Ctx& c, u32x4* stage, Regs& r) {
+  // ---- registers -> split -> LDS, and refill of the ring slot ----------------------------
+  // Unit by unit: split one unit, write its slots, and right away issue the loads that refill
+  // that unit's registers for K step k_next (ISSUE).  Spreading the loads between the VALU
+  // batches keeps the texture-address unit busy while the splits run; issued in one burst
+  // they would stall the wave on the full address FIFO with no VALU work to overlap.
+  template <bool ISSUE>
+  static __device__ __forceinline__ void restage(const Ctx& c, u32x4* stage, Regs& r, int k_next) {
     u32x4* sb = stage + TERMS * LL::kATerm;
+    const int soff_a = k_next * ES;
 #pragma unroll
     for (int it = 0; it < A_IT; ++it) {
-      if (A_UNITS % TL::NTP != 0 && c.lds_a[it] < 0) continue;
-      u32x4 t[TERMS];
-      split8<FMT, TERMS>(r.a[it], t);
+      if (A_UNITS % TL::NTP == 0 || c.lds_a[it] >= 0) {
+        u32x4 t[TERMS];
+        split8<FMT, TERMS>(r.a[it], t);
 #pragma unroll
-      for (int i = 0; i < TERMS; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+        for (int i = 0; i < TERMS; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+      }
+      if (ISSUE) {
+        const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
+        const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          r.a[it][e] = v0[e];
+          r.a[it][4 + e] = v1[e];
+        }
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < Q_IT; ++it) {
+      if (Q_UNITS % TL::NTP == 0 || c.lds_q[it] >= 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float x[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = r.q[it][e][i];
+          u32x4 t[TERMS];
+          split8<FMT, TERMS>(x, t);
+#pragma unroll
+          for (int tt = 0; tt < TERMS; ++tt) sb[tt * LL::kBTerm + c.lds_q[it] + i * 32] = t[tt];
+        }
+      }
+      if (ISSUE) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], (k_next + e) * c.ldb_bytes, 0);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
+        }
+      }
     }
 #pragma unroll
     for (int it = 0; it < B_IT; ++it) {
-      if (B_UNITS % TL::NTP != 0 && c.lds_b[it] < 0) continue;
-      u32x4 t[TERMS];
-      split8<FMT, TERMS>(r.b[it], t);
+      if (B_UNITS % TL::NTP == 0 || c.lds_b[it] >= 0) {
+        u32x4 t[TERMS];
+        split8<FMT, TERMS>(r.b[it], t);
 #pragma unroll
-      for (int i = 0; i < TERMS; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+        for (int i = 0; i < TERMS; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+      }
+      if (ISSUE) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], (k_next + e) * c.ldb_bytes, 0);
+      }
     }
   }
 
@@ -302,8 +402,12 @@ struct TileGemm {
     for (; s + 2 * D <= ktiles; s += D) {
 #pragma unroll
       for (int d = 0; d < D; ++d) {
-        store(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d]);
-        issue(s + d + D, ring[d]);
+        if (FAST) {
+          restage<true>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], (s + d + D) * TL::BK);
+        } else {
+          restage<false>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], 0);
+          issue(s + d + D, ring[d]);
+        }
         __syncthreads();
       }
     }
@@ -311,8 +415,12 @@ struct TileGemm {
     for (int dd = 0; dd < 2 * D; ++dd) {
       const int d = dd % D;
       if (s + dd < ktiles) {
-        store(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d]);
-        if (s + dd + D < ktiles) issue(s + dd + D, ring[d]);
+        if (FAST && s + dd + D < ktiles) {
+          restage<true>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], (s + dd + D) * TL::BK);
+        } else {
+          restage<false>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], 0);
+          if (s + dd + D < ktiles) issue(s + dd + D, ring[d]);
+        }
         __syncthreads();
       }
     }
@@ -385,14 +493,32 @@ struct TileGemm {
     IoT* C = (IoT*)p.C;
     const IoT* bias = (const IoT*)p.bias;
     const bool interior = (m0 + TL::BM <= p.M) && (n0 + TL::BN <= p.N) && p.ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
-    if (IODT == CASCMM_DT_F32 && interior) {
-      // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask.
-      // A store instruction writes two full 128-byte row segments.
+    constexpr int NQ = TL::BNQ / 32;  // leading MFMA column blocks that hold permuted columns
+    if (IODT == CASCMM_DT_F32 && interior && (p.ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0) {
+      // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask
       const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * p.ldc + n0 + wn0, 0x7FFFFFFF);
       const int ldc_bytes = (int)p.ldc * ES;
+      // permuted groups: blocks 4*gq .. 4*gq+3 of lane l31 are columns 128*gq + 4*l31 + {0..3}
+#pragma unroll
+      for (int gq = 0; gq < NQ / 4; ++gq) {
+        const int voff = g * 4 * ldc_bytes + (gq * 128 + 4 * l31) * ES;
+        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+        if (bias) bv = *(const f32x4*)(bias + n0 + wn0 + gq * 128 + 4 * l31);
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const f32x4 v = {res[mi][4 * gq][4 * q + e] + bv[0], res[mi][4 * gq + 1][4 * q + e] + bv[1],
+                               res[mi][4 * gq + 2][4 * q + e] + bv[2], res[mi][4 * gq + 3][4 * q + e] + bv[3]};
+              llvm_raw_buffer_store_v4f32(v, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+            }
+      }
+      // unpermuted blocks: a store instruction writes two full 128-byte row segments
       const int voff = g * 4 * ldc_bytes + l31 * ES;
 #pragma unroll
-      for (int ni = 0; ni < TL::NTL; ++ni) {
+      for (int ni = NQ; ni < TL::NTL; ++ni) {
         const float bv = bias ? IoType<IODT>::load(bias + n0 + wn0 + ni * 32 + l31) : 0.f;
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi)
@@ -407,7 +533,7 @@ struct TileGemm {
     }
 #pragma unroll
     for (int ni = 0; ni < TL::NTL; ++ni) {
-      const int col = n0 + wn0 + ni * 32 + l31;
+      const int col = n0 + wn0 + (ni < NQ ? (ni >> 2) * 128 + 4 * l31 + (ni & 3) : ni * 32 + l31);
       if (col >= p.N) continue;
       const float bv = bias ? IoType<IODT>::load(bias + col) : 0.f;
 #pragma unroll

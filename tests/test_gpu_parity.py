@@ -68,7 +68,7 @@ def _int_case(M, K, N, hi, seed):
 
 
 INT_SHAPES = [(16, 32, 16), (17, 33, 19), (154, 64, 48), (1, 7, 1), (130, 40, 81), (256, 192, 160), (300, 128, 200),
-              (257, 64, 161)]
+              (257, 64, 161), (257, 64, 164), (96, 128, 384)]
 
 
 @pytest.mark.parametrize("shape", INT_SHAPES)
@@ -85,8 +85,8 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
         terms = int(name.split(fmt + "x")[1][0])
         products = "full" if "_full" in name else "tri"
         bk = int(name.split("_")[0].split("x")[2])
-        if "generic" not in name and (K % bk != 0):
-            continue  # fast variants need K % BK == 0 (rejected by the library otherwise)
+        if "generic" not in name and (K % bk != 0 or N % 4 != 0):
+            continue  # fast variants need K % BK == 0 and N % 4 == 0 (rejected by the library otherwise)
         _say("int-exact", shape, name)
         out = cascaded_lowp_matmul(at, bt, lowp=fmt, terms=terms, products=products, variant=vi)
         torch.cuda.synchronize()
