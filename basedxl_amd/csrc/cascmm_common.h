@@ -123,6 +123,9 @@ template <int FMT, int TERMS, bool FULL> struct AccClasses {
   static constexpr int kCount = kScaled ? ProductSet<TERMS, FULL>::kClasses : (TERMS >= 3 ? 3 : 1);
   static constexpr float kFoldScale = kScaled ? 1.0f / (float)(1 << Lowp<FMT>::kShift) : 1.0f;
   static constexpr __host__ __device__ int index(int s) { return kCount == 1 ? 0 : (s < kCount ? s : kCount - 1); }
+  // cascades that reach the fp32 rounding floor accumulate class 0 in blocks of kChunkK
+  static constexpr bool kChunked = kScaled ? (TERMS >= 2) : (TERMS >= 3);
+  static constexpr int kChunkK = 256;
 };
 
 struct GemmParams {

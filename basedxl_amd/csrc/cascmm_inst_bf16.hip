@@ -8,21 +8,21 @@ namespace cascmm {
 
 static const VariantDesc kTable[] = {
     // headline: two terms, three products.  name, BM, BN, BK, WM, WN, WK, DEPTH (4 producer waves)
-    CASCMM_TILE_VARIANT("t64x160x64_w2x1x2_d3_bf16x2_tri", 64, 160, 64, 2, 1, 2, 3, F32, BF, 2, false, true),
-    CASCMM_TILE_VARIANT("t256x128x32_w4x1x1_d3_bf16x2_tri", 256, 128, 32, 4, 1, 1, 3, F32, BF, 2, false, true),
-    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d4_bf16x2_tri", 128, 128, 32, 4, 1, 1, 4, F32, BF, 2, false, true),
+    CASCMM_TILE_VARIANT("t64x160x64_w2x1x2_d2_bf16x2_tri", 64, 160, 64, 2, 1, 2, 2, F32, BF, 2, false, true),
+    CASCMM_TILE_VARIANT("t256x128x32_w4x1x1_d2_bf16x2_tri", 256, 128, 32, 4, 1, 1, 2, F32, BF, 2, false, true),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d3_bf16x2_tri", 128, 128, 32, 4, 1, 1, 3, F32, BF, 2, false, true),
     CASCMM_TILE_VARIANT("t128x128x64_w2x1x2_d2_bf16x2_tri", 128, 128, 64, 2, 1, 2, 2, F32, BF, 2, false, true),
     CASCMM_TILE_VARIANT("t64x128x64_w2x1x2_d3_bf16x2_tri", 64, 128, 64, 2, 1, 2, 3, F32, BF, 2, false, true),
     CASCMM_TILE_VARIANT("t64x64x64_w2x2x1_d3_bf16x2_tri", 64, 64, 64, 2, 2, 1, 3, F32, BF, 2, false, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x2_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 2, false, false),
     // other term counts / product sets
-    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d4_bf16x1", 128, 128, 32, 4, 1, 1, 4, F32, BF, 1, false, true),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d3_bf16x1", 128, 128, 32, 4, 1, 1, 3, F32, BF, 1, false, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x1_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 1, false, false),
-    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d4_bf16x2_full", 128, 128, 32, 4, 1, 1, 4, F32, BF, 2, true, true),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d3_bf16x2_full", 128, 128, 32, 4, 1, 1, 3, F32, BF, 2, true, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x2_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 2, true, false),
-    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d4_bf16x3_tri", 128, 128, 32, 4, 1, 1, 4, F32, BF, 3, false, true),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_bf16x3_tri", 128, 128, 32, 4, 2, 1, 2, F32, BF, 3, false, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x3_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 3, false, false),
-    CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d4_bf16x3_full", 128, 128, 32, 4, 1, 1, 4, F32, BF, 3, true, true),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_bf16x3_full", 128, 128, 32, 4, 2, 1, 2, F32, BF, 3, true, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x3_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 3, true, false),
 };
 

@@ -59,7 +59,9 @@ struct Tile {
   // B columns: the first BNQ (whole groups of 128) are loaded four at a time (16-byte loads)
   // and stored permuted in LDS; the remaining BNS columns are loaded one at a time.
   static constexpr int BNQ = (BN / 128) * 128, BNS = BN - BNQ;
-  static_assert(BNQ == 0 || WN == 1, "permuted B columns need one consumer wave column");
+  // a consumer wave must own whole runs of permuted blocks: all four of a group, or two
+  static_assert(BNQ == 0 || WTN % 128 == 0 || WTN == 64 || (WN == 1), "wave tile vs permuted B columns");
+  static_assert(BNQ == 0 || WN == 1 || BNS == 0, "mixed B column layouts need one consumer wave column");
   static_assert(BK == 32 || BK == 64 || BK == 128, "BK");
   static_assert(BM % (32 * WM) == 0 && BN % (32 * WN) == 0, "wave tile must be a multiple of 32");
   static_assert(KSUB % WK == 0, "k slices must divide evenly among the wave groups");
@@ -111,6 +113,8 @@ __device__ float llvm_raw_buffer_load_f32(i32x4 rsrc, int voffset, int soffset, 
 __device__ f32x4 llvm_raw_buffer_load_v4f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
 __device__ void llvm_raw_buffer_store_f32(float v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.f32");
 __device__ void llvm_raw_buffer_store_v4f32(f32x4 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v4f32");
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ void llvm_raw_buffer_store_v2f32(f32x2 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v2f32");
 
 // gfx9-family raw buffer descriptor: 48-bit base, stride 0, byte count, 32-bit data format
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
@@ -444,10 +448,41 @@ struct TileGemm {
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[c][mi][ni][e] = 0.f;
 
+    // Blocked accumulation for the cascades whose error sits at the fp32 rounding floor: the
+    // big class-0 sum is collected in chunks of kChunkK and the chunks are added into a master
+    // accumulator, so the chunk sums round at a fraction of the final magnitude and the master
+    // rounds K / kChunkK times instead of K / 16 times.
+    f32x16 master[AC::kChunked ? TL::MT : 1][AC::kChunked ? TL::NTL : 1];
+    if constexpr (AC::kChunked) {
+#pragma unroll
+      for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < TL::NTL; ++ni)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) master[mi][ni][e] = 0.f;
+    }
+    constexpr int kChunkSteps = (AC::kChunkK / TL::BK) > 0 ? (AC::kChunkK / TL::BK) : 1;
+
     __syncthreads();
     for (int kt = 0; kt < ktiles; ++kt) {
       compute(lds + (kt & 1) * LL::kStage, wm0, wn0, wk, acc);
+      if constexpr (AC::kChunked) if ((kt % kChunkSteps) == kChunkSteps - 1) {
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < TL::NTL; ++ni) {
+            master[mi][ni] += acc[0][mi][ni];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[0][mi][ni][e] = 0.f;
+          }
+      }
       __syncthreads();
+    }
+    if constexpr (AC::kChunked) {
+#pragma unroll
+      for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < TL::NTL; ++ni) acc[0][mi][ni] += master[mi][ni];
     }
 
     // fold the scale classes (smallest first), then the cross-wave-group reduction (WK == 2):
@@ -493,47 +528,62 @@ struct TileGemm {
     IoT* C = (IoT*)p.C;
     const IoT* bias = (const IoT*)p.bias;
     const bool interior = (m0 + TL::BM <= p.M) && (n0 + TL::BN <= p.N) && p.ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
-    constexpr int NQ = TL::BNQ / 32;  // leading MFMA column blocks that hold permuted columns
-    if (IODT == CASCMM_DT_F32 && interior && (p.ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0) {
+    // Column blocks of this wave that hold permuted columns come in runs of RUN blocks of one
+    // 128-column group: block b of the tile (b = wn0/32 + ni), lane l31 <-> column
+    // 128*(b/4) + 4*l31 + b%4.
+    constexpr int NQ = (TL::BNQ == 0) ? 0 : (TL::WN == 1 ? TL::BNQ / 32 : TL::NTL);
+    constexpr int RUN = (NQ % 4 == 0) ? 4 : 2;
+    const int b0 = wn0 >> 5;
+    if (IODT == CASCMM_DT_F32 && interior && (p.ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0 &&
+        (bias == nullptr || (((uintptr_t)bias) & 15) == 0)) {
       // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask
-      const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * p.ldc + n0 + wn0, 0x7FFFFFFF);
+      const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * p.ldc + n0, 0x7FFFFFFF);
       const int ldc_bytes = (int)p.ldc * ES;
-      // permuted groups: blocks 4*gq .. 4*gq+3 of lane l31 are columns 128*gq + 4*l31 + {0..3}
 #pragma unroll
-      for (int gq = 0; gq < NQ / 4; ++gq) {
-        const int voff = g * 4 * ldc_bytes + (gq * 128 + 4 * l31) * ES;
-        f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-        if (bias) bv = *(const f32x4*)(bias + n0 + wn0 + gq * 128 + 4 * l31);
+      for (int r0 = 0; r0 < NQ; r0 += RUN) {
+        const int b = b0 + r0;
+        const int col = (b >> 2) * 128 + 4 * l31 + (b & 3);
+        const int voff = g * 4 * ldc_bytes + col * ES;
+        float bv[RUN];
+#pragma unroll
+        for (int i = 0; i < RUN; ++i) bv[i] = bias ? IoType<IODT>::load(bias + n0 + col + i) : 0.f;
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const f32x4 v = {res[mi][4 * gq][4 * q + e] + bv[0], res[mi][4 * gq + 1][4 * q + e] + bv[1],
-                               res[mi][4 * gq + 2][4 * q + e] + bv[2], res[mi][4 * gq + 3][4 * q + e] + bv[3]};
-              llvm_raw_buffer_store_v4f32(v, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+              const int soff = (mi * 32 + q * 8 + e) * ldc_bytes;
+              if constexpr (RUN == 4) {
+                const f32x4 v = {res[mi][r0][4 * q + e] + bv[0], res[mi][r0 + 1][4 * q + e] + bv[1],
+                                 res[mi][r0 + 2][4 * q + e] + bv[2], res[mi][r0 + 3][4 * q + e] + bv[3]};
+                llvm_raw_buffer_store_v4f32(v, rc, voff, soff, 0);
+              } else {
+                const f32x2 v = {res[mi][r0][4 * q + e] + bv[0], res[mi][r0 + 1][4 * q + e] + bv[1]};
+                llvm_raw_buffer_store_v2f32(v, rc, voff, soff, 0);
+              }
             }
       }
       // unpermuted blocks: a store instruction writes two full 128-byte row segments
-      const int voff = g * 4 * ldc_bytes + l31 * ES;
 #pragma unroll
       for (int ni = NQ; ni < TL::NTL; ++ni) {
-        const float bv = bias ? IoType<IODT>::load(bias + n0 + wn0 + ni * 32 + l31) : 0.f;
+        const int col = wn0 + ni * 32 + l31;
+        const int voff = g * 4 * ldc_bytes + col * ES;
+        const float bv = bias ? IoType<IODT>::load(bias + n0 + col) : 0.f;
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              llvm_raw_buffer_store_f32(res[mi][ni][4 * q + e] + bv, rc, voff,
-                                        (mi * 32 + q * 8 + e) * ldc_bytes + ni * 32 * ES, 0);
+              llvm_raw_buffer_store_f32(res[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
       }
       return;
     }
 #pragma unroll
     for (int ni = 0; ni < TL::NTL; ++ni) {
-      const int col = n0 + wn0 + (ni < NQ ? (ni >> 2) * 128 + 4 * l31 + (ni & 3) : ni * 32 + l31);
+      const int b = b0 + ni;
+      const int col = n0 + (ni < NQ ? (b >> 2) * 128 + 4 * l31 + (b & 3) : wn0 + ni * 32 + l31);
       if (col >= p.N) continue;
       const float bv = bias ? IoType<IODT>::load(bias + col) : 0.f;
 #pragma unroll
