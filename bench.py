@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path shards by rows of A with no "
@@ -112,6 +115,14 @@ def main():
     err_o = oc.error_metrics(oc.cascade_matmul_ref(cpu_in[1], cpu_in[2][3], "bf16", 2, "tri"), exp)
     if not (err_k["rel_fro"] <= 1.25 * err_o["rel_fro"] and err_k["max_abs"] <= 1.25 * err_o["max_abs"]):
         sys.exit(f"bench.py: kernel error {err_k} exceeds 1.25x the oracle cascade's {err_o}")
+
+    if args.copy_calibration:
+        src = torch.empty(64 * 1024 * 1024, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     graph = None
     if not args.no_graph:
