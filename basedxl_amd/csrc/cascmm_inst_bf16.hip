@@ -14,6 +14,14 @@ static const VariantDesc kTable[] = {
     CASCMM_TILE_VARIANT("t128x128x64_w2x1x2_d2_bf16x2_tri", 128, 128, 64, 2, 1, 2, 2, F32, BF, 2, false, true),
     CASCMM_TILE_VARIANT("t64x128x64_w2x1x2_d3_bf16x2_tri", 64, 128, 64, 2, 1, 2, 3, F32, BF, 2, false, true),
     CASCMM_TILE_VARIANT("t64x64x64_w2x2x1_d3_bf16x2_tri", 64, 64, 64, 2, 2, 1, 3, F32, BF, 2, false, true),
+    CASCMM_TILE_VARIANT_P("t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 64, 160, 64, 2, 1, 2, 2, 8, F32, BF, 2, false, true),
+    CASCMM_TILE_VARIANT_P("t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 128, 128, 64, 4, 1, 1, 2, 8, F32, BF, 2, false, true),
+    CASCMM_BD_VARIANT("bd128x128x64_d3_p4_bf16x2_tri", 128, 4, 64, 3, 4, BF, 2, false),
+    CASCMM_BD_VARIANT("bd96x128x64_d3_p4_bf16x2_tri", 96, 4, 64, 3, 4, BF, 2, false),
+    CASCMM_BD_VARIANT("bd64x128x64_d3_p4_bf16x2_tri", 64, 4, 64, 3, 4, BF, 2, false),
+    CASCMM_BD_VARIANT("bd192x128x64_d2_p4_bf16x2_tri", 192, 4, 64, 2, 4, BF, 2, false),
+    CASCMM_BD_VARIANT("bd128x128x32_d3_p4_bf16x2_tri", 128, 4, 32, 3, 4, BF, 2, false),
+    CASCMM_BD_VARIANT("bd128x128x64_d3_p2_bf16x2_tri", 128, 4, 64, 3, 2, BF, 2, false),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x2_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 2, false, false),
     // other term counts / product sets
     CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d3_bf16x1", 128, 128, 32, 4, 1, 1, 3, F32, BF, 1, false, true),

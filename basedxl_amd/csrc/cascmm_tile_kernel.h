@@ -140,163 +140,97 @@ struct TileGemm {
   static constexpr int A_UNITS = TL::KG * TL::BM;
   static constexpr int Q_UNITS = TL::KG * (TL::BNQ / 4);   // 8(k) x 4(n) blocks of B
   static constexpr int B_UNITS = TL::KG * TL::BNS;         // 8(k) x 1(n) columns of B
-  static constexpr int A_IT = (A_UNITS + TL::NTP - 1) / TL::NTP;
-  static constexpr int Q_IT = (Q_UNITS + TL::NTP - 1) / TL::NTP;
-  static constexpr int B_IT = (B_UNITS + TL::NTP - 1) / TL::NTP;
   static constexpr int D = TL::DEPTH;
   static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // quads per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
-  static_assert((A_IT * 2 + Q_IT * 8 + B_IT * 8) * D <= 60, "too many loads in flight for the vmcnt counter");
 
-  struct Regs {
-    float a[A_IT][8];
-    float q[Q_IT > 0 ? Q_IT : 1][8][4];
-    float b[B_IT > 0 ? B_IT : 1][8];
-  };
+  // ---- producer waves: global -> split -> LDS, one stage per barrier interval -----------------
+  // Barrier protocol (both kinds of wave execute exactly ktiles + 1 barriers, plus one more
+  // for the WK reduction):
+  //   producer:  store(0) B0 store(1) B1 ... store(kt-1) B(kt-1)            B(kt)
+  //   consumer:           B0 compute(0) B1 ... compute(kt-2) B(kt-1) compute(kt-1) B(kt)
+  // store(s) writes LDS buffer s&1 between B(s-1) and B(s); the last reader of that buffer,
+  // compute(s-2), finished before B(s-1), and its first reader, compute(s), starts after B(s).
+  //
+  // ROLE says which staging units a producer wave handles: every kind (kAll), or, when the
+  // workgroup has eight producer waves, the 8x4 blocks of B for the first four (kQuads) and A
+  // plus the single B columns for the last four (kRest).  Two producer waves per SIMD with
+  // different roles keep the VALU busy while the other wave waits on the LDS or load queues.
+  enum { kAll = 0, kQuads = 1, kRest = 2 };
+  template <int ROLE>
+  struct Prod {
+    static constexpr bool HAS_A = ROLE != kQuads, HAS_Q = ROLE != kRest, HAS_S = ROLE != kQuads;
+    static constexpr int NTR = ROLE == kAll ? TL::NTP : TL::NTP / 2;    // threads of this role
+    static constexpr int T0 = ROLE == kRest ? TL::NTP / 2 : 0;          // first producer thread of it
+    static constexpr int A_IT = HAS_A ? (A_UNITS + NTR - 1) / NTR : 0;
+    static constexpr int Q_IT = HAS_Q ? (Q_UNITS + NTR - 1) / NTR : 0;
+    static constexpr int B_IT = HAS_S ? (B_UNITS + NTR - 1) / NTR : 0;
+    static_assert((A_IT * 2 + Q_IT * 8 + B_IT * 8) * D <= 60, "too many loads in flight for the vmcnt counter");
 
-  struct Ctx {
-    i32x4 ra, rb;
-    int voff_a[A_IT];   // bytes: row * lda + kg * 8
-    int voff_q[Q_IT > 0 ? Q_IT : 1];   // bytes: kg * 8 * ldb + 4 * quad
-    int voff_b[B_IT > 0 ? B_IT : 1];   // bytes: kg * 8 * ldb + col
-    int lds_a[A_IT];    // slot index inside a term plane set, -1 if this thread has no such unit
-    int lds_q[Q_IT > 0 ? Q_IT : 1];    // slot of column 4*quad (the other three follow at +32, +64, +96)
-    int lds_b[B_IT > 0 ? B_IT : 1];
-    int ldb_bytes;
-  };
+    struct Regs {
+      float a[A_IT > 0 ? A_IT : 1][8];
+      float q[Q_IT > 0 ? Q_IT : 1][8][4];
+      float b[B_IT > 0 ? B_IT : 1][8];
+    };
 
-  static __device__ __forceinline__ void init_ctx(Ctx& c, const GemmParams& p, int m0, int n0, int ptid) {
-    const IoT* A = (const IoT*)p.A + (int64_t)m0 * p.lda;
-    const IoT* B = (const IoT*)p.B + n0;
-    // bytes from the tile origin to the end of the matrix; rows and columns are also clamped
-    // below, so no access relies on the hardware range check
-    c.ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
-    c.rb = make_rsrc(B, ((int64_t)(p.K - 1) * p.ldb + (p.N - n0)) * ES);
-    c.ldb_bytes = (int)(p.ldb * ES);
-    const int last_row = p.M - 1 - m0, last_col = p.N - 1 - n0;
-#pragma unroll
-    for (int it = 0; it < A_IT; ++it) {
-      int u = ptid + it * TL::NTP;
-      const bool mine = u < A_UNITS;
-      u = mine ? u : A_UNITS - 1;
-      const int kg = u % TL::KG, r = u / TL::KG;
-      const int rc = r < last_row ? r : last_row;
-      c.voff_a[it] = (int)((rc * p.lda + kg * 8) * ES);
-      c.lds_a[it] = mine ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
-    }
-#pragma unroll
-    for (int it = 0; it < Q_IT; ++it) {
-      int u = ptid + it * TL::NTP;
-      const bool mine = u < Q_UNITS;
-      u = mine ? u : Q_UNITS - 1;
-      const int quad = u % QW, kg = u / QW;
-      const int last_quad = last_col >> 2;  // fast path: N % 4 == 0, a quad is wholly in or out
-      const int qc = quad < last_quad ? quad : last_quad;
-      c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc) * ES);
-      c.lds_q[it] = mine ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) : -1;
-    }
-#pragma unroll
-    for (int it = 0; it < B_IT; ++it) {
-      int u = ptid + it * TL::NTP;
-      const bool mine = u < B_UNITS;
-      u = mine ? u : B_UNITS - 1;
-      const int n = TL::BNQ + u % SW, kg = u / SW;
-      const int nc = n < last_col ? n : last_col;
-      c.voff_b[it] = (int)((kg * 8 * p.ldb + nc) * ES);
-      c.lds_b[it] = mine ? kg * LL::kBPlane + n : -1;
-    }
-  }
+    struct Ctx {
+      i32x4 ra, rb;
+      int voff_a[A_IT > 0 ? A_IT : 1];   // bytes: row * lda + kg * 8
+      int voff_q[Q_IT > 0 ? Q_IT : 1];   // bytes: kg * 8 * ldb + 4 * quad
+      int voff_b[B_IT > 0 ? B_IT : 1];   // bytes: kg * 8 * ldb + col
+      int lds_a[A_IT > 0 ? A_IT : 1];    // slot index inside a term plane set, -1 if this thread has no such unit
+      int lds_q[Q_IT > 0 ? Q_IT : 1];    // slot of column 4*quad (the other three follow at +32, +64, +96)
+      int lds_b[B_IT > 0 ? B_IT : 1];
+      int ldb_bytes;
+    };
 
-  // ---- global -> registers (fast path: fp32, K % BK == 0, 16-byte aligned A rows) ---------
-  static __device__ __forceinline__ void load_fast(const Ctx& c, int k0, Regs& r) {
-    const int soff_a = k0 * ES;
+    static __device__ __forceinline__ void init_ctx(Ctx& c, const GemmParams& p, int m0, int n0, int rtid) {
+      const IoT* A = (const IoT*)p.A + (int64_t)m0 * p.lda;
+      const IoT* B = (const IoT*)p.B + n0;
+      // bytes from the tile origin to the end of the matrix; rows and columns are also clamped
+      // below, so no access relies on the hardware range check
+      c.ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
+      c.rb = make_rsrc(B, ((int64_t)(p.K - 1) * p.ldb + (p.N - n0)) * ES);
+      c.ldb_bytes = (int)(p.ldb * ES);
+      const int last_row = p.M - 1 - m0, last_col = p.N - 1 - n0;
 #pragma unroll
-    for (int it = 0; it < A_IT; ++it) {
-      const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
-      const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        r.a[it][e] = v0[e];
-        r.a[it][4 + e] = v1[e];
+      for (int it = 0; it < A_IT; ++it) {
+        int u = rtid + it * NTR;
+        const bool mine = u < A_UNITS;
+        u = mine ? u : A_UNITS - 1;
+        const int kg = u % TL::KG, r = u / TL::KG;
+        const int rc = r < last_row ? r : last_row;
+        c.voff_a[it] = (int)((rc * p.lda + kg * 8) * ES);
+        c.lds_a[it] = mine ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
       }
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int soff_b = (k0 + e) * c.ldb_bytes;
 #pragma unroll
       for (int it = 0; it < Q_IT; ++it) {
-        const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], soff_b, 0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
+        int u = rtid + it * NTR;
+        const bool mine = u < Q_UNITS;
+        u = mine ? u : Q_UNITS - 1;
+        const int quad = u % QW, kg = u / QW;
+        const int last_quad = last_col >> 2;  // fast path: N % 4 == 0, a quad is wholly in or out
+        const int qc = quad < last_quad ? quad : last_quad;
+        c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc) * ES);
+        c.lds_q[it] = mine ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) : -1;
       }
 #pragma unroll
-      for (int it = 0; it < B_IT; ++it) r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], soff_b, 0);
+      for (int it = 0; it < B_IT; ++it) {
+        int u = rtid + it * NTR;
+        const bool mine = u < B_UNITS;
+        u = mine ? u : B_UNITS - 1;
+        const int n = TL::BNQ + u % SW, kg = u / SW;
+        const int nc = n < last_col ? n : last_col;
+        c.voff_b[it] = (int)((kg * 8 * p.ldb + nc) * ES);
+        c.lds_b[it] = mine ? kg * LL::kBPlane + n : -1;
+      }
     }
-  }
 
-  // ---- global -> registers (generic: any dtype, any K, element-wise, bounds-checked) ------
-  static __device__ __forceinline__ void load_generic(const GemmParams& p, int m0, int n0, int k0, int ptid, Regs& r) {
-    const IoT* A = (const IoT*)p.A;
-    const IoT* B = (const IoT*)p.B;
+    // global -> registers (fast path: fp32, K % BK == 0, 16-byte aligned rows)
+    static __device__ __forceinline__ void load_fast(const Ctx& c, int k0, Regs& r) {
+      const int soff_a = k0 * ES;
 #pragma unroll
-    for (int it = 0; it < A_IT; ++it) {
-      int u = ptid + it * TL::NTP;
-      u = u < A_UNITS ? u : A_UNITS - 1;
-      const int kg = u % TL::KG;
-      int row = m0 + u / TL::KG;
-      row = row < p.M ? row : p.M - 1;
-      const int k = k0 + kg * 8;
-      const IoT* src = A + (int64_t)row * p.lda + k;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) r.a[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + e) : 0.f;
-    }
-#pragma unroll
-    for (int it = 0; it < Q_IT; ++it) {
-      int u = ptid + it * TL::NTP;
-      u = u < Q_UNITS ? u : Q_UNITS - 1;
-      const int quad = u % QW, kg = u / QW;
-      const int k = k0 + kg * 8;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int col = n0 + 4 * quad + i;
-        col = col < p.N ? col : p.N - 1;
-        const IoT* src = B + (int64_t)k * p.ldb + col;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) r.q[it][e][i] = (k + e < p.K) ? IoType<IODT>::load(src + (int64_t)e * p.ldb) : 0.f;
-      }
-    }
-#pragma unroll
-    for (int it = 0; it < B_IT; ++it) {
-      int u = ptid + it * TL::NTP;
-      u = u < B_UNITS ? u : B_UNITS - 1;
-      const int kg = u / SW;
-      int col = n0 + TL::BNQ + u % SW;
-      col = col < p.N ? col : p.N - 1;
-      const int k = k0 + kg * 8;
-      const IoT* src = B + (int64_t)k * p.ldb + col;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) r.b[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + (int64_t)e * p.ldb) : 0.f;
-    }
-  }
-
-  // ---- registers -> split -> LDS, and refill of the ring slot ----------------------------
-  // Unit by unit: split one unit, write its slots, and right away issue the loads that refill
-  // that unit's registers for K step k_next (ISSUE).  Spreading the loads between the VALU
-  // batches keeps the texture-address unit busy while the splits run; issued in one burst
-  // they would stall the wave on the full address FIFO with no VALU work to overlap.
-  template <bool ISSUE>
-  static __device__ __forceinline__ void restage(const Ctx& c, u32x4* stage, Regs& r, int k_next) {
-    u32x4* sb = stage + TERMS * LL::kATerm;
-    const int soff_a = k_next * ES;
-#pragma unroll
-    for (int it = 0; it < A_IT; ++it) {
-      if (A_UNITS % TL::NTP == 0 || c.lds_a[it] >= 0) {
-        u32x4 t[TERMS];
-        split8<FMT, TERMS>(r.a[it], t);
-#pragma unroll
-        for (int i = 0; i < TERMS; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
-      }
-      if (ISSUE) {
+      for (int it = 0; it < A_IT; ++it) {
         const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
         const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
 #pragma unroll
@@ -305,45 +239,175 @@ struct TileGemm {
           r.a[it][4 + e] = v1[e];
         }
       }
-    }
 #pragma unroll
-    for (int it = 0; it < Q_IT; ++it) {
-      if (Q_UNITS % TL::NTP == 0 || c.lds_q[it] >= 0) {
+      for (int e = 0; e < 8; ++e) {
+        const int soff_b = (k0 + e) * c.ldb_bytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          float x[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = r.q[it][e][i];
-          u32x4 t[TERMS];
-          split8<FMT, TERMS>(x, t);
-#pragma unroll
-          for (int tt = 0; tt < TERMS; ++tt) sb[tt * LL::kBTerm + c.lds_q[it] + i * 32] = t[tt];
-        }
-      }
-      if (ISSUE) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], (k_next + e) * c.ldb_bytes, 0);
+        for (int it = 0; it < Q_IT; ++it) {
+          const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], soff_b, 0);
 #pragma unroll
           for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
         }
+#pragma unroll
+        for (int it = 0; it < B_IT; ++it) r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], soff_b, 0);
       }
     }
+
+    // global -> registers (generic: any dtype, any K, element-wise, bounds-checked)
+    static __device__ __forceinline__ void load_generic(const GemmParams& p, int m0, int n0, int k0, int rtid, Regs& r) {
+      const IoT* A = (const IoT*)p.A;
+      const IoT* B = (const IoT*)p.B;
 #pragma unroll
-    for (int it = 0; it < B_IT; ++it) {
-      if (B_UNITS % TL::NTP == 0 || c.lds_b[it] >= 0) {
-        u32x4 t[TERMS];
-        split8<FMT, TERMS>(r.b[it], t);
+      for (int it = 0; it < A_IT; ++it) {
+        int u = rtid + it * NTR;
+        u = u < A_UNITS ? u : A_UNITS - 1;
+        const int kg = u % TL::KG;
+        int row = m0 + u / TL::KG;
+        row = row < p.M ? row : p.M - 1;
+        const int k = k0 + kg * 8;
+        const IoT* src = A + (int64_t)row * p.lda + k;
 #pragma unroll
-        for (int i = 0; i < TERMS; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+        for (int e = 0; e < 8; ++e) r.a[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + e) : 0.f;
       }
-      if (ISSUE) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], (k_next + e) * c.ldb_bytes, 0);
+      for (int it = 0; it < Q_IT; ++it) {
+        int u = rtid + it * NTR;
+        u = u < Q_UNITS ? u : Q_UNITS - 1;
+        const int quad = u % QW, kg = u / QW;
+        const int k = k0 + kg * 8;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          int col = n0 + 4 * quad + i;
+          col = col < p.N ? col : p.N - 1;
+          const IoT* src = B + (int64_t)k * p.ldb + col;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) r.q[it][e][i] = (k + e < p.K) ? IoType<IODT>::load(src + (int64_t)e * p.ldb) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < B_IT; ++it) {
+        int u = rtid + it * NTR;
+        u = u < B_UNITS ? u : B_UNITS - 1;
+        const int kg = u / SW;
+        int col = n0 + TL::BNQ + u % SW;
+        col = col < p.N ? col : p.N - 1;
+        const int k = k0 + kg * 8;
+        const IoT* src = B + (int64_t)k * p.ldb + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.b[it][e] = (k + e < p.K) ? IoType<IODT>::load(src + (int64_t)e * p.ldb) : 0.f;
       }
     }
-  }
+
+    // registers -> split -> LDS, and refill of the ring slot.
+    // Unit by unit: split one unit, write its slots, and right away issue the loads that refill
+    // that unit's registers for K step k_next (ISSUE).  Spreading the loads between the VALU
+    // batches keeps the texture-address unit busy while the splits run; issued in one burst
+    // they would stall the wave on the full address FIFO with no VALU work to overlap.
+    template <bool ISSUE>
+    static __device__ __forceinline__ void restage(const Ctx& c, u32x4* stage, Regs& r, int k_next) {
+      u32x4* sb = stage + TERMS * LL::kATerm;
+      const int soff_a = k_next * ES;
+#pragma unroll
+      for (int it = 0; it < A_IT; ++it) {
+        if (A_UNITS % NTR == 0 || c.lds_a[it] >= 0) {
+          u32x4 t[TERMS];
+          split8<FMT, TERMS>(r.a[it], t);
+#pragma unroll
+          for (int i = 0; i < TERMS; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+        }
+        if (ISSUE) {
+          const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
+          const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            r.a[it][e] = v0[e];
+            r.a[it][4 + e] = v1[e];
+          }
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < Q_IT; ++it) {
+        if (Q_UNITS % NTR == 0 || c.lds_q[it] >= 0) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = r.q[it][e][i];
+            u32x4 t[TERMS];
+            split8<FMT, TERMS>(x, t);
+#pragma unroll
+            for (int tt = 0; tt < TERMS; ++tt) sb[tt * LL::kBTerm + c.lds_q[it] + i * 32] = t[tt];
+          }
+        }
+        if (ISSUE) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], (k_next + e) * c.ldb_bytes, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
+          }
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < B_IT; ++it) {
+        if (B_UNITS % NTR == 0 || c.lds_b[it] >= 0) {
+          u32x4 t[TERMS];
+          split8<FMT, TERMS>(r.b[it], t);
+#pragma unroll
+          for (int i = 0; i < TERMS; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+        }
+        if (ISSUE) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], (k_next + e) * c.ldb_bytes, 0);
+        }
+      }
+    }
+
+    template <bool FAST>
+    static __device__ __forceinline__ void loop(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles) {
+      const int rtid = threadIdx.x - TL::NCW * kWave - T0;
+      Ctx ctx;
+      init_ctx(ctx, p, m0, n0, rtid);
+      Regs ring[D];
+      // loads are only ever issued for k steps that exist (s < ktiles)
+      auto issue = [&](int s, Regs& r) {
+        if (FAST) load_fast(ctx, s * TL::BK, r);
+        else load_generic(p, m0, n0, s * TL::BK, rtid, r);
+      };
+#pragma unroll
+      for (int d = 0; d < D; ++d)
+        if (d < ktiles) issue(d, ring[d]);
+      int s = 0;
+      for (; s + 2 * D <= ktiles; s += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+          if (FAST) {
+            restage<true>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], (s + d + D) * TL::BK);
+          } else {
+            restage<false>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], 0);
+            issue(s + d + D, ring[d]);
+          }
+          __syncthreads();
+        }
+      }
+#pragma unroll
+      for (int dd = 0; dd < 2 * D; ++dd) {
+        const int d = dd % D;
+        if (s + dd < ktiles) {
+          if (FAST && s + dd + D < ktiles) {
+            restage<true>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], (s + dd + D) * TL::BK);
+          } else {
+            restage<false>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], 0);
+            if (s + dd + D < ktiles) issue(s + dd + D, ring[d]);
+          }
+          __syncthreads();
+        }
+      }
+      __syncthreads();
+      if (TL::WK > 1) __syncthreads();
+    }
+  };
 
   // ---- LDS -> MFMA ----------------------------------------------------------------------
   static __device__ __forceinline__ void compute(const u32x4* stage, int wm0, int wn0, int wk,
@@ -379,57 +443,6 @@ struct TileGemm {
             for (int ni = 0; ni < TL::NTL; ++ni) acc[cls][mi][ni] = LP::mfma(a[i][mi], b[j][ni], acc[cls][mi][ni]);
         }
     }
-  }
-
-  // ---- producer waves: global -> split -> LDS, one stage per barrier interval -----------------
-  // Barrier protocol (both kinds of wave execute exactly ktiles + 1 barriers, plus one more
-  // for the WK reduction):
-  //   producer:  store(0) B0 store(1) B1 ... store(kt-1) B(kt-1)            B(kt)
-  //   consumer:           B0 compute(0) B1 ... compute(kt-2) B(kt-1) compute(kt-1) B(kt)
-  // store(s) writes LDS buffer s&1 between B(s-1) and B(s); the last reader of that buffer,
-  // compute(s-2), finished before B(s-1), and its first reader, compute(s), starts after B(s).
-  template <bool FAST>
-  static __device__ __forceinline__ void producer(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles) {
-    const int ptid = threadIdx.x - TL::NCW * kWave;
-    Ctx ctx;
-    init_ctx(ctx, p, m0, n0, ptid);
-    Regs ring[D];
-    // loads are only ever issued for k steps that exist (s < ktiles)
-    auto issue = [&](int s, Regs& r) {
-      if (FAST) load_fast(ctx, s * TL::BK, r);
-      else load_generic(p, m0, n0, s * TL::BK, ptid, r);
-    };
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-      if (d < ktiles) issue(d, ring[d]);
-    int s = 0;
-    for (; s + 2 * D <= ktiles; s += D) {
-#pragma unroll
-      for (int d = 0; d < D; ++d) {
-        if (FAST) {
-          restage<true>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], (s + d + D) * TL::BK);
-        } else {
-          restage<false>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], 0);
-          issue(s + d + D, ring[d]);
-        }
-        __syncthreads();
-      }
-    }
-#pragma unroll
-    for (int dd = 0; dd < 2 * D; ++dd) {
-      const int d = dd % D;
-      if (s + dd < ktiles) {
-        if (FAST && s + dd + D < ktiles) {
-          restage<true>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], (s + dd + D) * TL::BK);
-        } else {
-          restage<false>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], 0);
-          if (s + dd + D < ktiles) issue(s + dd + D, ring[d]);
-        }
-        __syncthreads();
-      }
-    }
-    __syncthreads();
-    if (TL::WK > 1) __syncthreads();
   }
 
   // ---- consumer waves: LDS -> MFMA, then the epilogue --------------------------------------
@@ -607,8 +620,14 @@ struct TileGemm {
     const int m0 = tm * TL::BM, n0 = tn * TL::BN;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ktiles = (p.K + TL::BK - 1) / TL::BK;
-    if (wave >= TL::NCW) producer<FAST>(p, lds, m0, n0, ktiles);
-    else consumer(p, lds, m0, n0, ktiles, wave);
+    if (wave < TL::NCW) {
+      consumer(p, lds, m0, n0, ktiles, wave);
+    } else if constexpr (TL::NP < 8 || TL::BNQ == 0) {
+      Prod<kAll>::template loop<FAST>(p, lds, m0, n0, ktiles);
+    } else {
+      if (wave < TL::NCW + TL::NP / 2) Prod<kQuads>::template loop<FAST>(p, lds, m0, n0, ktiles);
+      else Prod<kRest>::template loop<FAST>(p, lds, m0, n0, ktiles);
+    }
   }
 };
 

@@ -2,7 +2,7 @@
 #pragma once
 #include <mutex>
 
-#include "cascmm_tile_kernel.h"
+#include "cascmm_bdirect_kernel.h"
 
 namespace cascmm {
 
@@ -40,6 +40,36 @@ int launch_tile(const GemmParams& p, hipStream_t stream) {
   {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH>::NT,       \
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, TERMS>::kBytes, FAST,                               \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, IODT, FMT, TERMS, FULL, FAST>}
+
+// same with the number of producer waves given explicitly
+#define CASCMM_TILE_VARIANT_P(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)    \
+  {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>::NT,   \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, TERMS>::kBytes, FAST,                           \
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, IODT, FMT, TERMS, FULL, FAST>}
+
+template <class TL, int FMT, int TERMS, bool FULL>
+int launch_bdirect(const GemmParams& p, hipStream_t stream) {
+  auto kfn = cascmm_bdirect_kernel<TL, FMT, TERMS, FULL>;
+  constexpr int lds = LdsLayoutA<TL, TERMS>::kBytes;
+  static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
+  if (lds > 64 * 1024) {
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+      attr_err = hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    });
+    if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
+  }
+  const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n;
+  hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
+  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+}
+
+// B-direct kernels: fp32 operands, fast path only
+#define CASCMM_BD_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                                \
+  {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, 32 * WN, BK, TileBD<BM, WN, BK, DEPTH, NP>::NT, \
+   LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true,                                      \
+   &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL>}
 
 // each instantiation unit exports its slice of the table
 const VariantDesc* variants_bf16(int* n);
