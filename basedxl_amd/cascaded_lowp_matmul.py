@@ -71,6 +71,62 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
     _lib.check(st, "cascmm_gemm")
 
 
+def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp: str = "bf16", terms: int = 2,
+                                 products: str = "tri", variant: int = -1):
+    """Several independent cascade GEMMs of one shape in ONE kernel launch.
+
+    ``a_list[i]`` ([..., K], the same tensor may appear several times) times ``b_list[i]``
+    ([K, N], contiguous) -> ``outs[i]``.  This is what the reference gets for to_k / to_v by
+    concatenating the two weights into one Linear (basedxl/modules/attn.py:23-39); here the
+    weights stay separate and up to 8 problems share one persistent launch, which removes
+    the launch gap and the cold start of every GEMM after the first.
+    """
+    import ctypes
+
+    n = len(a_list)
+    if n == 0 or n != len(b_list) or n > 8:
+        raise ValueError("need 1..8 problems, one b per a")
+    if lowp not in _lib.FMT_BY_NAME or products not in _lib.PROD_BY_NAME:
+        raise ValueError("bad lowp / products")
+    fmt, prod = _lib.FMT_BY_NAME[lowp], _lib.PROD_BY_NAME[products]
+    K, N = b_list[0].shape[-2], b_list[0].shape[-1]
+    a2s, res = [], []
+    for i, (a, b) in enumerate(zip(a_list, b_list)):
+        assert a.shape[-1] == b.shape[-2], "Incompatible dimensions"
+        assert b.is_contiguous(), "Matrix B must be contiguous"
+        _check_device_tensor(a, "a")
+        _check_device_tensor(b, "b")
+        if b.dim() != 2 or tuple(b.shape) != (K, N) or a.dtype != a_list[0].dtype or b.dtype != a.dtype:
+            raise ValueError("grouped problems must share one shape and dtype")
+        a2s.append(_rows(a.reshape(-1, K)))
+    M = a2s[0].shape[0]
+    lda = a2s[0].stride(0) if M > 1 else max(K, 1)
+    for a2 in a2s:
+        if a2.shape[0] != M or (M > 1 and a2.stride(0) != lda):
+            raise ValueError("grouped problems must share M and the row stride of a")
+    if a_list[0].dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {a_list[0].dtype}")
+    dev = a_list[0].device
+    if outs is None:
+        outs = [torch.empty((M, N), device=dev, dtype=a_list[0].dtype) for _ in range(n)]
+    for o in outs:
+        _check_device_tensor(o, "out")
+        if o.numel() != M * N or not o.is_contiguous() or o.dtype != a_list[0].dtype:
+            raise ValueError("every out must be a contiguous [M, N] tensor of the dtype of a")
+    if biases is not None:
+        biases = [None if bb is None else bb.contiguous() for bb in biases]
+    arr = ctypes.c_void_p * n
+    pa = arr(*[t.data_ptr() for t in a2s])
+    pb = arr(*[t.data_ptr() for t in b_list])
+    pc = arr(*[t.data_ptr() for t in outs])
+    pbias = arr(*[(None if bb is None else bb.data_ptr()) for bb in biases]) if biases is not None else None
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    st = _lib.lib().cascmm_gemm_grouped(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), max(N, 1),
+                                        _DTYPES[a_list[0].dtype], fmt, terms, prod, None, None, 0, stream, variant)
+    _lib.check(st, "cascmm_gemm_grouped")
+    return [o.reshape(*a.shape[:-1], N) for o, a in zip(outs, a_list)]
+
+
 def _rows(t: torch.Tensor) -> torch.Tensor:
     """2-D view whose rows are contiguous (row stride free); copies only when it must."""
     if t.stride(-1) != 1 and t.shape[-1] > 1:

@@ -56,25 +56,33 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   return true;
 }
 
-// Cost model: time ~ rounds over the 256 CUs x per-tile time, where a tile costs its MFMA
-// work (BM*BN) plus a staging term proportional to the operand rows it has to load, split
-// and write to LDS per k (BM+BN).  Constants fitted on MI355X measurements.
-static double variant_cost(const VariantDesc& v, const Problem& q) {
-  const double tiles = (double)((q.M + v.BM - 1) / v.BM) * (double)((q.N + v.BN - 1) / v.BN);
-  const double slots = 256.0;
-  const double rounds = (double)(int64_t)((tiles + slots - 1) / slots);
-  const double per_tile = (double)v.BM * v.BN + 64.0 * (v.BM + v.BN);
-  return rounds * per_tile + (v.fast ? 0.0 : 1e-3);
+// Cost model, fitted on MI355X sweeps.  A 64-deep K step of a full round of 256 tiles costs
+// about (BM*BN + 64*(BM+BN)) / 20000 microseconds: MFMA work grows with BM*BN, while loading,
+// splitting and staging the operands grows with BM+BN and weighs about as much at these tile
+// sizes.  A round that fills only part of the CUs runs its steps faster (less contention for
+// the caches), hence the discount.  Eight producer waves are ~6 % faster than four, the
+// B-direct kernels ~15 % slower.
+static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
+  const double tiles = (double)count * (double)((q.M + v.BM - 1) / v.BM) * (double)((q.N + v.BN - 1) / v.BN);
+  const double full = (double)(int64_t)(tiles / kNumCUs);
+  const double rem = tiles - full * kNumCUs;
+  const double rounds = full + (rem > 0 ? 0.55 + 0.45 * rem / kNumCUs : 0.0);
+  double step = ((double)v.BM * v.BN + 64.0 * (v.BM + v.BN)) / 20000.0;
+  const char* name = v.name;
+  if (strstr(name, "_p8_")) step *= 0.94;
+  if (name[0] == 'b' && name[1] == 'd') step *= 1.15;
+  const double ksteps = (double)((q.K + 63) / 64);
+  return rounds * step * ksteps + (v.fast ? 0.0 : 1e3);
 }
 
-static int select_variant(const Problem& q, const void* A, const void* B) {
-  const bool fast = fast_ok(q, A, B);
+static int select_variant(const Problem& q, bool fast, int count) {
   const auto& t = table();
   int best = -1;
   double best_cost = 0;
   for (int i = 0; i < (int)t.size(); ++i) {
     if (!variant_matches(t[i], q, fast)) continue;
-    const double c = variant_cost(t[i], q);
+    if (count > 1 && !t[i].grouped) continue;
+    const double c = variant_cost(t[i], q, count);
     if (best < 0 || c < best_cost) { best = i; best_cost = c; }
   }
   return best < 0 ? (int)CASCMM_ERR_BAD_FORMAT : best;
@@ -122,48 +130,62 @@ static int launch_split(const void* x, float* out, int64_t n, int terms, int ten
   return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
-static int gemm_impl(const void* A, const void* B, void* C, const void* bias, const Problem& q,
-                     const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
+// One launch for `count` problems of one shape (count == 1: a plain GEMM).
+static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
+                     const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
                      hipStream_t stream, int variant) {
+  (void)tensor_exps; (void)workspace; (void)workspace_bytes;
   int st = check_problem(q);
   if (st != CASCMM_OK) return st;
+  if (count < 1 || count > kMaxGroup) return CASCMM_ERR_BAD_SHAPE;
   if (q.M == 0 || q.N == 0) return CASCMM_OK;
-  if (!C) return CASCMM_ERR_NULL_POINTER;
   const size_t es = dtype_size(q.dtype);
-  if (!aligned_to(C, es) || !aligned_to(bias, es)) return CASCMM_ERR_ALIGNMENT;
+  for (int i = 0; i < count; ++i) {
+    if (!C[i]) return CASCMM_ERR_NULL_POINTER;
+    if (!aligned_to(C[i], es) || (bias && !aligned_to(bias[i], es))) return CASCMM_ERR_ALIGNMENT;
+  }
   if (q.K == 0) {
     const int64_t total = q.M * q.N;
     const unsigned grid = (unsigned)((total + 255) / 256);
-    if (q.dtype == CASCMM_DT_F32)
-      hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, stream, C, bias, (int)q.M, (int)q.N, q.ldc);
-    else if (q.dtype == CASCMM_DT_F16)
-      hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, stream, C, bias, (int)q.M, (int)q.N, q.ldc);
-    else
-      hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, stream, C, bias, (int)q.M, (int)q.N, q.ldc);
+    for (int i = 0; i < count; ++i) {
+      const void* b = bias ? bias[i] : nullptr;
+      if (q.dtype == CASCMM_DT_F32)
+        hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
+      else if (q.dtype == CASCMM_DT_F16)
+        hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
+      else
+        hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
+    }
     return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
   }
-  if (!A || !B) return CASCMM_ERR_NULL_POINTER;
-  if (!aligned_to(A, es) || !aligned_to(B, es)) return CASCMM_ERR_ALIGNMENT;
+  bool fast = true;
+  for (int i = 0; i < count; ++i) {
+    if (!A[i] || !B[i]) return CASCMM_ERR_NULL_POINTER;
+    if (!aligned_to(A[i], es) || !aligned_to(B[i], es)) return CASCMM_ERR_ALIGNMENT;
+    fast = fast && fast_ok(q, A[i], B[i]);
+  }
 
   const auto& t = table();
   if (variant < 0) {
-    variant = select_variant(q, A, B);
+    variant = select_variant(q, fast, count);
     if (variant < 0) return variant;
   } else {
     if (variant >= (int)t.size()) return CASCMM_ERR_BAD_VARIANT;
-    if (!variant_matches(t[variant], q, fast_ok(q, A, B))) return CASCMM_ERR_BAD_VARIANT;
+    if (!variant_matches(t[variant], q, fast)) return CASCMM_ERR_BAD_VARIANT;
   }
   const VariantDesc& v = t[variant];
-  GemmParams p;
+  if (count > 1 && !v.grouped) return CASCMM_ERR_BAD_VARIANT;
+  GroupParams p;
   memset(&p, 0, sizeof(p));
-  p.A = A; p.B = B; p.C = C; p.bias = bias;
   p.M = (int)q.M; p.N = (int)q.N; p.K = (int)q.K;
   p.lda = q.lda; p.ldb = q.ldb; p.ldc = q.ldc;
   const int64_t tm = (q.M + v.BM - 1) / v.BM, tn = (q.N + v.BN - 1) / v.BN;
-  if (tm * tn > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (tm * tn * count > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
-  p.tensor_exps = tensor_exps;
-  (void)workspace; (void)workspace_bytes;
+  p.count = count;
+  for (int i = 0; i < count; ++i) {
+    p.A[i] = A[i]; p.B[i] = B[i]; p.C[i] = C[i]; p.bias[i] = bias ? bias[i] : nullptr;
+  }
   return v.launch(p, stream);
 }
 
@@ -178,7 +200,17 @@ int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,
                         const int32_t* tensor_exps, void* workspace, size_t workspace_bytes, void* stream,
                         int variant) {
   const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
-  return gemm_impl(A, B, C, bias, q, tensor_exps, workspace, workspace_bytes, (hipStream_t)stream, variant);
+  return gemm_impl(1, &A, &B, &C, bias ? &bias : nullptr, q, tensor_exps, workspace, workspace_bytes, (hipStream_t)stream,
+                   variant);
+}
+
+int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
+                        int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt,
+                        int terms, int products, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
+                        void* stream, int variant) {
+  if (!A || !B || !C) return CASCMM_ERR_NULL_POINTER;
+  const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  return gemm_impl(count, A, B, C, bias, q, tensor_exps, workspace, workspace_bytes, (hipStream_t)stream, variant);
 }
 
 int cascmm_gemm(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -198,7 +230,7 @@ int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
   const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
   const int st = check_problem(q);
   if (st != CASCMM_OK) return st;
-  return select_variant(q, nullptr, nullptr);
+  return select_variant(q, fast_ok(q, nullptr, nullptr), 1);
 }
 
 int cascmm_variant_count(void) { return (int)table().size(); }

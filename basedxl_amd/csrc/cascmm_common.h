@@ -143,4 +143,18 @@ struct GemmParams {
   const int32_t* tensor_exps;
 };
 
+// A group of GEMMs of one shape launched as one kernel (count == 1 for a plain GEMM).  Work
+// item i = problem i / tiles, tile i % tiles; workgroup w runs items w, w + grid, w + 2 grid ...
+constexpr int kMaxGroup = 8;
+struct GroupParams {
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  int tiles_m, tiles_n;
+  int count;
+  const void* A[kMaxGroup];
+  const void* B[kMaxGroup];
+  void* C[kMaxGroup];
+  const void* bias[kMaxGroup];
+};
+
 }  // namespace cascmm

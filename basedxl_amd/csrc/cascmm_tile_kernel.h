@@ -31,6 +31,11 @@
 // indexed by compile-time constants), the LDS stage is double buffered, and there is one
 // barrier per K step.
 //
+// The kernel is persistent and grouped: a launch covers `count` GEMMs of one shape, the grid
+// is at most one workgroup per CU, and a workgroup walks its work items (tiles) in turn.  The
+// producers' prefetch ring runs across item boundaries, so the load latency of a tile's first
+// operands is hidden behind the previous tile's last steps and result stores.
+//
 // The workgroup is specialised.  WM x WN x WK "consumer" waves only read fragments from LDS
 // and issue MFMAs; NP "producer" waves only load, split and write LDS.  With one wave of each
 // kind per SIMD, the producer's VALU work issues in the gaps the consumer's MFMAs leave on
@@ -145,12 +150,14 @@ struct TileGemm {
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
 
   // ---- producer waves: global -> split -> LDS, one stage per barrier interval -----------------
-  // Barrier protocol (both kinds of wave execute exactly ktiles + 1 barriers, plus one more
-  // for the WK reduction):
-  //   producer:  store(0) B0 store(1) B1 ... store(kt-1) B(kt-1)            B(kt)
-  //   consumer:           B0 compute(0) B1 ... compute(kt-2) B(kt-1) compute(kt-1) B(kt)
-  // store(s) writes LDS buffer s&1 between B(s-1) and B(s); the last reader of that buffer,
-  // compute(s-2), finished before B(s-1), and its first reader, compute(s), starts after B(s).
+  // Barrier protocol over the global step sequence g of a workgroup (every wave executes the
+  // same number of barriers):
+  //   producer:  store(0) B0 store(1) B1 store(2) B2 ...
+  //   consumer:           B0 compute(0) B1 compute(1) B2 ...
+  // store(g) writes LDS buffer g&1 between B(g-1) and B(g); the last reader of that buffer,
+  // compute(g-2), finished before B(g-1), and its first reader, compute(g), starts after B(g).
+  // At the end of an item with WK == 2 both sides add three barriers around the reduction of
+  // the two K halves, which reuses the stage buffers.
   //
   // ROLE says which staging units a producer wave handles: every kind (kAll), or, when the
   // workgroup has eight producer waves, the 8x4 blocks of B for the first four (kQuads) and A
@@ -184,9 +191,33 @@ struct TileGemm {
       int ldb_bytes;
     };
 
-    static __device__ __forceinline__ void init_ctx(Ctx& c, const GemmParams& p, int m0, int n0, int rtid) {
-      const IoT* A = (const IoT*)p.A + (int64_t)m0 * p.lda;
-      const IoT* B = (const IoT*)p.B + n0;
+    // LDS slot of every unit this thread stages (fixed for the whole kernel)
+    static __device__ __forceinline__ void init_lds(Ctx& c, int rtid) {
+#pragma unroll
+      for (int it = 0; it < A_IT; ++it) {
+        const int u = rtid + it * NTR;
+        const int kg = u % TL::KG, r = u / TL::KG;
+        c.lds_a[it] = u < A_UNITS ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
+      }
+#pragma unroll
+      for (int it = 0; it < Q_IT; ++it) {
+        const int u = rtid + it * NTR;
+        const int quad = u % QW, kg = u / QW;
+        c.lds_q[it] = u < Q_UNITS ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) : -1;
+      }
+#pragma unroll
+      for (int it = 0; it < B_IT; ++it) {
+        const int u = rtid + it * NTR;
+        const int n = TL::BNQ + u % SW, kg = u / SW;
+        c.lds_b[it] = u < B_UNITS ? kg * LL::kBPlane + n : -1;
+      }
+    }
+
+    // point the loads at tile (m0, n0) of problem `prob`: buffer descriptors at the tile origin
+    // and per-lane offsets with rows / columns clamped to the last valid one
+    static __device__ __forceinline__ void set_tile(Ctx& c, const GroupParams& p, int prob, int m0, int n0, int rtid) {
+      const IoT* A = (const IoT*)p.A[prob] + (int64_t)m0 * p.lda;
+      const IoT* B = (const IoT*)p.B[prob] + n0;
       // bytes from the tile origin to the end of the matrix; rows and columns are also clamped
       // below, so no access relies on the hardware range check
       c.ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
@@ -196,33 +227,27 @@ struct TileGemm {
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
         int u = rtid + it * NTR;
-        const bool mine = u < A_UNITS;
-        u = mine ? u : A_UNITS - 1;
+        u = u < A_UNITS ? u : A_UNITS - 1;
         const int kg = u % TL::KG, r = u / TL::KG;
         const int rc = r < last_row ? r : last_row;
         c.voff_a[it] = (int)((rc * p.lda + kg * 8) * ES);
-        c.lds_a[it] = mine ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
       }
 #pragma unroll
       for (int it = 0; it < Q_IT; ++it) {
         int u = rtid + it * NTR;
-        const bool mine = u < Q_UNITS;
-        u = mine ? u : Q_UNITS - 1;
+        u = u < Q_UNITS ? u : Q_UNITS - 1;
         const int quad = u % QW, kg = u / QW;
         const int last_quad = last_col >> 2;  // fast path: N % 4 == 0, a quad is wholly in or out
         const int qc = quad < last_quad ? quad : last_quad;
         c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc) * ES);
-        c.lds_q[it] = mine ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) : -1;
       }
 #pragma unroll
       for (int it = 0; it < B_IT; ++it) {
         int u = rtid + it * NTR;
-        const bool mine = u < B_UNITS;
-        u = mine ? u : B_UNITS - 1;
+        u = u < B_UNITS ? u : B_UNITS - 1;
         const int n = TL::BNQ + u % SW, kg = u / SW;
         const int nc = n < last_col ? n : last_col;
         c.voff_b[it] = (int)((kg * 8 * p.ldb + nc) * ES);
-        c.lds_b[it] = mine ? kg * LL::kBPlane + n : -1;
       }
     }
 
@@ -254,9 +279,9 @@ struct TileGemm {
     }
 
     // global -> registers (generic: any dtype, any K, element-wise, bounds-checked)
-    static __device__ __forceinline__ void load_generic(const GemmParams& p, int m0, int n0, int k0, int rtid, Regs& r) {
-      const IoT* A = (const IoT*)p.A;
-      const IoT* B = (const IoT*)p.B;
+    static __device__ __forceinline__ void load_generic(const GroupParams& p, int prob, int m0, int n0, int k0, int rtid, Regs& r) {
+      const IoT* A = (const IoT*)p.A[prob];
+      const IoT* B = (const IoT*)p.B[prob];
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
         int u = rtid + it * NTR;
@@ -364,48 +389,81 @@ struct TileGemm {
       }
     }
 
+    // The producer walks the global step sequence gs = 0 .. items * ktiles - 1 of this
+    // workgroup (item j = work item blockIdx.x + j * gridDim.x, step gs % ktiles of it).  The
+    // prefetch ring runs across item boundaries, so the first operands of the next tile are
+    // already in registers while the consumers finish the current one and store its result.
     template <bool FAST>
-    static __device__ __forceinline__ void loop(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles) {
+    static __device__ __forceinline__ void loop(const GroupParams& p, u32x4* lds, int ktiles, int nitems) {
       const int rtid = threadIdx.x - TL::NCW * kWave - T0;
+      const int tiles = p.tiles_m * p.tiles_n;
+      const int gsteps = nitems * ktiles;
       Ctx ctx;
-      init_ctx(ctx, p, m0, n0, rtid);
+      init_lds(ctx, rtid);
       Regs ring[D];
-      // loads are only ever issued for k steps that exist (s < ktiles)
-      auto issue = [&](int s, Regs& r) {
-        if (FAST) load_fast(ctx, s * TL::BK, r);
-        else load_generic(p, m0, n0, s * TL::BK, rtid, r);
+      // loads for global step g (only ever called with g < gsteps): retarget on a new item
+      int cur_item = -1, prob = 0, m0 = 0, n0 = 0;
+      auto target = [&](int g) {
+        const int j = g / ktiles;
+        if (j != cur_item) {
+          cur_item = j;
+          const int item = blockIdx.x + j * gridDim.x;
+          prob = item / tiles;
+          int tm, tn;
+          tile_coords(item - prob * tiles, p.tiles_m, p.tiles_n, tm, tn);
+          m0 = tm * TL::BM;
+          n0 = tn * TL::BN;
+          set_tile(ctx, p, prob, m0, n0, rtid);
+        }
+        return (g - j * ktiles) * TL::BK;
+      };
+      auto issue = [&](int g, Regs& r) {
+        const int k0 = target(g);
+        if (FAST) load_fast(ctx, k0, r);
+        else load_generic(p, prob, m0, n0, k0, rtid, r);
+      };
+      // after the last step of an item the consumers reduce their K halves through LDS (WK == 2):
+      // three barriers during which nothing may be staged
+      auto item_end = [&](int g) {
+        if (TL::WK > 1 && (g + 1) % ktiles == 0) {
+          __syncthreads();
+          __syncthreads();
+          __syncthreads();
+        }
       };
 #pragma unroll
       for (int d = 0; d < D; ++d)
-        if (d < ktiles) issue(d, ring[d]);
-      int s = 0;
-      for (; s + 2 * D <= ktiles; s += D) {
+        if (d < gsteps) issue(d, ring[d]);
+      int g = 0;
+      for (; g + 2 * D <= gsteps; g += D) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
           if (FAST) {
-            restage<true>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], (s + d + D) * TL::BK);
+            const int k_next = target(g + d + D);
+            restage<true>(ctx, lds + ((g + d) & 1) * LL::kStage, ring[d], k_next);
           } else {
-            restage<false>(ctx, lds + ((s + d) & 1) * LL::kStage, ring[d], 0);
-            issue(s + d + D, ring[d]);
+            restage<false>(ctx, lds + ((g + d) & 1) * LL::kStage, ring[d], 0);
+            issue(g + d + D, ring[d]);
           }
           __syncthreads();
+          item_end(g + d);
         }
       }
 #pragma unroll
       for (int dd = 0; dd < 2 * D; ++dd) {
         const int d = dd % D;
-        if (s + dd < ktiles) {
-          if (FAST && s + dd + D < ktiles) {
-            restage<true>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], (s + dd + D) * TL::BK);
+        if (g + dd < gsteps) {
+          if (FAST && g + dd + D < gsteps) {
+            const int k_next = target(g + dd + D);
+            restage<true>(ctx, lds + ((g + dd) & 1) * LL::kStage, ring[d], k_next);
           } else {
-            restage<false>(ctx, lds + ((s + dd) & 1) * LL::kStage, ring[d], 0);
-            if (s + dd + D < ktiles) issue(s + dd + D, ring[d]);
+            restage<false>(ctx, lds + ((g + dd) & 1) * LL::kStage, ring[d], 0);
+            if (g + dd + D < gsteps) issue(g + dd + D, ring[d]);
           }
           __syncthreads();
+          item_end(g + dd);
         }
       }
-      __syncthreads();
-      if (TL::WK > 1) __syncthreads();
     }
   };
 
@@ -445,59 +503,72 @@ struct TileGemm {
     }
   }
 
-  // ---- consumer waves: LDS -> MFMA, then the epilogue --------------------------------------
-  static __device__ __forceinline__ void consumer(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles, int wave) {
+  // ---- consumer waves: LDS -> MFMA, then the epilogue, item after item --------------------------
+  static __device__ __forceinline__ void consumer(const GroupParams& p, u32x4* lds, int ktiles, int nitems, int wave) {
     const int wk = wave / (TL::WM * TL::WN);
     const int wmn = wave - wk * (TL::WM * TL::WN);
     const int wm0 = (wmn / TL::WN) * TL::WTM, wn0 = (wmn % TL::WN) * TL::WTN;
-
-    f32x16 acc[NCLS][TL::MT][TL::NTL];
-#pragma unroll
-    for (int c = 0; c < NCLS; ++c)
-#pragma unroll
-      for (int mi = 0; mi < TL::MT; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < TL::NTL; ++ni)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) acc[c][mi][ni][e] = 0.f;
-
-    // Blocked accumulation for the cascades whose error sits at the fp32 rounding floor: the
-    // big class-0 sum is collected in chunks of kChunkK and the chunks are added into a master
-    // accumulator, so the chunk sums round at a fraction of the final magnitude and the master
-    // rounds K / kChunkK times instead of K / 16 times.
-    f32x16 master[AC::kChunked ? TL::MT : 1][AC::kChunked ? TL::NTL : 1];
-    if constexpr (AC::kChunked) {
-#pragma unroll
-      for (int mi = 0; mi < TL::MT; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < TL::NTL; ++ni)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) master[mi][ni][e] = 0.f;
-    }
+    const int tiles = p.tiles_m * p.tiles_n;
     constexpr int kChunkSteps = (AC::kChunkK / TL::BK) > 0 ? (AC::kChunkK / TL::BK) : 1;
+    int g = 0;
+    for (int j = 0; j < nitems; ++j) {
+      const int item = blockIdx.x + j * gridDim.x;
+      const int prob = item / tiles;
+      int tm, tn;
+      tile_coords(item - prob * tiles, p.tiles_m, p.tiles_n, tm, tn);
+      const int m0 = tm * TL::BM, n0 = tn * TL::BN;
 
-    __syncthreads();
-    for (int kt = 0; kt < ktiles; ++kt) {
-      compute(lds + (kt & 1) * LL::kStage, wm0, wn0, wk, acc);
-      if constexpr (AC::kChunked) if ((kt % kChunkSteps) == kChunkSteps - 1) {
+      f32x16 acc[NCLS][TL::MT][TL::NTL];
+#pragma unroll
+      for (int c = 0; c < NCLS; ++c)
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi)
 #pragma unroll
-          for (int ni = 0; ni < TL::NTL; ++ni) {
-            master[mi][ni] += acc[0][mi][ni];
+          for (int ni = 0; ni < TL::NTL; ++ni)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[0][mi][ni][e] = 0.f;
-          }
-      }
-      __syncthreads();
-    }
-    if constexpr (AC::kChunked) {
-#pragma unroll
-      for (int mi = 0; mi < TL::MT; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < TL::NTL; ++ni) acc[0][mi][ni] += master[mi][ni];
-    }
+            for (int e = 0; e < 16; ++e) acc[c][mi][ni][e] = 0.f;
 
+      // Blocked accumulation for the cascades whose error sits at the fp32 rounding floor: the
+      // big class-0 sum is collected in chunks of kChunkK and the chunks are added into a master
+      // accumulator, so the chunk sums round at a fraction of the final magnitude and the master
+      // rounds K / kChunkK times instead of K / 16 times.
+      f32x16 master[AC::kChunked ? TL::MT : 1][AC::kChunked ? TL::NTL : 1];
+      if constexpr (AC::kChunked) {
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < TL::NTL; ++ni)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) master[mi][ni][e] = 0.f;
+      }
+
+      for (int kt = 0; kt < ktiles; ++kt, ++g) {
+        __syncthreads();
+        compute(lds + (g & 1) * LL::kStage, wm0, wn0, wk, acc);
+        if constexpr (AC::kChunked) if ((kt % kChunkSteps) == kChunkSteps - 1) {
+#pragma unroll
+          for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < TL::NTL; ++ni) {
+              master[mi][ni] += acc[0][mi][ni];
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[0][mi][ni][e] = 0.f;
+            }
+        }
+      }
+      if constexpr (AC::kChunked) {
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < TL::NTL; ++ni) acc[0][mi][ni] += master[mi][ni];
+      }
+      finish(p, lds, prob, m0, n0, wk, wmn, wm0, wn0, acc);
+    }
+  }
+
+  // ---- end of an item: fold, reduce the K halves, store -----------------------------------------
+  static __device__ __forceinline__ void finish(const GroupParams& p, u32x4* lds, int prob, int m0, int n0, int wk, int wmn,
+                                                int wm0, int wn0, f32x16 (&acc)[NCLS][TL::MT][TL::NTL]) {
     // fold the scale classes (smallest first), then the cross-wave-group reduction (WK == 2):
     // group 1 parks its tile in LDS, group 0 adds it
     f32x16 res[TL::MT][TL::NTL];
@@ -512,7 +583,11 @@ struct TileGemm {
       }
     const int lane = threadIdx.x & 63, l31 = lane & 31, g = lane >> 5;
     if (TL::WK > 1) {
+      // the reduction buffer overlays the stage buffers: barrier 1 = every consumer is done
+      // reading them, barrier 2 = the parked tiles are visible, barrier 3 = they have been read
+      // (the producers, which execute the same three barriers, may stage again)
       f32x4* red = (f32x4*)lds + wmn * (TL::MT * TL::NTL * 4 * 64) + lane;
+      __syncthreads();
       if (wk == 1) {
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi)
@@ -524,22 +599,25 @@ struct TileGemm {
                   (f32x4){res[mi][ni][4 * q], res[mi][ni][4 * q + 1], res[mi][ni][4 * q + 2], res[mi][ni][4 * q + 3]};
       }
       __syncthreads();
+      if (wk == 0) {
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int ni = 0; ni < TL::NTL; ++ni)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const f32x4 o = red[((mi * TL::NTL + ni) * 4 + q) * 64];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) res[mi][ni][4 * q + e] += o[e];
+            }
+      }
+      __syncthreads();
       if (wk == 1) return;
-#pragma unroll
-      for (int mi = 0; mi < TL::MT; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < TL::NTL; ++ni)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f32x4 o = red[((mi * TL::NTL + ni) * 4 + q) * 64];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) res[mi][ni][4 * q + e] += o[e];
-          }
     }
 
     // epilogue: of every 32x32 tile a lane holds column lane%32 and rows 8*q + 4*(lane/32) + e
-    IoT* C = (IoT*)p.C;
-    const IoT* bias = (const IoT*)p.bias;
+    IoT* C = (IoT*)p.C[prob];
+    const IoT* bias = (const IoT*)p.bias[prob];
     const bool interior = (m0 + TL::BM <= p.M) && (n0 + TL::BN <= p.N) && p.ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
     // Column blocks of this wave that hold permuted columns come in runs of RUN blocks of one
     // 128-column group: block b of the tile (b = wn0/32 + ni), lane l31 <-> column
@@ -614,25 +692,24 @@ struct TileGemm {
   }
 
   template <bool FAST>
-  static __device__ __forceinline__ void run(const GemmParams& p, u32x4* lds) {
-    int tm, tn;
-    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-    const int m0 = tm * TL::BM, n0 = tn * TL::BN;
+  static __device__ __forceinline__ void run(const GroupParams& p, u32x4* lds) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ktiles = (p.K + TL::BK - 1) / TL::BK;
+    const int total = p.count * p.tiles_m * p.tiles_n;
+    const int nitems = (total - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;  // grid <= total
     if (wave < TL::NCW) {
-      consumer(p, lds, m0, n0, ktiles, wave);
+      consumer(p, lds, ktiles, nitems, wave);
     } else if constexpr (TL::NP < 8 || TL::BNQ == 0) {
-      Prod<kAll>::template loop<FAST>(p, lds, m0, n0, ktiles);
+      Prod<kAll>::template loop<FAST>(p, lds, ktiles, nitems);
     } else {
-      if (wave < TL::NCW + TL::NP / 2) Prod<kQuads>::template loop<FAST>(p, lds, m0, n0, ktiles);
-      else Prod<kRest>::template loop<FAST>(p, lds, m0, n0, ktiles);
+      if (wave < TL::NCW + TL::NP / 2) Prod<kQuads>::template loop<FAST>(p, lds, ktiles, nitems);
+      else Prod<kRest>::template loop<FAST>(p, lds, ktiles, nitems);
     }
   }
 };
 
 template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
-__global__ __launch_bounds__(TL::NT) void cascmm_tile_kernel(const GemmParams p) {
+__global__ __launch_bounds__(TL::NT) void cascmm_tile_kernel(const GroupParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char cascmm_smem[];
   TileGemm<TL, IODT, FMT, TERMS, FULL>::template run<FAST>(p, (u32x4*)cascmm_smem);
 }

@@ -1,5 +1,6 @@
 // Host-side table of compiled kernel variants and the launcher template that fills it.
 #pragma once
+#include <cstring>
 #include <mutex>
 
 #include "cascmm_bdirect_kernel.h"
@@ -7,6 +8,7 @@
 namespace cascmm {
 
 enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1 };
+constexpr int kNumCUs = 256;  // MI355X
 
 struct VariantDesc {
   const char* name;
@@ -15,11 +17,12 @@ struct VariantDesc {
   int BM, BN, BK, threads;
   int lds_bytes;
   bool fast;  // needs fp32 operands, K % BK == 0, 16-byte aligned A rows
-  int (*launch)(const GemmParams&, hipStream_t);
+  bool grouped;  // one launch may run several same-shape problems and several tiles per workgroup
+  int (*launch)(const GroupParams&, hipStream_t);
 };
 
 template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
-int launch_tile(const GemmParams& p, hipStream_t stream) {
+int launch_tile(const GroupParams& p, hipStream_t stream) {
   auto kfn = cascmm_tile_kernel<TL, IODT, FMT, TERMS, FULL, FAST>;
   constexpr int lds = LdsLayout<TL, TERMS>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
@@ -31,24 +34,39 @@ int launch_tile(const GemmParams& p, hipStream_t stream) {
     });
     if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
   }
-  const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n;
+  // persistent grid: at most as many workgroups as can be resident at once
+  static std::once_flag occ_once;
+  static int per_cu = 1;
+  std::call_once(occ_once, [&] {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kfn, TL::NT, lds) == hipSuccess && n > 0) per_cu = n;
+  });
+  const int64_t total = (int64_t)p.count * p.tiles_m * p.tiles_n;
+  const int64_t resident = (int64_t)kNumCUs * per_cu;
+  const unsigned grid = (unsigned)(total < resident ? total : resident);
   hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
   return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
 #define CASCMM_TILE_VARIANT(NAME, BM, BN, BK, WM, WN, WK, DEPTH, IODT, FMT, TERMS, FULL, FAST)         \
   {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH>::NT,       \
-   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, TERMS>::kBytes, FAST,                               \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, TERMS>::kBytes, FAST, true,                         \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, IODT, FMT, TERMS, FULL, FAST>}
 
 // same with the number of producer waves given explicitly
 #define CASCMM_TILE_VARIANT_P(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)    \
   {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>::NT,   \
-   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, TERMS>::kBytes, FAST,                           \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, TERMS>::kBytes, FAST, true,                     \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, IODT, FMT, TERMS, FULL, FAST>}
 
 template <class TL, int FMT, int TERMS, bool FULL>
-int launch_bdirect(const GemmParams& p, hipStream_t stream) {
+int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
+  if (gp.count != 1) return CASCMM_ERR_BAD_VARIANT;
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  p.A = gp.A[0]; p.B = gp.B[0]; p.C = gp.C[0]; p.bias = gp.bias[0];
+  p.M = gp.M; p.N = gp.N; p.K = gp.K; p.lda = gp.lda; p.ldb = gp.ldb; p.ldc = gp.ldc;
+  p.tiles_m = gp.tiles_m; p.tiles_n = gp.tiles_n;
   auto kfn = cascmm_bdirect_kernel<TL, FMT, TERMS, FULL>;
   constexpr int lds = LdsLayoutA<TL, TERMS>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
@@ -68,7 +86,7 @@ int launch_bdirect(const GemmParams& p, hipStream_t stream) {
 // B-direct kernels: fp32 operands, fast path only
 #define CASCMM_BD_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                                \
   {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, 32 * WN, BK, TileBD<BM, WN, BK, DEPTH, NP>::NT, \
-   LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true,                                      \
+   LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true, false,                               \
    &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL>}
 
 // each instantiation unit exports its slice of the table

@@ -83,6 +83,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
+    ap.add_argument("--group", choices=["qkv+o", "all", "none"], default="qkv+o",
+                    help="how the four GEMMs of a step are launched: to_q/to_k/to_v (same input) as one grouped launch "
+                         "plus to_out on its own (default), all four in one grouped launch, or four separate launches")
+    ap.add_argument("--streams", type=int, default=1,
+                    help="number of HIP streams the four independent GEMMs of a step are spread over")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -92,7 +97,7 @@ def main():
                  "exchange, so N GPUs run N independent copies of this step")
 
     import torch
-    from basedxl_amd import cascaded_lowp_matmul, _lib
+    from basedxl_amd import cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, _lib
     from oracle import cascade as oc
 
     if not torch.cuda.is_available():
@@ -101,11 +106,29 @@ def main():
     cpu_in, (x, y, ws) = make_inputs(dev)
     outs = [torch.empty(M, N, device=dev, dtype=torch.float32) for _ in range(N_PROJ)]
 
+    ins = [x, x, x, y]
+    extra = [torch.cuda.Stream() for _ in range(max(0, min(args.streams, N_PROJ) - 1))]
+
     def step():
-        cascaded_lowp_matmul(x, ws[0], out=outs[0])
-        cascaded_lowp_matmul(x, ws[1], out=outs[1])
-        cascaded_lowp_matmul(x, ws[2], out=outs[2])
-        cascaded_lowp_matmul(y, ws[3], out=outs[3])
+        # the four projections are independent GEMMs; with --streams > 1 they are enqueued on
+        # several streams (forked from and joined back into the current one) so that the tail
+        # of one kernel overlaps the start of the next
+        if args.group == "qkv+o":
+            cascaded_lowp_matmul_grouped(ins[:3], ws[:3], outs=outs[:3])
+            cascaded_lowp_matmul(ins[3], ws[3], out=outs[3])
+            return
+        if args.group == "all":
+            cascaded_lowp_matmul_grouped(ins, ws, outs=outs)
+            return
+        cur = torch.cuda.current_stream()
+        lanes = [cur] + extra
+        for s_ in extra:
+            s_.wait_stream(cur)
+        for i in range(N_PROJ):
+            with torch.cuda.stream(lanes[i % len(lanes)]):
+                cascaded_lowp_matmul(ins[i], ws[i], out=outs[i])
+        for s_ in extra:
+            cur.wait_stream(s_)
 
     # correctness of what is being timed: error vs fp64 next to the oracle cascade's error
     step()
@@ -152,7 +175,9 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     flops_step = N_PROJ * 2.0 * M * N * K
     value = flops_step / (wall / args.steps) * 1e-12
-    # the GEMM kernel: 4 identical launches per step; average launch duration from the events
+    # the GEMM kernel: every launch of a step runs the same kernel on 1, 3 or 4 of the GEMMs;
+    # per-launch figures are quoted per GEMM (launch duration / GEMMs in it), from the events
+    launches_per_step = {"qkv+o": 2, "all": 1, "none": N_PROJ}[args.group]
     launch_us = ev_ms * 1e3 / (args.steps * N_PROJ)
     mfma_tflops = PRODUCTS_PER_ELEMENT * 2.0 * M * N * K / (launch_us * 1e-6) * 1e-12
     l = _lib.lib()
@@ -175,7 +200,10 @@ def main():
             "workload": "cfg2: X fp32 [4096,640] ~N(0,1) x W fp32 [640,640] ~N(0,0.02), q/k/v/out = 4 GEMMs per step, "
                         "hi=bf16(x), lo=bf16(x-hi), products hi.hi+hi.lo+lo.hi, fp32 accumulate, fp32 out",
             "M": M, "N": N, "K": K, "gemms_per_step": N_PROJ, "terms": TERMS, "products": "tri",
-            "launch": "hip graph replay" if graph is not None else "python ctypes",
+            "launch": ("hip graph replay" if graph is not None else "python ctypes") + f", {len(extra) + 1} stream(s), "
+                      + {"qkv+o": "2 launches per step: to_q/to_k/to_v grouped (3 GEMMs, one activation tensor) + to_out",
+                         "all": "1 grouped launch per step (4 GEMMs)", "none": "4 launches per step"}[args.group],
+            "launches_per_step": launches_per_step,
             "kernel": vname, "seed": SEED,
             "cache_regime": "same buffers every step (70 MB working set, resident in the 256 MB Infinity Cache)",
         },
@@ -187,6 +215,7 @@ def main():
             "frac": round(mfma_tflops / PEAK_BF16_TFLOPS, 4),
             "traffic": None,
             "launch_us": round(launch_us, 3),
+            "launch_us_is": "event time of the timed region / GEMMs executed (a grouped launch runs several GEMMs)",
             "flops_per_launch": PRODUCTS_PER_ELEMENT * 2 * M * N * K,
             "fp32_equiv_tflops_per_launch": round(2.0 * M * N * K / (launch_us * 1e-6) * 1e-12, 2),
             "frac_of_peak_over_terms": round(2.0 * M * N * K / (launch_us * 1e-6) * 1e-12 / (PEAK_BF16_TFLOPS / TERMS), 4),

@@ -85,6 +85,21 @@ int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,
                         const int32_t* tensor_exps,
                         void* workspace, size_t workspace_bytes, void* stream, int variant);
 
+/* `count` (1..8) independent GEMMs of one shape, layout and cascade in ONE launch: problem i
+ * computes C[i] = A[i] . B[i] (+ bias[i]); A, B, C, bias are HOST arrays of device pointers
+ * (bias may be NULL, or hold NULL entries).  Pointers may repeat (the same activations times
+ * several weights).  The kernels are persistent, so the launch gap and the cold first loads of
+ * every GEMM after the first disappear.  Counterpart in the reference: the fused to_k/to_v
+ * Linear of basedxl/modules/attn.py:23-39, which gets the same effect by concatenating the
+ * weights; here the weights stay separate tensors. */
+int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, void* const* C,
+                        const void* const* bias,
+                        int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc,
+                        int dtype, int fmt, int terms, int products,
+                        const int32_t* tensor_exps,
+                        void* workspace, size_t workspace_bytes, void* stream, int variant);
+
 /* Bytes of device workspace cascmm_gemm needs for this problem (0 for most shapes).
  * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,
  * cascaded_lowp_matmul.py:155-156); the caller allocates, as it allocates `out` (:161). */

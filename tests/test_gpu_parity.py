@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from basedxl_amd import _lib, cascaded_lowp_matmul, BasedXLLowPLinear
+from basedxl_amd import _lib, cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, BasedXLLowPLinear
 from oracle import cascade as oc
 
 pytestmark = pytest.mark.gpu
@@ -229,3 +229,37 @@ def test_lowp_linear_module(gpu_device):
         + lin.bias.detach().cpu()
     assert y.shape == (2, 77, 320)
     assert torch.allclose(y.cpu().reshape(-1, 320), want, rtol=0, atol=2e-5)
+
+
+def test_grouped_launch_equals_separate_launches(gpu_device):
+    """to_q / to_k / to_v style: one activation tensor, several weights, one launch; every
+    output must be bit-identical to the single-GEMM launch of the same kernel."""
+    g = torch.Generator().manual_seed(14)
+    for (M, K, N) in [(4096, 640, 640), (300, 128, 200), (2048, 1280, 1280)]:
+        x = _gpu(torch.randn(M, K, generator=g))
+        y = _gpu(torch.randn(M, K, generator=g))
+        ws = [_gpu(torch.randn(K, N, generator=g) * 0.02) for _ in range(4)]
+        bs = [_gpu(torch.randn(N, generator=g)) for _ in range(4)]
+        _say("grouped", M, K, N)
+        outs = cascaded_lowp_matmul_grouped([x, x, x, y], ws, biases=[bs[0], None, bs[2], None])
+        torch.cuda.synchronize()
+        for i, a in enumerate([x, x, x, y]):
+            single = cascaded_lowp_matmul(a, ws[i], bias=bs[i] if i in (0, 2) else None)
+            assert torch.equal(outs[i], single), (M, K, N, i)
+    with pytest.raises(ValueError):
+        cascaded_lowp_matmul_grouped([x], [ws[0], ws[1]])
+
+
+def test_more_tiles_than_resident_workgroups(gpu_device):
+    """Persistent kernels: a workgroup walks several tiles; the prefetch ring crosses tile
+    boundaries.  Exact integer check on a problem with many more tiles than CUs."""
+    rng = np.random.default_rng(15)
+    M, K, N = 2304, 192, 1408   # 36 x 11 tiles of 64x128 ... several tiles per workgroup for every variant
+    a = rng.integers(-50, 51, size=(M, K))
+    b = rng.integers(-50, 51, size=(K, N))
+    want = a @ b
+    at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
+    for vi, name in _variants_for("bf16x2_tri"):
+        _say("many-tiles", name)
+        got = cascaded_lowp_matmul(at, bt, variant=vi).cpu().numpy().astype(np.int64)
+        assert np.array_equal(got, want), name
