@@ -53,6 +53,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   const int full = (q.products == CASCMM_PROD_FULL && q.terms > 1) ? 1 : 0;
   if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full) return false;
   if (v.fast && (!fast || q.K % v.BK != 0)) return false;
+  if (v.kind == KIND_SPLITK && (q.M > 5 * v.BM || q.K < 4 * v.BK)) return false;  // skinny: few row tiles, deep K
   return true;
 }
 
@@ -72,16 +73,27 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
   if (strstr(name, "_p8_")) step *= 0.94;
   if (name[0] == 'b' && name[1] == 'd') step *= 1.15;
   const double ksteps = (double)((q.K + 63) / 64);
+  if (v.kind == KIND_SPLITK) {
+    // Problems with too few tiles to occupy the chip: splitting K wins whenever the plain tile
+    // kernels would leave more than half of the CUs idle; among the split-K variants the
+    // smaller row tile was faster wherever both were measured.
+    if ((double)((q.M + 63) / 64) * (double)((q.N + 127) / 128) >= kNumCUs / 2) return 1e9;
+    return 1e-6 * (double)(((q.M + v.BM - 1) / v.BM) * v.BM) + 1e-8 * v.BM;
+  }
   return rounds * step * ksteps + (v.fast ? 0.0 : 1e3);
 }
 
-static int select_variant(const Problem& q, bool fast, int count) {
+// ws_bytes: workspace the caller brought (split-K variants that need more are skipped)
+static int select_variant(const Problem& q, bool fast, int count, size_t ws_bytes = (size_t)-1) {
   const auto& t = table();
   int best = -1;
   double best_cost = 0;
   for (int i = 0; i < (int)t.size(); ++i) {
     if (!variant_matches(t[i], q, fast)) continue;
     if (count > 1 && !t[i].grouped) continue;
+    if (t[i].kind == KIND_SPLITK &&
+        skinny_workspace_bytes(q.M, q.N, q.K, t[i].BM, t[i].BN, t[i].BK) > ws_bytes)
+      continue;
     const double c = variant_cost(t[i], q, count);
     if (best < 0 || c < best_cost) { best = i; best_cost = c; }
   }
@@ -134,7 +146,7 @@ static int launch_split(const void* x, float* out, int64_t n, int terms, int ten
 static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
                      const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
                      hipStream_t stream, int variant) {
-  (void)tensor_exps; (void)workspace; (void)workspace_bytes;
+  (void)tensor_exps;
   int st = check_problem(q);
   if (st != CASCMM_OK) return st;
   if (count < 1 || count > kMaxGroup) return CASCMM_ERR_BAD_SHAPE;
@@ -167,7 +179,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
 
   const auto& t = table();
   if (variant < 0) {
-    variant = select_variant(q, fast, count);
+    variant = select_variant(q, fast, count, workspace ? workspace_bytes : 0);
     if (variant < 0) return variant;
   } else {
     if (variant >= (int)t.size()) return CASCMM_ERR_BAD_VARIANT;
@@ -183,6 +195,8 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   if (tm * tn * count > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
   p.tiles_m = (int)tm; p.tiles_n = (int)tn;
   p.count = count;
+  p.workspace = workspace;
+  p.workspace_bytes = workspace_bytes;
   for (int i = 0; i < count; ++i) {
     p.A[i] = A[i]; p.B[i] = B[i]; p.C[i] = C[i]; p.bias[i] = bias ? bias[i] : nullptr;
   }
@@ -221,8 +235,17 @@ int cascmm_gemm(const void* A, const void* B, void* C, const void* bias, int64_t
 }
 
 size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms, int products) {
-  (void)M; (void)N; (void)K; (void)dtype; (void)fmt; (void)terms; (void)products;
-  return 0;
+  // upper bound over the skinny variants that could be selected for this problem (the
+  // selection also depends on pointer alignment, which is not known here)
+  const Problem q{M, N, K, K, N, N, dtype, fmt, terms, products};
+  if (check_problem(q) != CASCMM_OK) return 0;
+  size_t need = 0;
+  for (const auto& v : table()) {
+    if (v.kind != KIND_SPLITK || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
+    const size_t n = skinny_workspace_bytes(M, N, K, v.BM, v.BN, v.BK);
+    need = n > need ? n : need;
+  }
+  return need;
 }
 
 int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt,

@@ -42,7 +42,16 @@ struct LdsLayoutA {
   static __device__ __forceinline__ int swz(int kg) { return (kg * (TL::KG >= 8 ? 1 : 8 / TL::KG)) & 7; }
 };
 
-template <class TL, int FMT, int TERMS, bool FULL>
+// SPLITK: the grid is tiles x k_splits; workgroup (tile, split) multiplies the K range
+// [split * k_per_split, (split + 1) * k_per_split) and leaves an fp32 partial tile in the
+// workspace; splitk_reduce_kernel adds the partials in split order and writes C.  (Letting the
+// last workgroup of a tile do the sum inside this kernel was measured 3x slower: the
+// device-scope release / acquire it needs writes back and invalidates the whole L2 of the
+// XCD for every workgroup.)  This is the path for skinny problems (M of a few row blocks, e.g. the 2 x 77 text
+// tokens of the cross-attention K/V projections): they have too few tiles to occupy the
+// chip and are bound by the latency of streaming the weight matrix, so K is split until
+// about half the CUs have a workgroup, each reading its slab of the weights once.
+template <class TL, int FMT, int TERMS, bool FULL, bool SPLITK = false>
 struct BDirectGemm {
   typedef Lowp<FMT> LP;
   typedef typename LP::Vec Vec;
@@ -58,10 +67,10 @@ struct BDirectGemm {
   static_assert(A_IT * 2 * D <= 60, "too many A loads in flight");
 
   // ---- producers: A only ---------------------------------------------------------------------
-  static __device__ __forceinline__ void producer(const GemmParams& p, u32x4* lds, int m0, int ktiles) {
+  static __device__ __forceinline__ void producer(const GemmParams& p, u32x4* lds, int m0, int ktiles, int kbase) {
     const int ptid = threadIdx.x - TL::NCW * kWave;
-    const float* A = (const float*)p.A + (int64_t)m0 * p.lda;
-    const i32x4 ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
+    const float* A = (const float*)p.A + (int64_t)m0 * p.lda + kbase;
+    const i32x4 ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K - kbase) * ES);
     const int last_row = p.M - 1 - m0;
     int voff[A_IT], slot[A_IT];
 #pragma unroll
@@ -128,13 +137,14 @@ struct BDirectGemm {
   }
 
   // ---- consumers: B straight from global memory, A fragments from LDS ----------------------------
-  static __device__ __forceinline__ void consumer(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles, int wave) {
+  static __device__ __forceinline__ void consumer(const GemmParams& p, u32x4* lds, int m0, int n0, int ktiles, int wave,
+                                                  int kbase, int split) {
     const int lane = threadIdx.x & 63, l31 = lane & 31, g = lane >> 5;
     const int wn0 = wave * 32;
     // this lane's column, clamped (results of clamped columns are never stored)
     const int col = (n0 + wn0 + l31 < p.N) ? (n0 + wn0 + l31) : (p.N - 1);
-    const float* B = (const float*)p.B;
-    const i32x4 rb = make_rsrc(B, ((int64_t)(p.K - 1) * p.ldb + p.N) * ES);
+    const float* B = (const float*)p.B + (int64_t)kbase * p.ldb;
+    const i32x4 rb = make_rsrc(B, ((int64_t)(p.K - 1 - kbase) * p.ldb + p.N) * ES);
     const int ldb_bytes = (int)(p.ldb * ES);
     const int voff_b = (g * 8) * ldb_bytes + col * ES;
 
@@ -210,9 +220,27 @@ struct BDirectGemm {
     }
 
     // epilogue: lane holds column l31 and rows 8*q + 4*g + e of every 32-row block
+    const int ccol = n0 + wn0 + l31;
+    if (SPLITK && p.k_splits > 1) {
+      // fp32 partial tile of this K range, no bias: workspace [split][M][N], leading dimension N
+      if (ccol >= p.N) return;
+      float* dst0 = p.partials + ((int64_t)split * p.M) * p.N + ccol;
+#pragma unroll
+      for (int mi = 0; mi < TL::MT; ++mi) {
+        f32x16 v = acc[NCLS - 1][mi];
+#pragma unroll
+        for (int c = NCLS - 2; c >= 0; --c) v = v * AC::kFoldScale + acc[c][mi];
+        const int row0 = m0 + mi * 32 + g * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (row0 + q * 8 + e < p.M) dst0[(int64_t)(row0 + q * 8 + e) * p.N] = v[4 * q + e];
+      }
+      return;
+    }
     float* C = (float*)p.C;
     const float* bias = (const float*)p.bias;
-    const int ccol = n0 + wn0 + l31;
     const bool interior = (m0 + TL::BM <= p.M) && (n0 + wn0 + 32 <= p.N) && p.ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
     if (interior) {
       const i32x4 rc = make_rsrc(C + (int64_t)m0 * p.ldc, 0x7FFFFFFF);
@@ -250,20 +278,61 @@ struct BDirectGemm {
   }
 
   static __device__ __forceinline__ void run(const GemmParams& p, u32x4* lds) {
-    int tm, tn;
-    tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    int tm, tn, split = 0, kbase = 0;
+    int ktiles = p.K / TL::BK;  // the host only selects this kernel when K % BK == 0
+    if (SPLITK) {
+      // the splits of one tile are neighbours in the grid: they run at the same time
+      const int tile = blockIdx.x / p.k_splits;
+      split = blockIdx.x - tile * p.k_splits;
+      tm = tile / p.tiles_n;
+      tn = tile - tm * p.tiles_n;
+      kbase = split * p.k_per_split;
+      ktiles = p.k_per_split / TL::BK;
+    } else {
+      tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+    }
     const int m0 = tm * TL::BM, n0 = tn * TL::BN;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ktiles = p.K / TL::BK;  // the host only selects this kernel when K % BK == 0
-    if (wave >= TL::NCW) producer(p, lds, m0, ktiles);
-    else consumer(p, lds, m0, n0, ktiles, wave);
+    if (wave >= TL::NCW) producer(p, lds, m0, ktiles, kbase);
+    else consumer(p, lds, m0, n0, ktiles, wave, kbase, split);
   }
 };
 
-template <class TL, int FMT, int TERMS, bool FULL>
+template <class TL, int FMT, int TERMS, bool FULL, bool SPLITK>
 __global__ __launch_bounds__(TL::NT) void cascmm_bdirect_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char cascmm_smem[];
-  BDirectGemm<TL, FMT, TERMS, FULL>::run(p, (u32x4*)cascmm_smem);
+  BDirectGemm<TL, FMT, TERMS, FULL, SPLITK>::run(p, (u32x4*)cascmm_smem);
+}
+
+// Second pass of the split-K path: C[m][n] = bias[n] + sum over splits, in split order (so the
+// result does not depend on scheduling), of partials[split][m][n].  Four consecutive columns
+// per thread (N % 4 == 0 on this path), the loads of eight splits in flight.
+static __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partials, int k_splits, int M,
+                                                                   int N, const float* __restrict__ bias,
+                                                                   float* __restrict__ C, int64_t ldc, int vec_out) {
+  const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  const int64_t total = (int64_t)M * N;
+  if (i >= total) return;
+  const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+  const f32x4* src = (const f32x4*)(partials + i);
+  const int64_t stride = total / 4;
+  f32x4 s = src[0];
+  int k = 1;
+  for (; k + 8 <= k_splits; k += 8) {
+    f32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + (int64_t)(k + u) * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; k < k_splits; ++k) s += __builtin_nontemporal_load(src + (int64_t)k * stride);
+  if (vec_out) {  // C rows and bias 16-byte aligned
+    if (bias) s += *(const f32x4*)(bias + n);
+    *(f32x4*)(C + (int64_t)m * ldc + n) = s;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) C[(int64_t)m * ldc + n + e] = s[e] + (bias ? bias[n + e] : 0.f);
+  }
 }
 
 }  // namespace cascmm

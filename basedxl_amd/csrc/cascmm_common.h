@@ -155,6 +155,8 @@ struct GroupParams {
   const void* B[kMaxGroup];
   void* C[kMaxGroup];
   const void* bias[kMaxGroup];
+  void* workspace;          // split-K partials (skinny path)
+  size_t workspace_bytes;
 };
 
 }  // namespace cascmm

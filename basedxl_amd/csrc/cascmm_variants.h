@@ -59,7 +59,26 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, TERMS>::kBytes, FAST, true,                     \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, IODT, FMT, TERMS, FULL, FAST>}
 
-template <class TL, int FMT, int TERMS, bool FULL>
+// K splits of the skinny path: enough workgroups to occupy every CU, each with at least one
+// K step of `bk`; the same function sizes the workspace
+inline int skinny_splits(int64_t M, int64_t N, int64_t K, int bm, int bn, int bk) {
+  const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+  int best = 1;
+  for (int s = 1; s <= 64; ++s) {
+    if (K % ((int64_t)s * bk) != 0) continue;
+    best = s;
+    if (tiles * s >= kNumCUs / 2) break;  // measured optimum on 154 x 2048 x 1280
+  }
+  return best;
+}
+
+// Split-K workspace: one fp32 [M][N] partial result per split
+inline size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int bm, int bn, int bk) {
+  const int splits = skinny_splits(M, N, K, bm, bn, bk);
+  return splits <= 1 ? 0 : (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
+}
+
+template <class TL, int FMT, int TERMS, bool FULL, bool SPLITK>
 int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   if (gp.count != 1) return CASCMM_ERR_BAD_VARIANT;
   GemmParams p;
@@ -67,7 +86,19 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   p.A = gp.A[0]; p.B = gp.B[0]; p.C = gp.C[0]; p.bias = gp.bias[0];
   p.M = gp.M; p.N = gp.N; p.K = gp.K; p.lda = gp.lda; p.ldb = gp.ldb; p.ldc = gp.ldc;
   p.tiles_m = gp.tiles_m; p.tiles_n = gp.tiles_n;
-  auto kfn = cascmm_bdirect_kernel<TL, FMT, TERMS, FULL>;
+  p.k_splits = 1;
+  p.k_per_split = gp.K;
+  if (SPLITK) {
+    p.k_splits = skinny_splits(gp.M, gp.N, gp.K, TL::BM, TL::BN, TL::BK);
+    p.k_per_split = gp.K / p.k_splits;
+    if (p.k_splits > 1) {
+      const size_t need = skinny_workspace_bytes(gp.M, gp.N, gp.K, TL::BM, TL::BN, TL::BK);
+      if (!gp.workspace || gp.workspace_bytes < need) return CASCMM_ERR_WORKSPACE;
+      if ((uintptr_t)gp.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
+      p.partials = (float*)gp.workspace;
+    }
+  }
+  auto kfn = cascmm_bdirect_kernel<TL, FMT, TERMS, FULL, SPLITK>;
   constexpr int lds = LdsLayoutA<TL, TERMS>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
@@ -78,16 +109,30 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
     });
     if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
   }
-  const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n;
+  const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n * (unsigned)p.k_splits;
   hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+  if (SPLITK && p.k_splits > 1) {
+    const int64_t total = (int64_t)gp.M * gp.N;
+    const int vec_out = gp.ldc % 4 == 0 && (uintptr_t)p.C % 16 == 0 && (uintptr_t)p.bias % 16 == 0;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, p.partials,
+                       p.k_splits, gp.M, gp.N, (const float*)p.bias, (float*)p.C, gp.ldc, vec_out);
+    if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+  }
+  return CASCMM_OK;
 }
 
 // B-direct kernels: fp32 operands, fast path only
 #define CASCMM_BD_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                                \
   {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, 32 * WN, BK, TileBD<BM, WN, BK, DEPTH, NP>::NT, \
    LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true, false,                               \
-   &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL>}
+   &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL, false>}
+
+// skinny split-K kernels (one row tile): B-direct + partials + reduction
+#define CASCMM_SKINNY_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                            \
+  {NAME, KIND_SPLITK, CASCMM_DT_F32, FMT, TERMS, FULL, BM, 32 * WN, BK, TileBD<BM, WN, BK, DEPTH, NP>::NT, \
+   LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true, false,                               \
+   &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL, true>}
 
 // each instantiation unit exports its slice of the table
 const VariantDesc* variants_bf16(int* n);

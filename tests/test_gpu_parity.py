@@ -68,13 +68,16 @@ def _int_case(M, K, N, hi, seed):
 
 
 INT_SHAPES = [(16, 32, 16), (17, 33, 19), (154, 64, 48), (1, 7, 1), (130, 40, 81), (256, 192, 160), (300, 128, 200),
-              (257, 64, 161), (257, 64, 164), (96, 128, 384)]
+              (257, 64, 161), (257, 64, 164), (96, 128, 384), (154, 512, 256), (30, 256, 132), (64, 1024, 128),
+              (160, 320, 1284)]
 
 
 @pytest.mark.parametrize("shape", INT_SHAPES)
 def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
     M, K, N = shape
     a, b, want = _int_case(M, K, N, 100, seed=M + K + N)
+    hi = 100 if K <= 256 else 40
+    a, b, want = _int_case(M, K, N, hi, seed=M + K + N)
     assert np.abs(want).max() < 2 ** 24
     at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
     l = _lib.lib()
@@ -87,6 +90,8 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
         bk = int(name.split("_")[0].split("x")[2])
         if "generic" not in name and (K % bk != 0 or N % 4 != 0):
             continue  # fast variants need K % BK == 0 and N % 4 == 0 (rejected by the library otherwise)
+        if name.startswith("skinny") and (M > 5 * int(name.split("x")[0][6:]) or K < 4 * bk):
+            continue  # split-K variants take at most five row tiles and at least four K steps
         _say("int-exact", shape, name)
         out = cascaded_lowp_matmul(at, bt, lowp=fmt, terms=terms, products=products, variant=vi)
         torch.cuda.synchronize()
@@ -158,12 +163,52 @@ def test_every_headline_variant_meets_the_bound(gpu_device):
     ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exp)
     ad, bd = _gpu(a), _gpu(b)
     for vi, name in _variants_for("bf16x2_tri"):
+        if name.startswith("skinny"):
+            continue  # few row tiles only; covered by test_skinny_split_k_meets_the_bound
         _say("variant", name)
         got = oc.error_metrics(cascaded_lowp_matmul(ad, bd, variant=vi).cpu(), exp)
         assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"], name
 
 
-def test_repeated_launches_are_bit_identical(gpu_device):
+@pytest.mark.parametrize("shape", [(154, 2048, 1280), (154, 2048, 640), (32, 1024, 384), (77, 768, 320)])
+def test_skinny_split_k_meets_the_bound(gpu_device, shape):
+    """Text-token shapes (cross-attention K/V projections): the automatic choice is a split-K
+    variant, its result meets the bound and is bit-identical from launch to launch."""
+    M, K, N = shape
+    a, b = oc.make_operands(M, K, N, seed=21, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exp)
+    ad, bd = _gpu(a), _gpu(b)
+    l = _lib.lib()
+    chosen = l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0)
+    assert _lib.variant_names()[chosen].startswith("skinny"), _lib.variant_names()[chosen]
+    assert l.cascmm_workspace_bytes(M, N, K, 0, 0, 2, 0) >= M * N * 4
+    _say("skinny", shape, _lib.variant_names()[chosen])
+    bias = _gpu(torch.randn(N))
+    first = cascaded_lowp_matmul(ad, bd, bias=bias).clone()
+    got = oc.error_metrics((first - bias).cpu(), exp)
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"] + 1e-6, (got, ref)
+    for _ in range(5):
+        assert torch.equal(cascaded_lowp_matmul(ad, bd, bias=bias), first)
+
+
+def test_skinny_without_workspace_falls_back_or_reports(gpu_device):
+    """Through the C ABI with no workspace: automatic selection avoids the split-K variants,
+    a forced split-K variant reports CASCMM_ERR_WORKSPACE."""
+    M, K, N = 64, 512, 256
+    a, b = _gpu(torch.randn(M, K)), _gpu(torch.randn(K, N))
+    out = torch.empty(M, N, device=a.device)
+    l = _lib.lib()
+    st = l.cascmm_gemm(a.data_ptr(), b.data_ptr(), out.data_ptr(), None, M, N, K, K, N, N, 0, 0, 2, 0, None, None, 0,
+                       torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out, cascaded_lowp_matmul(a, b), rtol=1e-4, atol=1e-3)
+    forced = [i for i, n in enumerate(_lib.variant_names()) if n.startswith("skinny64") and "bf16x2_tri" in n][0]
+    st = l.cascmm_gemm_variant(a.data_ptr(), b.data_ptr(), out.data_ptr(), None, M, N, K, K, N, N, 0, 0, 2, 0, None,
+                               None, 0, torch.cuda.current_stream().cuda_stream, forced)
+    assert st == -5
+
     a, b = oc.make_operands(1000, 648, 640, seed=10, w_std=0.02)
     ad, bd = _gpu(a), _gpu(b)
     first = cascaded_lowp_matmul(ad, bd).clone()
@@ -233,7 +278,8 @@ def test_lowp_linear_module(gpu_device):
 
 def test_grouped_launch_equals_separate_launches(gpu_device):
     """to_q / to_k / to_v style: one activation tensor, several weights, one launch; every
-    output must be bit-identical to the single-GEMM launch of the same kernel."""
+    output must be bit-identical to the single-GEMM launch of the same kernel variant (the
+    automatic choice may differ between a group and a single GEMM: then only close)."""
     g = torch.Generator().manual_seed(14)
     for (M, K, N) in [(4096, 640, 640), (300, 128, 200), (2048, 1280, 1280)]:
         x = _gpu(torch.randn(M, K, generator=g))
@@ -245,7 +291,14 @@ def test_grouped_launch_equals_separate_launches(gpu_device):
         torch.cuda.synchronize()
         for i, a in enumerate([x, x, x, y]):
             single = cascaded_lowp_matmul(a, ws[i], bias=bs[i] if i in (0, 2) else None)
-            assert torch.equal(outs[i], single), (M, K, N, i)
+            torch.testing.assert_close(outs[i], single, rtol=1e-4, atol=1e-4)
+        for vi, name in _variants_for("bf16x2_tri"):
+            if name.startswith(("bd", "skinny")) or "generic" in name or K % int(name.split("_")[0].split("x")[2]):
+                continue
+            outs = cascaded_lowp_matmul_grouped([x, x, x, y], ws, biases=[bs[0], None, bs[2], None], variant=vi)
+            for i, a in enumerate([x, x, x, y]):
+                single = cascaded_lowp_matmul(a, ws[i], bias=bs[i] if i in (0, 2) else None, variant=vi)
+                assert torch.equal(outs[i], single), (M, K, N, i, name)
     with pytest.raises(ValueError):
         cascaded_lowp_matmul_grouped([x], [ws[0], ws[1]])
 
@@ -260,6 +313,8 @@ def test_more_tiles_than_resident_workgroups(gpu_device):
     want = a @ b
     at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
     for vi, name in _variants_for("bf16x2_tri"):
+        if name.startswith("skinny"):
+            continue
         _say("many-tiles", name)
         got = cascaded_lowp_matmul(at, bt, variant=vi).cpu().numpy().astype(np.int64)
         assert np.array_equal(got, want), name
