@@ -121,8 +121,19 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
     pc = arr(*[t.data_ptr() for t in outs])
     pbias = arr(*[(None if bb is None else bb.data_ptr()) for bb in biases]) if biases is not None else None
     stream = torch.cuda.current_stream(dev).cuda_stream
+    exps = None
+    if fmt == _lib.FMT_FP8:
+        # tensor scale exponents {e_A, e_B} of every problem, computed on the device
+        exps = torch.empty(2 * n, dtype=torch.int32, device=dev)
+        dt = _DTYPES[a_list[0].dtype]
+        for i in range(n):
+            _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, dt, exps.data_ptr() + 8 * i, stream),
+                       "cascmm_tensor_exp(A)")
+            _lib.check(_lib.lib().cascmm_tensor_exp(b_list[i].data_ptr(), K, N, max(N, 1), dt,
+                                                    exps.data_ptr() + 8 * i + 4, stream), "cascmm_tensor_exp(B)")
     st = _lib.lib().cascmm_gemm_grouped(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), max(N, 1),
-                                        _DTYPES[a_list[0].dtype], fmt, terms, prod, None, None, 0, stream, variant)
+                                        _DTYPES[a_list[0].dtype], fmt, terms, prod,
+                                        exps.data_ptr() if exps is not None else None, None, 0, stream, variant)
     _lib.check(st, "cascmm_gemm_grouped")
     return [o.reshape(*a.shape[:-1], N) for o, a in zip(outs, a_list)]
 

@@ -1,4 +1,5 @@
 // extern "C" entry points: argument checks, kernel selection, small utility kernels.
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <vector>
@@ -17,6 +18,8 @@ static const std::vector<VariantDesc>& table() {
     const VariantDesc* p = variants_bf16(&n);
     v.insert(v.end(), p, p + n);
     p = variants_fp16(&n);
+    v.insert(v.end(), p, p + n);
+    p = variants_fp8(&n);
     v.insert(v.end(), p, p + n);
     return v;
   }();
@@ -112,6 +115,40 @@ __global__ void fill_bias_kernel(void* C, const void* bias, int M, int N, int64_
   IoType<IODT>::store((T*)C + (int64_t)r * ldc + c, bias ? IoType<IODT>::load((const T*)bias + c) : 0.f);
 }
 
+// fp8 tensor scale, three stream-ordered steps on the caller's int32: zero it, fold in the bit
+// pattern of max|x| (non-negative floats order like their bit patterns), turn it into the
+// exponent e with max|x| * 2^e in (224, 448]
+__global__ void amax_begin_kernel(int32_t* exp_out) { *exp_out = 0; }
+
+template <int IODT>
+__global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld, int32_t* exp_out) {
+  typedef typename IoType<IODT>::T T;
+  const int64_t total = rows * cols;
+  unsigned best = 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / cols, c = i - r * cols;
+    const unsigned bits = __builtin_bit_cast(unsigned, IoType<IODT>::load((const T*)x + r * ld + c)) & 0x7FFFFFFFu;
+    best = bits > best ? bits : best;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned other = (unsigned)__shfl_xor((int)best, off, 64);
+    best = other > best ? other : best;
+  }
+  if ((threadIdx.x & 63) == 0 && best != 0) atomicMax((unsigned*)exp_out, best);
+}
+
+__global__ void amax_end_kernel(int32_t* exp_out) {
+  const unsigned bits = (unsigned)*exp_out;
+  int e = 0;
+  if (bits != 0 && bits < 0x7F800000u) {   // finite and non-zero
+    int ex;
+    const float m = frexpf(__builtin_bit_cast(float, bits), &ex);   // m in [0.5, 1)
+    e = m <= 0.875f ? 9 - ex : 8 - ex;                              // 448 = 0.875 * 2^9
+  }
+  *exp_out = e;
+}
+
 template <int IODT, int FMT, int TERMS>
 __global__ void split_terms_kernel(const void* x, float* out, int64_t n, int tensor_exp) {
   typedef typename IoType<IODT>::T T;
@@ -121,12 +158,11 @@ __global__ void split_terms_kernel(const void* x, float* out, int64_t n, int ten
   r[0] = IoType<IODT>::load((const T*)x + i) * __builtin_ldexpf(1.0f, tensor_exp);
 #pragma unroll
   for (int e = 1; e < 8; ++e) r[e] = 0.f;
-  u32x4 t[TERMS];
+  u32x4 t[Lowp<FMT>::planes(TERMS)];
   split8<FMT, TERMS>(r, t);
 #pragma unroll
   for (int k = 0; k < TERMS; ++k) {
-    typename Lowp<FMT>::Vec v = __builtin_bit_cast(typename Lowp<FMT>::Vec, t[k]);
-    out[(int64_t)k * n + i] = (float)v[0];
+    out[(int64_t)k * n + i] = Lowp<FMT>::element0(t[Lowp<FMT>::plane(k)], k);
   }
 }
 
@@ -146,7 +182,6 @@ static int launch_split(const void* x, float* out, int64_t n, int terms, int ten
 static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
                      const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
                      hipStream_t stream, int variant) {
-  (void)tensor_exps;
   int st = check_problem(q);
   if (st != CASCMM_OK) return st;
   if (count < 1 || count > kMaxGroup) return CASCMM_ERR_BAD_SHAPE;
@@ -197,6 +232,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   p.count = count;
   p.workspace = workspace;
   p.workspace_bytes = workspace_bytes;
+  p.tensor_exps = q.fmt == CASCMM_FMT_FP8 ? tensor_exps : nullptr;
   for (int i = 0; i < count; ++i) {
     p.A[i] = A[i]; p.B[i] = B[i]; p.C[i] = C[i]; p.bias[i] = bias ? bias[i] : nullptr;
   }
@@ -265,8 +301,25 @@ const char* cascmm_variant_name(int variant) {
 
 int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, int32_t* exp_out,
                       void* stream) {
-  (void)x; (void)rows; (void)cols; (void)ld; (void)dtype; (void)exp_out; (void)stream;
-  return CASCMM_ERR_BAD_FORMAT;
+  if (dtype != CASCMM_DT_F32 && dtype != CASCMM_DT_F16 && dtype != CASCMM_DT_BF16) return CASCMM_ERR_BAD_DTYPE;
+  if (rows < 0 || cols < 0 || ld < cols) return CASCMM_ERR_BAD_SHAPE;
+  if (!exp_out || (rows * cols > 0 && !x)) return CASCMM_ERR_NULL_POINTER;
+  if (rows > INT32_MAX || cols > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  hipStream_t s = (hipStream_t)stream;
+  // *exp_out holds the bit pattern of the running max|x| until the last kernel replaces it
+  hipLaunchKernelGGL(amax_begin_kernel, dim3(1), dim3(1), 0, s, exp_out);
+  const int64_t total = rows * cols;
+  if (total > 0) {
+    const unsigned grid = (unsigned)std::min<int64_t>((total + 1023) / 1024, 2048);
+    if (dtype == CASCMM_DT_F32)
+      hipLaunchKernelGGL((amax_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
+    else if (dtype == CASCMM_DT_F16)
+      hipLaunchKernelGGL((amax_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
+    else
+      hipLaunchKernelGGL((amax_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
+  }
+  hipLaunchKernelGGL(amax_end_kernel, dim3(1), dim3(1), 0, s, exp_out);
+  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
 int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms, int tensor_exp,
@@ -278,6 +331,7 @@ int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt,
   hipStream_t s = (hipStream_t)stream;
   if (fmt == CASCMM_FMT_BF16) return launch_split<CASCMM_DT_F32, CASCMM_FMT_BF16>(x, out, n, terms, tensor_exp, s);
   if (fmt == CASCMM_FMT_FP16) return launch_split<CASCMM_DT_F32, CASCMM_FMT_FP16>(x, out, n, terms, tensor_exp, s);
+  if (fmt == CASCMM_FMT_FP8) return launch_split<CASCMM_DT_F32, CASCMM_FMT_FP8>(x, out, n, terms, tensor_exp, s);
   return CASCMM_ERR_BAD_FORMAT;
 }
 

@@ -47,7 +47,14 @@ template <int FMT> struct Lowp;
 
 template <> struct Lowp<CASCMM_FMT_BF16> {
   static constexpr int kShift = 0;
+  static constexpr bool kTensorScaled = false;
   typedef bf16x8 Vec;
+  // LDS planes (16-byte slots per 8 k of one row) that hold `terms` terms, the plane of term i
+  // and the MFMA operand of term i inside a slot read from that plane
+  static constexpr __host__ __device__ int planes(int terms) { return terms; }
+  static constexpr __host__ __device__ int plane(int i) { return i; }
+  static __device__ __forceinline__ Vec operand(u32x4 slot, int) { return __builtin_bit_cast(Vec, slot); }
+  static __device__ __forceinline__ float element0(u32x4 slot, int) { return (float)__builtin_bit_cast(Vec, slot)[0]; }
   static __device__ __forceinline__ f32x16 mfma(Vec a, Vec b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
@@ -75,7 +82,12 @@ template <> struct Lowp<CASCMM_FMT_BF16> {
 
 template <> struct Lowp<CASCMM_FMT_FP16> {
   static constexpr int kShift = 11;
+  static constexpr bool kTensorScaled = false;
   typedef f16x8 Vec;
+  static constexpr __host__ __device__ int planes(int terms) { return terms; }
+  static constexpr __host__ __device__ int plane(int i) { return i; }
+  static __device__ __forceinline__ Vec operand(u32x4 slot, int) { return __builtin_bit_cast(Vec, slot); }
+  static __device__ __forceinline__ float element0(u32x4 slot, int) { return (float)__builtin_bit_cast(Vec, slot)[0]; }
   static __device__ __forceinline__ f32x16 mfma(Vec a, Vec b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -94,11 +106,69 @@ template <> struct Lowp<CASCMM_FMT_FP16> {
   }
 };
 
+// fp8 (OCP e4m3, finite range +-448): 8 values of a term are 8 bytes, so one 16-byte slot
+// holds two terms of the same 8 k (terms 0 | 1 in plane 0, term 2 in the low half of plane 1)
+// and v_mfma_f32_32x32x16_fp8_fp8 takes a 64-bit half slot as its operand.  The term shift
+// is 4 bits; the tensor scale 2^e (max|x| * 2^e in (224, 448]) is applied before the split and
+// undone once on the result.
+template <> struct Lowp<CASCMM_FMT_FP8> {
+  static constexpr int kShift = 4;
+  static constexpr bool kTensorScaled = true;
+  typedef long Vec;
+  static constexpr __host__ __device__ int planes(int terms) { return (terms + 1) / 2; }
+  static constexpr __host__ __device__ int plane(int i) { return i / 2; }
+  static __device__ __forceinline__ Vec operand(u32x4 slot, int i) {
+    const unsigned lo = (i & 1) ? slot[2] : slot[0], hi = (i & 1) ? slot[3] : slot[1];
+    return (long)(((unsigned long)hi << 32) | lo);
+  }
+  static __device__ __forceinline__ float element0(u32x4 slot, int i) {
+    return __builtin_amdgcn_cvt_pk_f32_fp8((int)((i & 1) ? slot[2] : slot[0]), false)[0];
+  }
+  static __device__ __forceinline__ f32x16 mfma(Vec a, Vec b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
+  }
+  // round the 8 residuals (already scaled for this term) to fp8: two packed words; unless LAST,
+  // the residuals become (r - t) * 16, the input of the next term (both steps exact)
+  template <bool LAST>
+  static __device__ __forceinline__ u32x2 peel(float (&r)[8]) {
+    u32x2 out;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      int w = 0;
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(r[4 * h], r[4 * h + 1], w, false);
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(r[4 * h + 2], r[4 * h + 3], w, true);
+      out[h] = (unsigned)w;
+      if (!LAST) {
+        const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+        const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+        r[4 * h] = (r[4 * h] - lo[0]) * 16.f;
+        r[4 * h + 1] = (r[4 * h + 1] - lo[1]) * 16.f;
+        r[4 * h + 2] = (r[4 * h + 2] - hi[0]) * 16.f;
+        r[4 * h + 3] = (r[4 * h + 3] - hi[1]) * 16.f;
+      }
+    }
+    return out;
+  }
+};
+
+// split 8 consecutive k of one row / column into the LDS slots of every plane; in_scale is the
+// tensor scale (formats with kTensorScaled only)
 template <int FMT, int TERMS>
-__device__ __forceinline__ void split8(float (&r)[8], u32x4 (&out)[TERMS]) {
-  out[0] = Lowp<FMT>::template peel<0, TERMS == 1>(r);
-  if constexpr (TERMS > 1) out[1] = Lowp<FMT>::template peel<1, TERMS == 2>(r);
-  if constexpr (TERMS > 2) out[2] = Lowp<FMT>::template peel<2, TERMS == 3>(r);
+__device__ __forceinline__ void split8(float (&r)[8], u32x4 (&out)[Lowp<FMT>::planes(TERMS)], float in_scale = 1.f) {
+  if constexpr (FMT == CASCMM_FMT_FP8) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] *= in_scale;
+    const u32x2 t0 = Lowp<FMT>::template peel<TERMS == 1>(r);
+    u32x2 t1 = {0u, 0u}, t2 = {0u, 0u};
+    if constexpr (TERMS > 1) t1 = Lowp<FMT>::template peel<TERMS == 2>(r);
+    if constexpr (TERMS > 2) t2 = Lowp<FMT>::template peel<true>(r);
+    out[0] = (u32x4){t0[0], t0[1], t1[0], t1[1]};
+    if constexpr (TERMS > 2) out[1] = (u32x4){t2[0], t2[1], 0u, 0u};
+  } else {
+    out[0] = Lowp<FMT>::template peel<0, TERMS == 1>(r);
+    if constexpr (TERMS > 1) out[1] = Lowp<FMT>::template peel<1, TERMS == 2>(r);
+    if constexpr (TERMS > 2) out[2] = Lowp<FMT>::template peel<2, TERMS == 3>(r);
+  }
 }
 
 // scale class of product (i, j) is i + j; products kept: i + j <= TERMS-1 (tri) or all (full)
@@ -124,7 +194,8 @@ template <int FMT, int TERMS, bool FULL> struct AccClasses {
   static constexpr float kFoldScale = kScaled ? 1.0f / (float)(1 << Lowp<FMT>::kShift) : 1.0f;
   static constexpr __host__ __device__ int index(int s) { return kCount == 1 ? 0 : (s < kCount ? s : kCount - 1); }
   // cascades that reach the fp32 rounding floor accumulate class 0 in blocks of kChunkK
-  static constexpr bool kChunked = kScaled ? (TERMS >= 2) : (TERMS >= 3);
+  // (not fp8: its 12 bits of three terms stay far above that floor)
+  static constexpr bool kChunked = FMT == CASCMM_FMT_FP8 ? false : (kScaled ? (TERMS >= 2) : (TERMS >= 3));
   static constexpr int kChunkK = 256;
 };
 
@@ -157,6 +228,7 @@ struct GroupParams {
   const void* bias[kMaxGroup];
   void* workspace;          // split-K partials (skinny path)
   size_t workspace_bytes;
+  const int32_t* tensor_exps;  // fp8: {e_A, e_B} of problem i at [2i], [2i + 1]; NULL = all zero
 };
 
 }  // namespace cascmm

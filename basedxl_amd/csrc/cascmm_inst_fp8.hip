@@ -1,0 +1,27 @@
+// Instantiations: fp8 (OCP e4m3) terms with a power-of-two tensor scale, fp32 operands in memory.
+#include "cascmm_variants.h"
+
+namespace cascmm {
+
+#define F32 CASCMM_DT_F32
+#define F8 CASCMM_FMT_FP8
+
+static const VariantDesc kTable[] = {
+    // three terms (12 significand bits), six products.  name, BM, BN, BK, WM, WN, WK, DEPTH
+    CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp8x3_tri", 128, 128, 32, 4, 2, 1, 2, F32, F8, 3, false, true),
+    CASCMM_TILE_VARIANT("t64x64x64_w2x2x1_d2_fp8x3_tri", 64, 64, 64, 2, 2, 1, 2, F32, F8, 3, false, true),
+    CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x3_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 3, false, false),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp8x2_tri", 128, 128, 32, 4, 2, 1, 2, F32, F8, 2, false, true),
+    CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x2_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 2, false, false),
+    CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp8x1", 128, 128, 32, 4, 2, 1, 2, F32, F8, 1, false, true),
+    CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x1_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 1, false, false),
+    CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x3_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 3, true, false),
+    CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x2_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 2, true, false),
+};
+
+const VariantDesc* variants_fp8(int* n) {
+  *n = (int)(sizeof(kTable) / sizeof(kTable[0]));
+  return kTable;
+}
+
+}  // namespace cascmm

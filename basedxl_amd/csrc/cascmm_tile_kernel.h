@@ -136,7 +136,8 @@ template <class TL, int IODT, int FMT, int TERMS, bool FULL>
 struct TileGemm {
   typedef Lowp<FMT> LP;
   typedef typename LP::Vec Vec;
-  typedef LdsLayout<TL, TERMS> LL;
+  static constexpr int PL = LP::planes(TERMS);   // LDS planes per operand
+  typedef LdsLayout<TL, PL> LL;
   typedef ProductSet<TERMS, FULL> PS;
   typedef AccClasses<FMT, TERMS, FULL> AC;
   typedef typename IoType<IODT>::T IoT;
@@ -189,6 +190,7 @@ struct TileGemm {
       int lds_q[Q_IT > 0 ? Q_IT : 1];    // slot of column 4*quad (the other three follow at +32, +64, +96)
       int lds_b[B_IT > 0 ? B_IT : 1];
       int ldb_bytes;
+      float scale_a, scale_b;            // tensor scales 2^e_A, 2^e_B (fp8), else 1
     };
 
     // LDS slot of every unit this thread stages (fixed for the whole kernel)
@@ -223,6 +225,13 @@ struct TileGemm {
       c.ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
       c.rb = make_rsrc(B, ((int64_t)(p.K - 1) * p.ldb + (p.N - n0)) * ES);
       c.ldb_bytes = (int)(p.ldb * ES);
+      c.scale_a = c.scale_b = 1.f;
+      if constexpr (LP::kTensorScaled) {
+        if (p.tensor_exps) {
+          c.scale_a = __builtin_ldexpf(1.f, p.tensor_exps[2 * prob]);
+          c.scale_b = __builtin_ldexpf(1.f, p.tensor_exps[2 * prob + 1]);
+        }
+      }
       const int last_row = p.M - 1 - m0, last_col = p.N - 1 - n0;
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
@@ -330,15 +339,15 @@ struct TileGemm {
     // they would stall the wave on the full address FIFO with no VALU work to overlap.
     template <bool ISSUE>
     static __device__ __forceinline__ void restage(const Ctx& c, u32x4* stage, Regs& r, int k_next) {
-      u32x4* sb = stage + TERMS * LL::kATerm;
+      u32x4* sb = stage + PL * LL::kATerm;
       const int soff_a = k_next * ES;
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
         if (A_UNITS % NTR == 0 || c.lds_a[it] >= 0) {
-          u32x4 t[TERMS];
-          split8<FMT, TERMS>(r.a[it], t);
+          u32x4 t[PL];
+          split8<FMT, TERMS>(r.a[it], t, c.scale_a);
 #pragma unroll
-          for (int i = 0; i < TERMS; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+          for (int i = 0; i < PL; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
         }
         if (ISSUE) {
           const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
@@ -358,10 +367,10 @@ struct TileGemm {
             float x[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = r.q[it][e][i];
-            u32x4 t[TERMS];
-            split8<FMT, TERMS>(x, t);
+            u32x4 t[PL];
+            split8<FMT, TERMS>(x, t, c.scale_b);
 #pragma unroll
-            for (int tt = 0; tt < TERMS; ++tt) sb[tt * LL::kBTerm + c.lds_q[it] + i * 32] = t[tt];
+            for (int tt = 0; tt < PL; ++tt) sb[tt * LL::kBTerm + c.lds_q[it] + i * 32] = t[tt];
           }
         }
         if (ISSUE) {
@@ -376,10 +385,10 @@ struct TileGemm {
 #pragma unroll
       for (int it = 0; it < B_IT; ++it) {
         if (B_UNITS % NTR == 0 || c.lds_b[it] >= 0) {
-          u32x4 t[TERMS];
-          split8<FMT, TERMS>(r.b[it], t);
+          u32x4 t[PL];
+          split8<FMT, TERMS>(r.b[it], t, c.scale_b);
 #pragma unroll
-          for (int i = 0; i < TERMS; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+          for (int i = 0; i < PL; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
         }
         if (ISSUE) {
 #pragma unroll
@@ -472,20 +481,20 @@ struct TileGemm {
                                                  f32x16 (&acc)[NCLS][TL::MT][TL::NTL]) {
     const int lane = threadIdx.x & 63, l31 = lane & 31, g = lane >> 5;
     const u32x4* sa = stage;
-    const u32x4* sb = stage + TERMS * LL::kATerm;
+    const u32x4* sb = stage + PL * LL::kATerm;
 #pragma unroll
     for (int kk = 0; kk < TL::KSUB / TL::WK; ++kk) {
       const int ks = kk * TL::WK + wk;
       const int kg = ks * 2 + g;
-      Vec a[TERMS][TL::MT], b[TERMS][TL::NTL];
+      u32x4 a[PL][TL::MT], b[PL][TL::NTL];
 #pragma unroll
-      for (int i = 0; i < TERMS; ++i) {
+      for (int i = 0; i < PL; ++i) {
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi)
-          a[i][mi] = __builtin_bit_cast(Vec, sa[i * LL::kATerm + kg * LL::kAPlane + wm0 + mi * 32 + (l31 ^ LL::swz(kg))]);
+          a[i][mi] = sa[i * LL::kATerm + kg * LL::kAPlane + wm0 + mi * 32 + (l31 ^ LL::swz(kg))];
 #pragma unroll
         for (int ni = 0; ni < TL::NTL; ++ni)
-          b[i][ni] = __builtin_bit_cast(Vec, sb[i * LL::kBTerm + kg * LL::kBPlane + wn0 + ni * 32 + l31]);
+          b[i][ni] = sb[i * LL::kBTerm + kg * LL::kBPlane + wn0 + ni * 32 + l31];
       }
       // smallest products first; consecutive MFMAs go to different accumulators
 #pragma unroll
@@ -498,7 +507,9 @@ struct TileGemm {
 #pragma unroll
           for (int mi = 0; mi < TL::MT; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < TL::NTL; ++ni) acc[cls][mi][ni] = LP::mfma(a[i][mi], b[j][ni], acc[cls][mi][ni]);
+            for (int ni = 0; ni < TL::NTL; ++ni)
+              acc[cls][mi][ni] = LP::mfma(LP::operand(a[LP::plane(i)][mi], i), LP::operand(b[LP::plane(j)][ni], j),
+                                          acc[cls][mi][ni]);
         }
     }
   }
@@ -572,6 +583,10 @@ struct TileGemm {
     // fold the scale classes (smallest first), then the cross-wave-group reduction (WK == 2):
     // group 1 parks its tile in LDS, group 0 adds it
     f32x16 res[TL::MT][TL::NTL];
+    float out_scale = 1.f;   // undoes the tensor scales of both operands (fp8)
+    if constexpr (LP::kTensorScaled) {
+      if (p.tensor_exps) out_scale = __builtin_ldexpf(1.f, -(p.tensor_exps[2 * prob] + p.tensor_exps[2 * prob + 1]));
+    }
 #pragma unroll
     for (int mi = 0; mi < TL::MT; ++mi)
 #pragma unroll
@@ -579,6 +594,7 @@ struct TileGemm {
         f32x16 v = acc[NCLS - 1][mi][ni];
 #pragma unroll
         for (int c = NCLS - 2; c >= 0; --c) v = v * AC::kFoldScale + acc[c][mi][ni];
+        if constexpr (LP::kTensorScaled) v = v * out_scale;
         res[mi][ni] = v;
       }
     const int lane = threadIdx.x & 63, l31 = lane & 31, g = lane >> 5;

@@ -24,7 +24,7 @@ struct VariantDesc {
 template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
 int launch_tile(const GroupParams& p, hipStream_t stream) {
   auto kfn = cascmm_tile_kernel<TL, IODT, FMT, TERMS, FULL, FAST>;
-  constexpr int lds = LdsLayout<TL, TERMS>::kBytes;
+  constexpr int lds = LdsLayout<TL, Lowp<FMT>::planes(TERMS)>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
     static std::once_flag once;
@@ -50,13 +50,13 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
 
 #define CASCMM_TILE_VARIANT(NAME, BM, BN, BK, WM, WN, WK, DEPTH, IODT, FMT, TERMS, FULL, FAST)         \
   {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH>::NT,       \
-   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, TERMS>::kBytes, FAST, true,                         \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, Lowp<FMT>::planes(TERMS)>::kBytes, FAST, true,       \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH>, IODT, FMT, TERMS, FULL, FAST>}
 
 // same with the number of producer waves given explicitly
 #define CASCMM_TILE_VARIANT_P(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)    \
   {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>::NT,   \
-   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, TERMS>::kBytes, FAST, true,                     \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, Lowp<FMT>::planes(TERMS)>::kBytes, FAST, true,   \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, IODT, FMT, TERMS, FULL, FAST>}
 
 // K splits of the skinny path: enough workgroups to occupy every CU, each with at least one
@@ -137,6 +137,7 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
 // each instantiation unit exports its slice of the table
 const VariantDesc* variants_bf16(int* n);
 const VariantDesc* variants_fp16(int* n);
+const VariantDesc* variants_fp8(int* n);
 const VariantDesc* variants_io16(int* n);
 
 }  // namespace cascmm

@@ -16,6 +16,12 @@ from oracle import cascade as oc
 pytestmark = pytest.mark.gpu
 
 TOL = 1.25  # kernel error may be at most this multiple of the oracle cascade's error
+# v_mfma_f32_32x32x16_fp8_fp8 adds the 8 products of one lane in a window of about 15 bits below
+# the largest of them (measured: 448*448 + 2^2 returns 448*448, + 2^3 is kept; across the two
+# lane groups and into the accumulator it adds in full fp32).  That truncation, about 1.5e-5
+# relative, is below the error of the fp8 cascades that drop products, but it is what is left
+# when all nine products of three terms are kept: that one cascade gets a wider bound.
+TOL_FP8_FULL = 2.0
 
 
 def _say(*a):
@@ -57,6 +63,48 @@ def test_split_matches_oracle_bit_for_bit(gpu_device, fmt, terms):
         assert bad.numel() == 0, (fmt, terms, i, [(float(x[j]), float(got[i][j]), float(want[i][j])) for j in bad[:8]])
 
 
+@pytest.mark.parametrize("terms", [1, 2, 3])
+@pytest.mark.parametrize("scale", [1.0, 0.02, 37.5])
+def test_fp8_split_and_tensor_scale_match_oracle(gpu_device, terms, scale):
+    """fp8-e4m3 terms with the power-of-two tensor scale: the exponent found on the device and
+    every term must equal the oracle's, bit for bit (e4m3 subnormals and the 448 edge included)."""
+    _say("fp8 split", terms, scale)
+    g = torch.Generator().manual_seed(3)
+    x = torch.cat([torch.randn(50_000, generator=g), torch.randn(5_000, generator=g) * 1e-3,
+                   torch.tensor([0.0, -0.0, 1.0, 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -10, 1.0625, 1.03125, -1.09375])]).float()
+    x = x * scale
+    e = oc.tensor_scale_exp(x, "fp8")
+    xd = _gpu(x)
+    l = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    ed = torch.full((1,), 12345, dtype=torch.int32, device=xd.device)
+    assert l.cascmm_tensor_exp(xd.data_ptr(), 1, x.numel(), x.numel(), _lib.DT_F32, ed.data_ptr(), stream) == 0
+    assert int(ed.cpu()[0]) == e
+    want, _ = oc.split_terms(x, "fp8", terms, tensor_exp=e)
+    out = torch.empty(terms, x.numel(), dtype=torch.float32, device=xd.device)
+    assert l.cascmm_split_terms(xd.data_ptr(), out.data_ptr(), x.numel(), _lib.DT_F32, _lib.FMT_BY_NAME["fp8"], terms, e,
+                                stream) == 0
+    got = out.cpu()
+    for i in range(terms):
+        both_zero = (got[i] == 0) & (want[i] == 0)
+        bad = ((got[i].view(torch.int32) != want[i].view(torch.int32)) & ~both_zero).nonzero().flatten()
+        assert bad.numel() == 0, (terms, i, [(float(x[j]), float(got[i][j]), float(want[i][j])) for j in bad[:8]])
+
+
+@pytest.mark.parametrize("values", [[0.0, 0.0], [448.0, -3.0], [448.0001, 1.0], [224.0, 1.0], [224.0001, 0.5],
+                                    [3.5e-3, -7e-3], [1e-30, 0.0], [2.0 ** -140, 0.0], [float("inf"), 1.0]])
+def test_tensor_exp_edges(gpu_device, values):
+    x = torch.tensor(values, dtype=torch.float32).repeat(3, 1)       # [3, 2] with a padded leading dimension
+    xd = _gpu(torch.zeros(3, 5))
+    xd[:, :2] = _gpu(x)
+    xd[:, 2:] = 1e30                                                  # outside the [rows, cols] window
+    ed = torch.zeros(1, dtype=torch.int32, device=xd.device)
+    st = _lib.lib().cascmm_tensor_exp(xd.data_ptr(), 3, 2, 5, _lib.DT_F32, ed.data_ptr(),
+                                      torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    assert int(ed.cpu()[0]) == oc.tensor_scale_exp(x, "fp8"), values
+
+
 # ---------------------------------------------------------------------------------------
 # exact integer known-answer tests, every kernel variant, ragged shapes
 # ---------------------------------------------------------------------------------------
@@ -80,23 +128,29 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
     a, b, want = _int_case(M, K, N, hi, seed=M + K + N)
     assert np.abs(want).max() < 2 ** 24
     at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
+    # operands that fit one fp8 term (4 significand bits), for the cascades that keep too few
+    # products of the lower terms to be exact on 7-bit integers
+    a7, b7, want7 = _int_case(M, K, N, 7, seed=M + K + N + 1)
+    at7, bt7 = _gpu(torch.tensor(a7, dtype=torch.float32)), _gpu(torch.tensor(b7, dtype=torch.float32))
     l = _lib.lib()
     names = _lib.variant_names()
     ran = 0
     for vi, name in enumerate(names):
-        fmt = "bf16" if "bf16" in name else "fp16"
+        fmt = [f for f in ("bf16", "fp16", "fp8") if f + "x" in name][0]
         terms = int(name.split(fmt + "x")[1][0])
         products = "full" if "_full" in name else "tri"
+        small = fmt == "fp8" and (terms == 1 or (terms == 2 and products == "tri"))
         bk = int(name.split("_")[0].split("x")[2])
         if "generic" not in name and (K % bk != 0 or N % 4 != 0):
             continue  # fast variants need K % BK == 0 and N % 4 == 0 (rejected by the library otherwise)
         if name.startswith("skinny") and (M > 5 * int(name.split("x")[0][6:]) or K < 4 * bk):
             continue  # split-K variants take at most five row tiles and at least four K steps
         _say("int-exact", shape, name)
-        out = cascaded_lowp_matmul(at, bt, lowp=fmt, terms=terms, products=products, variant=vi)
+        out = cascaded_lowp_matmul(at7 if small else at, bt7 if small else bt, lowp=fmt, terms=terms, products=products,
+                                   variant=vi)
         torch.cuda.synchronize()
         got = out.cpu().numpy()
-        assert np.array_equal(got.astype(np.int64), want), (name, shape)
+        assert np.array_equal(got.astype(np.int64), want7 if small else want), (name, shape)
         ran += 1
     assert ran >= 5
 
@@ -137,7 +191,7 @@ ACC_CASES = [
     ("ragged", 333, 456, 211, 1.0, 6),
 ]
 ACC_FORMATS = [("bf16", 2, "tri"), ("bf16", 2, "full"), ("bf16", 3, "tri"), ("fp16", 3, "tri"), ("fp16", 2, "tri"),
-               ("bf16", 1, "tri")]
+               ("bf16", 1, "tri"), ("fp8", 3, "tri"), ("fp8", 2, "tri"), ("fp8", 1, "tri"), ("fp8", 3, "full")]
 
 
 @pytest.mark.parametrize("case", ACC_CASES, ids=[c[0] for c in ACC_CASES])
@@ -153,8 +207,9 @@ def test_error_vs_fp64_within_bound_of_oracle(gpu_device, case, fmt, terms, prod
     got = oc.error_metrics(out.cpu(), exp)
     _say(f"   rel_fro kernel {got['rel_fro']:.3e} oracle {ref['rel_fro']:.3e}  max_abs kernel {got['max_abs']:.3e} "
          f"oracle {ref['max_abs']:.3e}")
-    assert got["rel_fro"] <= TOL * ref["rel_fro"], (got["rel_fro"], ref["rel_fro"])
-    assert got["max_abs"] <= TOL * ref["max_abs"], (got["max_abs"], ref["max_abs"])
+    tol = TOL_FP8_FULL if (fmt, terms, products) == ("fp8", 3, "full") else TOL
+    assert got["rel_fro"] <= tol * ref["rel_fro"], (got["rel_fro"], ref["rel_fro"])
+    assert got["max_abs"] <= tol * ref["max_abs"], (got["max_abs"], ref["max_abs"])
 
 
 def test_every_headline_variant_meets_the_bound(gpu_device):
