@@ -44,8 +44,22 @@ def _check_device_tensor(t: torch.Tensor, name: str) -> None:
             "(there is no CPU fallback)")
 
 
+def tensor_scale_exp(x: torch.Tensor) -> torch.Tensor:
+    """Device int32[1]: the fp8 tensor-scale exponent e of ``x`` (max|x| * 2**e in (224, 448]),
+    computed on the GPU.  Callers with a constant operand (a layer's weight) compute it once and
+    pass it as ``b_exp``."""
+    _check_device_tensor(x, "x")
+    x2 = _rows(x.reshape(-1, x.shape[-1]))
+    e = torch.empty(1, dtype=torch.int32, device=x.device)
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    _lib.check(_lib.lib().cascmm_tensor_exp(x2.data_ptr(), x2.shape[0], x2.shape[1],
+                                            x2.stride(0) if x2.shape[0] > 1 else max(x2.shape[1], 1),
+                                            _DTYPES[x.dtype], e.data_ptr(), stream), "cascmm_tensor_exp")
+    return e
+
+
 def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optional[torch.Tensor],
-             fmt: int, terms: int, products: int, variant: int) -> None:
+             fmt: int, terms: int, products: int, variant: int, b_exp: Optional[torch.Tensor] = None) -> None:
     M, K = a2.shape
     N = b2.shape[1]
     dt = _DTYPES[a2.dtype]
@@ -58,8 +72,11 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
         exps = torch.empty(2, dtype=torch.int32, device=a2.device)
         _lib.check(l.cascmm_tensor_exp(a2.data_ptr(), M, K, a2.stride(0), dt, exps.data_ptr(), stream),
                    "cascmm_tensor_exp(A)")
-        _lib.check(l.cascmm_tensor_exp(b2.data_ptr(), K, N, b2.stride(0), dt, exps.data_ptr() + 4, stream),
-                   "cascmm_tensor_exp(B)")
+        if b_exp is not None:
+            exps[1:2].copy_(b_exp.reshape(1))
+        else:
+            _lib.check(l.cascmm_tensor_exp(b2.data_ptr(), K, N, b2.stride(0), dt, exps.data_ptr() + 4, stream),
+                       "cascmm_tensor_exp(B)")
     st = l.cascmm_gemm_variant(
         a2.data_ptr(), b2.data_ptr(), out2.data_ptr(), bias.data_ptr() if bias is not None else None,
         M, N, K, a2.stride(0) if M > 1 else max(K, 1), b2.stride(0) if K > 1 else max(N, 1),
@@ -158,6 +175,7 @@ def cascaded_lowp_matmul(
     products: str = "tri",
     bias: Optional[torch.Tensor] = None,
     variant: int = -1,
+    b_exp: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     assert a.shape[-1] == b.shape[-2], "Incompatible dimensions"
     # assert a.is_contiguous(), "Matrix A must be contiguous"
@@ -213,7 +231,7 @@ def cascaded_lowp_matmul(
     if N > 1 and out2.stride(1) != 1:
         raise ValueError("out must have unit stride along N")
 
-    _gemm_2d(a2, b, out2, bias, fmt, terms, prod, variant)
+    _gemm_2d(a2, b, out2, bias, fmt, terms, prod, variant, b_exp)
 
     if dump_ptx:
         # the reference writes the kernel's PTX (cascaded_lowp_matmul.py:170-171); there is no

@@ -123,12 +123,29 @@ __global__ void amax_begin_kernel(int32_t* exp_out) { *exp_out = 0; }
 template <int IODT>
 __global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld, int32_t* exp_out) {
   typedef typename IoType<IODT>::T T;
-  const int64_t total = rows * cols;
+  const T* src = (const T*)x;
   unsigned best = 0;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t r = i / cols, c = i - r * cols;
-    const unsigned bits = __builtin_bit_cast(unsigned, IoType<IODT>::load((const T*)x + r * ld + c)) & 0x7FFFFFFFu;
+  auto fold = [&](float v) {
+    const unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7FFFFFFFu;
     best = bits > best ? bits : best;
+  };
+  if (ld == cols) {
+    // contiguous: one flat range, 16-byte loads where the element type and alignment allow
+    const int64_t total = rows * cols;
+    if (IODT == CASCMM_DT_F32 && ((uintptr_t)x % 16) == 0) {
+      const int64_t quads = total / 4;
+      for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += (int64_t)gridDim.x * blockDim.x) {
+        const f32x4 v = ((const f32x4*)x)[i];
+        fold(v[0]); fold(v[1]); fold(v[2]); fold(v[3]);
+      }
+      if (blockIdx.x == 0 && threadIdx.x < total - quads * 4) fold(IoType<IODT>::load(src + quads * 4 + threadIdx.x));
+    } else {
+      for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x)
+        fold(IoType<IODT>::load(src + i));
+    }
+  } else {
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x)
+      for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) fold(IoType<IODT>::load(src + r * ld + c));
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -310,7 +327,7 @@ int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int
   hipLaunchKernelGGL(amax_begin_kernel, dim3(1), dim3(1), 0, s, exp_out);
   const int64_t total = rows * cols;
   if (total > 0) {
-    const unsigned grid = (unsigned)std::min<int64_t>((total + 1023) / 1024, 2048);
+    const unsigned grid = (unsigned)std::min<int64_t>((total + 4095) / 4096, 1024);
     if (dtype == CASCMM_DT_F32)
       hipLaunchKernelGGL((amax_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
     else if (dtype == CASCMM_DT_F16)

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from ..cascaded_lowp_matmul import cascaded_lowp_matmul
+from ..cascaded_lowp_matmul import cascaded_lowp_matmul, tensor_scale_exp
 
 
 class BasedXLLowPLinear(nn.Module):
@@ -19,10 +19,13 @@ class BasedXLLowPLinear(nn.Module):
         self.weight = submodule.weight.detach().T.contiguous().clone()
         self.bias = submodule.bias.detach().clone() if submodule.bias is not None else None
         self.lowp, self.terms, self.products = lowp, terms, products
+        self._weight_exp = None   # fp8: tensor-scale exponent of the weight, found on first use
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.lowp == "fp8" and (self._weight_exp is None or self._weight_exp.device != self.weight.device):
+            self._weight_exp = tensor_scale_exp(self.weight)
         return cascaded_lowp_matmul(x, self.weight, bias=self.bias, lowp=self.lowp, terms=self.terms,
-                                    products=self.products)
+                                    products=self.products, b_exp=self._weight_exp)
 
 
 def patch_linear_layers(model: nn.Module, **cascade_kwargs) -> nn.Module:

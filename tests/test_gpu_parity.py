@@ -331,6 +331,30 @@ def test_lowp_linear_module(gpu_device):
     assert torch.allclose(y.cpu().reshape(-1, 320), want, rtol=0, atol=2e-5)
 
 
+def test_lowp_linear_module_fp8_caches_the_weight_scale(gpu_device):
+    torch.manual_seed(16)
+    lin = torch.nn.Linear(640, 320).to("cuda:0")
+    mod = BasedXLLowPLinear(lin, lowp="fp8", terms=3)
+    x = torch.randn(2, 77, 640, device="cuda:0")
+    y1 = mod(x)
+    assert mod._weight_exp is not None
+    w = lin.weight.detach().cpu().t().contiguous()
+    assert int(mod._weight_exp.cpu()[0]) == oc.tensor_scale_exp(w, "fp8")
+    y2 = mod(x)   # second call reuses the cached exponent
+    assert torch.equal(y1, y2)
+    xa = x.cpu().reshape(-1, 640)
+    exp = oc.fp64_matmul(xa, w) + lin.bias.detach().cpu().double()
+    ref = oc.error_metrics(oc.cascade_matmul_ref(xa, w, "fp8", 3, "tri") + lin.bias.detach().cpu(), exp)
+    got = oc.error_metrics(y1.cpu().reshape(-1, 320), exp)
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+    # grouped launch with fp8 computes the exponents of every problem on the device
+    outs = cascaded_lowp_matmul_grouped([x, x], [mod.weight, mod.weight * 3.0], lowp="fp8", terms=3)
+    assert torch.equal(outs[0].reshape(-1, 320) + mod.bias, y1.reshape(-1, 320)) or \
+        torch.allclose(outs[0].reshape(-1, 320) + mod.bias, y1.reshape(-1, 320), rtol=1e-5, atol=1e-5)
+    got2 = oc.error_metrics(outs[1].cpu().reshape(-1, 320), oc.fp64_matmul(xa, w * 3.0))
+    assert got2["rel_fro"] <= TOL * ref["rel_fro"]
+
+
 def test_grouped_launch_equals_separate_launches(gpu_device):
     """to_q / to_k / to_v style: one activation tensor, several weights, one launch; every
     output must be bit-identical to the single-GEMM launch of the same kernel variant (the
