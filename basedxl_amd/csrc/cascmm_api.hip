@@ -21,6 +21,8 @@ static const std::vector<VariantDesc>& table() {
     v.insert(v.end(), p, p + n);
     p = variants_fp8(&n);
     v.insert(v.end(), p, p + n);
+    p = variants_io16(&n);
+    v.insert(v.end(), p, p + n);
     return v;
   }();
   return t;

@@ -33,7 +33,8 @@ def _gpu(t):
 
 
 def _variants_for(tag):
-    return [(i, n) for i, n in enumerate(_lib.variant_names()) if tag in n]
+    """fp32-operand variants whose name contains tag (the 16-bit-operand ones end in _ioh / _iob)"""
+    return [(i, n) for i, n in enumerate(_lib.variant_names()) if tag in n and "_io" not in n]
 
 
 # ---------------------------------------------------------------------------------------
@@ -136,6 +137,8 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
     names = _lib.variant_names()
     ran = 0
     for vi, name in enumerate(names):
+        if "_io" in name:
+            continue  # 16-bit operands in memory: test_sixteen_bit_operands_*
         fmt = [f for f in ("bf16", "fp16", "fp8") if f + "x" in name][0]
         terms = int(name.split(fmt + "x")[1][0])
         products = "full" if "_full" in name else "tri"
@@ -153,6 +156,58 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
         assert np.array_equal(got.astype(np.int64), want7 if small else want), (name, shape)
         ran += 1
     assert ran >= 5
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(17, 33, 19), (154, 64, 48), (256, 192, 160), (130, 40, 81)])
+def test_sixteen_bit_operands_integer_exact(gpu_device, dtype, shape):
+    """fp16 / bf16 tensors in memory (what the reference feeds its operator): small integers
+    are exact in both, every cascade must return the exact integer product (results below 2**11
+    resp. 2**8 so that the 16-bit output holds them exactly)."""
+    M, K, N = shape
+    hi = 3 if dtype == torch.float16 else 1
+    a, b, want = _int_case(M, K, N, hi, seed=M + N)
+    assert np.abs(want).max() <= (2 ** 11 if dtype == torch.float16 else 2 ** 8)
+    at, bt = _gpu(torch.tensor(a, dtype=dtype)), _gpu(torch.tensor(b, dtype=dtype))
+    tag = "_ioh" if dtype == torch.float16 else "_iob"
+    ran = 0
+    for vi, name in enumerate(_lib.variant_names()):
+        if tag not in name:
+            continue
+        fmt = [f for f in ("bf16", "fp16", "fp8") if f + "x" in name][0]
+        terms = int(name.split(fmt + "x")[1][0])
+        _say("int-exact 16-bit", shape, name)
+        out = cascaded_lowp_matmul(at, bt, lowp=fmt, terms=terms, variant=vi)
+        assert out.dtype == dtype
+        assert np.array_equal(out.float().cpu().numpy().astype(np.int64), want), (name, shape)
+        ran += 1
+    assert ran >= 4
+
+
+@pytest.mark.parametrize("dtype,fmt,terms", [(torch.float16, "fp16", 1), (torch.float16, "bf16", 2),
+                                             (torch.bfloat16, "bf16", 1), (torch.bfloat16, "fp16", 2)])
+def test_sixteen_bit_operands_match_oracle(gpu_device, dtype, fmt, terms):
+    """Random fp16 / bf16 operands: same result as the oracle's wrapper (cascade in fp32, output
+    rounded once to the operand dtype) up to one unit in the last place of the output where the
+    fp32 sums differ in their last bits; bias is added in fp32 before that rounding."""
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(2, 77, 320, generator=g).to(dtype)
+    b = (torch.randn(320, 200, generator=g) * 0.05).to(dtype)
+    bias = torch.randn(200, generator=g).to(dtype)
+    want32 = oc.cascade_matmul_ref(a.reshape(-1, 320).float(), b.float(), fmt, terms, "tri") + bias.float()
+    out = cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp=fmt, terms=terms, bias=_gpu(bias))
+    assert out.dtype == dtype and out.shape == (2, 77, 200)
+    got = out.cpu().reshape(-1, 200)
+    want = want32.to(dtype)
+    ulp = torch.maximum(want.float().abs(), torch.tensor(1e-3)) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7)
+    assert bool(((got.float() - want.float()).abs() <= ulp).all())
+    assert float((got == want).float().mean()) > 0.98
+    # without the bias the oracle's own wrapper is the reference
+    want_nb = oc.cascaded_lowp_matmul_ref(a, b, fmt=fmt, terms=terms)
+    got_nb = cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp=fmt, terms=terms).cpu()
+    assert float((got_nb == want_nb).float().mean()) > 0.98
+    assert bool(((got_nb.float() - want_nb.float()).abs() <= torch.maximum(want_nb.float().abs(), torch.tensor(1e-3))
+                 * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7)).all())
 
 
 def test_fast_variant_is_refused_for_unaligned_k(gpu_device):
