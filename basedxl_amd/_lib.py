@@ -32,6 +32,7 @@ SIGNATURES = {
     "cascmm_gemm_grouped": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p] + _GEMM_ARGS[4:] + [c_int]),
     "cascmm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int]),
     "cascmm_select_variant": (c_int, [c_int64] * 6 + [c_int] * 4),
+    "cascmm_select_variant_grouped": (c_int, [c_int] + [c_int64] * 6 + [c_int] * 4),
     "cascmm_variant_count": (c_int, []),
     "cascmm_variant_name": (c_char_p, [c_int]),
     "cascmm_tensor_exp": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),

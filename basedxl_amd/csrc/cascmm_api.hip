@@ -311,6 +311,15 @@ int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
   return select_variant(q, fast_ok(q, nullptr, nullptr), 1);
 }
 
+int cascmm_select_variant_grouped(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                  int dtype, int fmt, int terms, int products) {
+  if (count < 1 || count > kMaxGroup) return CASCMM_ERR_BAD_SHAPE;
+  const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  return select_variant(q, fast_ok(q, nullptr, nullptr), count);
+}
+
 int cascmm_variant_count(void) { return (int)table().size(); }
 
 const char* cascmm_variant_name(int variant) {

@@ -30,6 +30,9 @@ M, K, N = 4096, 640, 640
 N_PROJ = 4
 TERMS, PRODUCTS_PER_ELEMENT = 2, 3  # bf16 hi/lo, tri product set
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+# HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
+# summary under profiles/ gives the commands and the calibration); keyed by (--group, GEMMs).
+TRAFFIC_BYTES_PER_LAUNCH = {("qkv+o", 3): 2 * 22046.4 * 1024 + 33840.0 * 1024}
 SEED = 1
 
 
@@ -154,18 +157,24 @@ def main():
         with torch.cuda.stream(side):
             step()
         torch.cuda.current_stream().wait_stream(side)
+        # one graph holds `per_graph` consecutive steps, as a UNet forward would hold hundreds of
+        # layers: the cost of starting a graph is not charged to every step
+        per_graph = max(d for d in range(1, 11) if args.steps % d == 0)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            step()
+            for _ in range(per_graph):
+                step()
+    else:
+        per_graph = 1
     run = graph.replay if graph is not None else step
 
-    for _ in range(args.warmup):
+    for _ in range(max(1, args.warmup // per_graph)):
         run()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(args.steps):
+    for _ in range(args.steps // per_graph):
         run()
     e1.record()
     torch.cuda.synchronize()
@@ -175,13 +184,46 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     flops_step = N_PROJ * 2.0 * M * N * K
     value = flops_step / (wall / args.steps) * 1e-12
-    # the GEMM kernel: every launch of a step runs the same kernel on 1, 3 or 4 of the GEMMs;
-    # per-launch figures are quoted per GEMM (launch duration / GEMMs in it), from the events
-    launches_per_step = {"qkv+o": 2, "all": 1, "none": N_PROJ}[args.group]
-    launch_us = ev_ms * 1e3 / (args.steps * N_PROJ)
-    mfma_tflops = PRODUCTS_PER_ELEMENT * 2.0 * M * N * K / (launch_us * 1e-6) * 1e-12
+
+    # The kernels of a step, each timed on its own: a graph that holds that launch REPS times
+    # back to back is replayed between two events on the launch stream (several launches per
+    # graph so that the replay overhead of a graph is not charged to the kernel).  The roofline
+    # object describes the one that takes most of the step.
+    REPS = 10
     l = _lib.lib()
-    vname = l.cascmm_variant_name(l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0)).decode()
+    kinds = {"qkv+o": [("to_q/to_k/to_v grouped", 3, lambda: cascaded_lowp_matmul_grouped(ins[:3], ws[:3], outs=outs[:3])),
+                       ("to_out", 1, lambda: cascaded_lowp_matmul(ins[3], ws[3], out=outs[3]))],
+             "all": [("q/k/v/out grouped", 4, lambda: cascaded_lowp_matmul_grouped(ins, ws, outs=outs))],
+             "none": [("one projection", 1, lambda: cascaded_lowp_matmul(ins[3], ws[3], out=outs[3]))]}[args.group]
+    per_kernel = []
+    for label, gemms, fn in kinds:
+        g1 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g1):
+            for _ in range(REPS):
+                fn()
+        nrep = max(1, args.steps // REPS)
+        for _ in range(max(1, args.warmup // REPS)):
+            g1.replay()
+        torch.cuda.synchronize()
+        k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        k0.record()
+        for _ in range(nrep):
+            g1.replay()
+        k1.record()
+        torch.cuda.synchronize()
+        us = k0.elapsed_time(k1) * 1e3 / (nrep * REPS)
+        vidx = l.cascmm_select_variant_grouped(gemms, M, N, K, K, N, N, 0, 0, 2, 0)
+        per_kernel.append({
+            "launch": label, "gemms": gemms, "kernel": l.cascmm_variant_name(vidx).decode(), "launch_us": round(us, 3),
+            "launches_per_step": (N_PROJ if args.group == "none" else 1),
+            "flops_per_launch": PRODUCTS_PER_ELEMENT * 2.0 * M * N * K * gemms,
+            "algorithmic_bytes_per_launch": 4 * (M * K + gemms * (K * N + M * N)),
+            "mfma_tflops": round(PRODUCTS_PER_ELEMENT * 2.0 * M * N * K * gemms / (us * 1e-6) * 1e-12, 2),
+            "fp32_equiv_tflops": round(2.0 * M * N * K * gemms / (us * 1e-6) * 1e-12, 2),
+        })
+    dom = max(per_kernel, key=lambda r: r["launch_us"] * r["launches_per_step"])
+    launches_per_step = {"qkv+o": 2, "all": 1, "none": N_PROJ}[args.group]
+    vname = dom["kernel"]
 
     result = {
         "metric": "fp32-equiv TFLOP/s, 2-term bf16 cascade, SDXL 64x64-stage self-attn projections (one GPU's patch share)",
@@ -200,7 +242,8 @@ def main():
             "workload": "cfg2: X fp32 [4096,640] ~N(0,1) x W fp32 [640,640] ~N(0,0.02), q/k/v/out = 4 GEMMs per step, "
                         "hi=bf16(x), lo=bf16(x-hi), products hi.hi+hi.lo+lo.hi, fp32 accumulate, fp32 out",
             "M": M, "N": N, "K": K, "gemms_per_step": N_PROJ, "terms": TERMS, "products": "tri",
-            "launch": ("hip graph replay" if graph is not None else "python ctypes") + f", {len(extra) + 1} stream(s), "
+            "launch": (f"hip graph replay ({per_graph} steps per graph)" if graph is not None else "python ctypes")
+                      + f", {len(extra) + 1} stream(s), "
                       + {"qkv+o": "2 launches per step: to_q/to_k/to_v grouped (3 GEMMs, one activation tensor) + to_out",
                          "all": "1 grouped launch per step (4 GEMMs)", "none": "4 launches per step"}[args.group],
             "launches_per_step": launches_per_step,
@@ -209,16 +252,23 @@ def main():
         },
         "roofline": {
             "bound": "mfma",
-            "achieved": round(mfma_tflops, 2),
+            "kernel": dom["kernel"] + " (" + dom["launch"] + ", " + str(dom["gemms"]) + " GEMMs per launch)",
+            "achieved": dom["mfma_tflops"],
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": round(mfma_tflops / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
-            "launch_us": round(launch_us, 3),
-            "launch_us_is": "event time of the timed region / GEMMs executed (a grouped launch runs several GEMMs)",
-            "flops_per_launch": PRODUCTS_PER_ELEMENT * 2 * M * N * K,
-            "fp32_equiv_tflops_per_launch": round(2.0 * M * N * K / (launch_us * 1e-6) * 1e-12, 2),
-            "frac_of_peak_over_terms": round(2.0 * M * N * K / (launch_us * 1e-6) * 1e-12 / (PEAK_BF16_TFLOPS / TERMS), 4),
+            "frac": round(dom["mfma_tflops"] / PEAK_BF16_TFLOPS, 4),
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.group, dom["gemms"])),
+            "traffic_is": "HBM-side bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE "
+                          "(x1.0), factors from a 256 MiB copy in the same runs; see profiles/",
+            "launch_us": dom["launch_us"],
+            "launch_us_is": "HIP events on the launch stream around graph replays of this launch alone (10 launches per "
+                            "graph) / launches",
+            "flops_per_launch": dom["flops_per_launch"],
+            "algorithmic_bytes_per_launch": dom["algorithmic_bytes_per_launch"],
+            "fp32_equiv_tflops": dom["fp32_equiv_tflops"],
+            "frac_of_peak_over_terms": round(dom["fp32_equiv_tflops"] / (PEAK_BF16_TFLOPS / TERMS), 4),
+            "step_time_us_from_events": round(ev_ms * 1e3 / args.steps, 3),
+            "kernels_of_a_step": per_kernel,
         },
         "error": {"kernel_rel_fro": err_k["rel_fro"], "oracle_rel_fro": err_o["rel_fro"],
                   "kernel_max_abs": err_k["max_abs"], "oracle_max_abs": err_o["max_abs"]},

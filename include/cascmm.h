@@ -109,6 +109,10 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
 /* Variant the automatic selection would run for this problem (index), or a negative status. */
 int cascmm_select_variant(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                           int dtype, int fmt, int terms, int products);
+/* Same for a grouped launch of `count` problems (the choice depends on how many tiles the
+ * group has in total). */
+int cascmm_select_variant_grouped(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                                  int64_t ldc, int dtype, int fmt, int terms, int products);
 int cascmm_variant_count(void);
 /* Static string: the device function name of the variant's kernel is a template
  * instantiation whose text contains this name (for filtering rocprof output), or NULL. */
