@@ -31,7 +31,8 @@ extern "C" {
 #define CASCMM_VERSION 100 /* major*10000 + minor*100 + patch */
 
 /* element type of A, B, C and bias as stored in memory (C has the type of A, like
- * `torch.empty((M, N), dtype=a.dtype)` at cascaded_lowp_matmul.py:161) */
+ * `torch.empty((M, N), dtype=a.dtype)` at cascaded_lowp_matmul.py:161).  The fast kernels take
+ * fp32; fp16 / bf16 run on bounds-checked kernels (bf16 or fp16 terms, 1 or 2 of them, tri). */
 enum cascmm_dtype { CASCMM_DT_F32 = 0, CASCMM_DT_F16 = 1, CASCMM_DT_BF16 = 2 };
 
 /* low-precision format of the cascade terms */
@@ -62,9 +63,11 @@ enum cascmm_status {
  *   fmt/terms/products: supported combinations are
  *       bf16: terms 1..3;  fp16: terms 1..3;  fp8: terms 1..3.
  *   tensor_exps: fp8 only -- device pointer to two int32 {e_A, e_B}: the operands are
- *       scaled by 2^e before rounding (see cascmm_tensor_exp); NULL means {0, 0}.
- *   workspace: needed only when cascmm_workspace_bytes(...) > 0 (the split-K path for
- *       skinny shapes); its first bytes must be zero on first use and are left zero.
+ *       scaled by 2^e before rounding (see cascmm_tensor_exp); NULL means {0, 0}.  (Grouped
+ *       launch: 2 * count values, problem i at [2i], [2i + 1].)
+ *   workspace: used only when cascmm_workspace_bytes(...) > 0 (the split-K path for skinny
+ *       shapes: fp32 partial results); 16-byte aligned, contents need no initialisation.  When it
+ *       is NULL or too small, a kernel that needs none is selected instead.
  *   M, N or K equal to 0 is valid (K == 0 writes bias or zeros).
  */
 int cascmm_gemm(const void* A, const void* B, void* C, const void* bias,
@@ -100,7 +103,7 @@ int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, v
                         const int32_t* tensor_exps,
                         void* workspace, size_t workspace_bytes, void* stream, int variant);
 
-/* Bytes of device workspace cascmm_gemm needs for this problem (0 for most shapes).
+/* Bytes of device workspace cascmm_gemm can use for this problem (0 for most shapes).
  * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,
  * cascaded_lowp_matmul.py:155-156); the caller allocates, as it allocates `out` (:161). */
 size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms,
