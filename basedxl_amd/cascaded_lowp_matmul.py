@@ -58,6 +58,94 @@ def tensor_scale_exp(x: torch.Tensor) -> torch.Tensor:
     return e
 
 
+class PreparedWeight:
+    """A constant right operand ``w`` ([K, N]: the ``[in, out]`` weight of
+    basedxl/modules/lowp_linear.py:12) split once on the GPU into the terms of a cascade and
+    kept as MFMA operand slots; ``cascaded_lowp_matmul(a, prepared)`` then splits only ``a``.
+    The arithmetic is the same as with the raw weight (same split, same products)."""
+
+    def __init__(self, w: torch.Tensor, *, lowp: str = "bf16", terms: int = 2):
+        _check_device_tensor(w, "w")
+        if w.dim() != 2 or w.dtype not in _DTYPES:
+            raise ValueError("PreparedWeight needs a 2-D fp32 / fp16 / bf16 tensor")
+        if lowp not in _lib.FMT_BY_NAME:
+            raise ValueError(f"lowp must be one of {sorted(_lib.FMT_BY_NAME)}, got {lowp!r}")
+        self.K, self.N = int(w.shape[0]), int(w.shape[1])
+        self.shape = (self.K, self.N)
+        self.lowp, self.terms, self.fmt = lowp, int(terms), _lib.FMT_BY_NAME[lowp]
+        self.dtype, self.device = w.dtype, w.device
+        w2 = _rows(w)
+        l = _lib.lib()
+        stream = torch.cuda.current_stream(w.device).cuda_stream
+        self.exp = tensor_scale_exp(w2) if self.fmt == _lib.FMT_FP8 else None
+        nbytes = l.cascmm_prepared_bytes(self.K, self.N, self.fmt, self.terms)
+        self.slots = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=w.device)
+        _lib.check(l.cascmm_prepare_weight(w2.data_ptr(), self.K, self.N, w2.stride(0) if self.K > 1 else max(self.N, 1),
+                                           _DTYPES[w.dtype], self.fmt, self.terms,
+                                           self.exp.data_ptr() if self.exp is not None else None,
+                                           self.slots.data_ptr(), self.slots.numel(), stream), "cascmm_prepare_weight")
+
+    def usable_with(self, a2: torch.Tensor) -> bool:
+        """Whether the prepared kernels take this left operand: fp32, K a multiple of 64, rows
+        16-byte aligned (anything else goes through the raw weight)."""
+        return (a2.dtype == torch.float32 and self.K % 64 == 0 and self.N % 4 == 0 and a2.data_ptr() % 16 == 0
+                and (a2.shape[0] <= 1 or a2.stride(0) % 4 == 0))
+
+
+def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, products: str = "tri", variant: int = -1):
+    """``a_list[i]`` ([..., K] fp32) times the prepared weight ``w_list[i]`` in ONE launch (1..8
+    problems of one shape and one cascade); returns the list of results."""
+    import ctypes
+
+    n = len(a_list)
+    if n == 0 or n != len(w_list) or n > 8:
+        raise ValueError("need 1..8 problems, one prepared weight per a")
+    w0 = w_list[0]
+    if products not in _lib.PROD_BY_NAME:
+        raise ValueError(f"products must be 'tri' or 'full', got {products!r}")
+    a2s = []
+    for a, w in zip(a_list, w_list):
+        if not isinstance(w, PreparedWeight):
+            raise TypeError("w_list must hold PreparedWeight objects")
+        assert a.shape[-1] == w.K, "Incompatible dimensions"
+        _check_device_tensor(a, "a")
+        if (w.K, w.N, w.fmt, w.terms) != (w0.K, w0.N, w0.fmt, w0.terms) or a.dtype != torch.float32:
+            raise ValueError("grouped problems must share one shape, cascade and fp32 activations")
+        a2s.append(_rows(a.reshape(-1, w.K)))
+    M, K, N = a2s[0].shape[0], w0.K, w0.N
+    lda = a2s[0].stride(0) if M > 1 else max(K, 1)
+    for a2 in a2s:
+        if a2.shape[0] != M or (M > 1 and a2.stride(0) != lda):
+            raise ValueError("grouped problems must share M and the row stride of a")
+    dev = a_list[0].device
+    if outs is None:
+        outs = [torch.empty((M, N), device=dev, dtype=torch.float32) for _ in range(n)]
+    for o in outs:
+        _check_device_tensor(o, "out")
+        if o.numel() != M * N or not o.is_contiguous() or o.dtype != torch.float32:
+            raise ValueError("every out must be a contiguous fp32 [M, N] tensor")
+    if biases is not None:
+        biases = [None if bb is None else bb.contiguous() for bb in biases]
+    arr = ctypes.c_void_p * n
+    pa = arr(*[t.data_ptr() for t in a2s])
+    pb = arr(*[w.slots.data_ptr() for w in w_list])
+    pc = arr(*[t.data_ptr() for t in outs])
+    pbias = arr(*[(None if bb is None else bb.data_ptr()) for bb in biases]) if biases is not None else None
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    exps = None
+    if w0.fmt == _lib.FMT_FP8:
+        exps = torch.empty(2 * n, dtype=torch.int32, device=dev)
+        for i in range(n):
+            _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _lib.DT_F32, exps.data_ptr() + 8 * i,
+                                                    stream), "cascmm_tensor_exp(A)")
+            exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
+    st = _lib.lib().cascmm_gemm_prepared(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), _lib.DT_F32, w0.fmt, w0.terms,
+                                         _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None,
+                                         stream, variant)
+    _lib.check(st, "cascmm_gemm_prepared")
+    return [o.reshape(*a.shape[:-1], N) for o, a in zip(outs, a_list)]
+
+
 def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optional[torch.Tensor],
              fmt: int, terms: int, products: int, variant: int, b_exp: Optional[torch.Tensor] = None) -> None:
     M, K = a2.shape
@@ -177,6 +265,11 @@ def cascaded_lowp_matmul(
     variant: int = -1,
     b_exp: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
+    if isinstance(b, PreparedWeight):
+        res = out.view(-1, b.N) if out is not None else None
+        return cascaded_lowp_matmul_prepared([a], [b], outs=None if res is None else [res],
+                                             biases=None if bias is None else [bias], products=products,
+                                             variant=variant)[0]
     assert a.shape[-1] == b.shape[-2], "Incompatible dimensions"
     # assert a.is_contiguous(), "Matrix A must be contiguous"
     assert b.is_contiguous(), "Matrix B must be contiguous"

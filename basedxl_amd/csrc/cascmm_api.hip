@@ -23,6 +23,8 @@ static const std::vector<VariantDesc>& table() {
     v.insert(v.end(), p, p + n);
     p = variants_io16(&n);
     v.insert(v.end(), p, p + n);
+    p = variants_bpre(&n);
+    v.insert(v.end(), p, p + n);
     return v;
   }();
   return t;
@@ -34,7 +36,14 @@ static size_t dtype_size(int dt) { return dt == CASCMM_DT_F32 ? 4 : 2; }
 struct Problem {
   int64_t M, N, K, lda, ldb, ldc;
   int dtype, fmt, terms, products;
+  bool bpre = false;  // B is a prepared (already split) weight buffer
 };
+
+// bytes of a prepared weight: planes x ceil(K/8) x N operand slots of 16 bytes
+static int64_t prepared_bytes(int64_t K, int64_t N, int fmt, int terms) {
+  const int planes = fmt == CASCMM_FMT_FP8 ? (terms + 1) / 2 : terms;
+  return (int64_t)planes * ((K + 7) / 8) * N * 16;
+}
 
 static int check_problem(const Problem& q) {
   if (q.dtype != CASCMM_DT_F32 && q.dtype != CASCMM_DT_F16 && q.dtype != CASCMM_DT_BF16) return CASCMM_ERR_BAD_DTYPE;
@@ -56,7 +65,7 @@ static bool fast_ok(const Problem& q, const void* A, const void* B) {
 
 static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   const int full = (q.products == CASCMM_PROD_FULL && q.terms > 1) ? 1 : 0;
-  if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full) return false;
+  if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full || v.bpre != q.bpre) return false;
   if (v.fast && (!fast || q.K % v.BK != 0)) return false;
   if (v.kind == KIND_SPLITK && (q.M > 5 * v.BM || q.K < 4 * v.BK)) return false;  // skinny: few row tiles, deep K
   return true;
@@ -197,6 +206,56 @@ static int launch_split(const void* x, float* out, int64_t n, int terms, int ten
   return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
+// Splits a weight once: thread (kg, n) reads the 8 values B[8 kg .. 8 kg + 7][n] (zero beyond K),
+// splits them like the GEMM kernels do and writes one 16-byte operand slot per plane to
+// out[(plane * K/8 + kg) * N + n].
+template <int IODT, int FMT, int TERMS>
+__global__ __launch_bounds__(256) void prepare_weight_kernel(const void* B, int K, int N, int64_t ldb,
+                                                            const int32_t* tensor_exp, u32x4* out) {
+  typedef typename IoType<IODT>::T T;
+  const int kgs = (K + 7) / 8;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)kgs * N) return;
+  const int kg = (int)(i / N), n = (int)(i - (int64_t)kg * N);
+  float r[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int k = kg * 8 + e;
+    r[e] = k < K ? IoType<IODT>::load((const T*)B + (int64_t)k * ldb + n) : 0.f;
+  }
+  constexpr int PL = Lowp<FMT>::planes(TERMS);
+  u32x4 t[PL];
+  float scale = 1.f;
+  if constexpr (Lowp<FMT>::kTensorScaled) {
+    if (tensor_exp) scale = __builtin_ldexpf(1.f, *tensor_exp);
+  }
+  split8<FMT, TERMS>(r, t, scale);
+#pragma unroll
+  for (int pl = 0; pl < PL; ++pl) out[((int64_t)pl * kgs + kg) * N + n] = t[pl];
+}
+
+template <int IODT, int FMT>
+static int launch_prepare(const void* B, int K, int N, int64_t ldb, int terms, const int32_t* e, u32x4* out, hipStream_t s) {
+  const int64_t total = (int64_t)((K + 7) / 8) * N;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  switch (terms) {
+    case 1: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out); break;
+    case 2: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out); break;
+    case 3: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out); break;
+    default: return CASCMM_ERR_BAD_FORMAT;
+  }
+  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+}
+
+template <int IODT>
+static int launch_prepare_fmt(const void* B, int K, int N, int64_t ldb, int fmt, int terms, const int32_t* e, u32x4* out,
+                              hipStream_t s) {
+  if (fmt == CASCMM_FMT_BF16) return launch_prepare<IODT, CASCMM_FMT_BF16>(B, K, N, ldb, terms, e, out, s);
+  if (fmt == CASCMM_FMT_FP16) return launch_prepare<IODT, CASCMM_FMT_FP16>(B, K, N, ldb, terms, e, out, s);
+  if (fmt == CASCMM_FMT_FP8) return launch_prepare<IODT, CASCMM_FMT_FP8>(B, K, N, ldb, terms, e, out, s);
+  return CASCMM_ERR_BAD_FORMAT;
+}
+
 // One launch for `count` problems of one shape (count == 1: a plain GEMM).
 static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
                      const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
@@ -227,8 +286,14 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   bool fast = true;
   for (int i = 0; i < count; ++i) {
     if (!A[i] || !B[i]) return CASCMM_ERR_NULL_POINTER;
-    if (!aligned_to(A[i], es) || !aligned_to(B[i], es)) return CASCMM_ERR_ALIGNMENT;
-    fast = fast && fast_ok(q, A[i], B[i]);
+    if (!aligned_to(A[i], es) || !aligned_to(B[i], q.bpre ? 16 : es)) return CASCMM_ERR_ALIGNMENT;
+    fast = fast && fast_ok(q, A[i], q.bpre ? nullptr : B[i]);
+  }
+  if (q.bpre) {
+    // prepared weights only have the fast kernels: fp32 A with 16-byte aligned rows, K a multiple
+    // of the kernel's K step (checked per variant), and a buffer the 32-bit offsets can span
+    if (!fast) return CASCMM_ERR_ALIGNMENT;
+    if (prepared_bytes(q.K, q.N, q.fmt, q.terms) > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
   }
 
   const auto& t = table();
@@ -287,6 +352,48 @@ int cascmm_gemm(const void* A, const void* B, void* C, const void* bias, int64_t
                 void* workspace, size_t workspace_bytes, void* stream) {
   return cascmm_gemm_variant(A, B, C, bias, M, N, K, lda, ldb, ldc, dtype, fmt, terms, products, tensor_exps,
                              workspace, workspace_bytes, stream, -1);
+}
+
+size_t cascmm_prepared_bytes(int64_t K, int64_t N, int fmt, int terms) {
+  if (K < 0 || N < 0 || terms < 1 || terms > 3) return 0;
+  if (fmt != CASCMM_FMT_BF16 && fmt != CASCMM_FMT_FP16 && fmt != CASCMM_FMT_FP8) return 0;
+  return (size_t)prepared_bytes(K, N, fmt, terms);
+}
+
+int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                          const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream) {
+  if (K < 0 || N < 0 || ldb < N) return CASCMM_ERR_BAD_SHAPE;
+  if (K > INT32_MAX || N > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (terms < 1 || terms > 3) return CASCMM_ERR_BAD_FORMAT;
+  if (fmt != CASCMM_FMT_BF16 && fmt != CASCMM_FMT_FP16 && fmt != CASCMM_FMT_FP8) return CASCMM_ERR_BAD_FORMAT;
+  if (K == 0 || N == 0) return CASCMM_OK;
+  if (!B || !out) return CASCMM_ERR_NULL_POINTER;
+  if (!aligned_to(out, 16)) return CASCMM_ERR_ALIGNMENT;
+  if (out_bytes < (size_t)prepared_bytes(K, N, fmt, terms)) return CASCMM_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == CASCMM_DT_F32) return launch_prepare_fmt<CASCMM_DT_F32>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s);
+  if (dtype == CASCMM_DT_F16) return launch_prepare_fmt<CASCMM_DT_F16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s);
+  if (dtype == CASCMM_DT_BF16) return launch_prepare_fmt<CASCMM_DT_BF16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s);
+  return CASCMM_ERR_BAD_DTYPE;
+}
+
+int cascmm_gemm_prepared(int count, const void* const* A, const void* const* Bprep, void* const* C,
+                         const void* const* bias, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int dtype,
+                         int fmt, int terms, int products, const int32_t* tensor_exps, void* stream, int variant) {
+  if (!A || !Bprep || !C) return CASCMM_ERR_NULL_POINTER;
+  Problem q{M, N, K, lda, N, ldc, dtype, fmt, terms, products};
+  q.bpre = true;
+  return gemm_impl(count, A, Bprep, C, bias, q, tensor_exps, nullptr, 0, (hipStream_t)stream, variant);
+}
+
+int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int dtype, int fmt,
+                                   int terms, int products) {
+  if (count < 1 || count > kMaxGroup) return CASCMM_ERR_BAD_SHAPE;
+  Problem q{M, N, K, lda, N, ldc, dtype, fmt, terms, products};
+  q.bpre = true;
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  return select_variant(q, fast_ok(q, nullptr, nullptr), count);
 }
 
 size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms, int products) {

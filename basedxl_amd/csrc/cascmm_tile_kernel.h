@@ -51,7 +51,7 @@
 
 namespace cascmm {
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2, int NP_ = 4>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2, int NP_ = 4, bool QUADS_ = true>
 struct Tile {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, WK = WK_, DEPTH = DEPTH_, NP = NP_;
   static constexpr int NCW = WM * WN * WK;   // consumer waves
@@ -63,7 +63,9 @@ struct Tile {
   static constexpr int KSUB = BK / 16;       // MFMA k slices per stage
   // B columns: the first BNQ (whole groups of 128) are loaded four at a time (16-byte loads)
   // and stored permuted in LDS; the remaining BNS columns are loaded one at a time.
-  static constexpr int BNQ = (BN / 128) * 128, BNS = BN - BNQ;
+  // (QUADS_ = false: every column one at a time, which gives units small enough to spread
+  // evenly over eight producer waves.)
+  static constexpr int BNQ = QUADS_ ? (BN / 128) * 128 : 0, BNS = BN - BNQ;
   // a consumer wave must own whole runs of permuted blocks: all four of a group, or two
   static_assert(BNQ == 0 || WTN % 128 == 0 || WTN == 64 || (WN == 1), "wave tile vs permuted B columns");
   static_assert(BNQ == 0 || WN == 1 || BNS == 0, "mixed B column layouts need one consumer wave column");
@@ -132,7 +134,10 @@ __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
   return r;
 }
 
-template <class TL, int IODT, int FMT, int TERMS, bool FULL>
+// BPRE: the right operand comes already split ("prepared", see prepare_weight_kernel in
+// cascmm_api.hip): B[i] points to 16-byte operand slots [plane][K/8][N], the producers copy
+// slots to LDS without touching the VALU.  Fast path only, every column staged singly.
+template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool BPRE = false>
 struct TileGemm {
   typedef Lowp<FMT> LP;
   typedef typename LP::Vec Vec;
@@ -147,6 +152,8 @@ struct TileGemm {
   static constexpr int Q_UNITS = TL::KG * (TL::BNQ / 4);   // 8(k) x 4(n) blocks of B
   static constexpr int B_UNITS = TL::KG * TL::BNS;         // 8(k) x 1(n) columns of B
   static constexpr int D = TL::DEPTH;
+  static_assert(!BPRE || TL::BNQ == 0, "prepared B is staged column by column");
+  static constexpr int BREGS = BPRE ? 4 * PL : 8;            // registers of one B unit in the ring
   static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // quads per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
 
@@ -173,12 +180,12 @@ struct TileGemm {
     static constexpr int A_IT = HAS_A ? (A_UNITS + NTR - 1) / NTR : 0;
     static constexpr int Q_IT = HAS_Q ? (Q_UNITS + NTR - 1) / NTR : 0;
     static constexpr int B_IT = HAS_S ? (B_UNITS + NTR - 1) / NTR : 0;
-    static_assert((A_IT * 2 + Q_IT * 8 + B_IT * 8) * D <= 60, "too many loads in flight for the vmcnt counter");
+    static_assert((A_IT * 2 + Q_IT * 8 + B_IT * (BPRE ? PL : 8)) * D <= 60, "too many loads in flight for the vmcnt counter");
 
     struct Regs {
       float a[A_IT > 0 ? A_IT : 1][8];
       float q[Q_IT > 0 ? Q_IT : 1][8][4];
-      float b[B_IT > 0 ? B_IT : 1][8];
+      float b[B_IT > 0 ? B_IT : 1][BREGS];
     };
 
     struct Ctx {
@@ -189,7 +196,8 @@ struct TileGemm {
       int lds_a[A_IT > 0 ? A_IT : 1];    // slot index inside a term plane set, -1 if this thread has no such unit
       int lds_q[Q_IT > 0 ? Q_IT : 1];    // slot of column 4*quad (the other three follow at +32, +64, +96)
       int lds_b[B_IT > 0 ? B_IT : 1];
-      int ldb_bytes;
+      int ldb_bytes;                     // prepared B: bytes of one k-group row of slots (N * 16)
+      int plane_bytes;                   // prepared B: bytes of one plane (K/8 * N * 16)
       float scale_a, scale_b;            // tensor scales 2^e_A, 2^e_B (fp8), else 1
     };
 
@@ -225,6 +233,15 @@ struct TileGemm {
       c.ra = make_rsrc(A, ((int64_t)(p.M - 1 - m0) * p.lda + p.K) * ES);
       c.rb = make_rsrc(B, ((int64_t)(p.K - 1) * p.ldb + (p.N - n0)) * ES);
       c.ldb_bytes = (int)(p.ldb * ES);
+      c.plane_bytes = 0;
+      if constexpr (BPRE) {
+        // the descriptor covers the whole prepared buffer; the tile's column goes into the
+        // per-lane offsets (the host checked that the buffer is smaller than 2 GiB)
+        const int kgs = (p.K + 7) / 8;
+        c.ldb_bytes = p.N * 16;
+        c.plane_bytes = kgs * c.ldb_bytes;
+        c.rb = make_rsrc(p.B[prob], (int64_t)PL * c.plane_bytes);
+      }
       c.scale_a = c.scale_b = 1.f;
       if constexpr (LP::kTensorScaled) {
         if (p.tensor_exps) {
@@ -256,7 +273,7 @@ struct TileGemm {
         u = u < B_UNITS ? u : B_UNITS - 1;
         const int n = TL::BNQ + u % SW, kg = u / SW;
         const int nc = n < last_col ? n : last_col;
-        c.voff_b[it] = (int)((kg * 8 * p.ldb + nc) * ES);
+        c.voff_b[it] = BPRE ? kg * c.ldb_bytes + (n0 + nc) * 16 : (int)((kg * 8 * p.ldb + nc) * ES);
       }
     }
 
@@ -273,6 +290,10 @@ struct TileGemm {
           r.a[it][4 + e] = v1[e];
         }
       }
+      if constexpr (BPRE) {
+        load_prepared(c, k0, r);
+        return;
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int soff_b = (k0 + e) * c.ldb_bytes;
@@ -285,6 +306,21 @@ struct TileGemm {
 #pragma unroll
         for (int it = 0; it < B_IT; ++it) r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], soff_b, 0);
       }
+    }
+
+    // prepared B: one 16-byte slot per plane and unit
+    static __device__ __forceinline__ void load_prepared_unit(const Ctx& c, int k0, int it, Regs& r) {
+      const int soff = (k0 >> 3) * c.ldb_bytes;
+#pragma unroll
+      for (int pl = 0; pl < PL; ++pl) {
+        const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_b[it] + pl * c.plane_bytes, soff, 0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r.b[it][4 * pl + e] = v[e];
+      }
+    }
+    static __device__ __forceinline__ void load_prepared(const Ctx& c, int k0, Regs& r) {
+#pragma unroll
+      for (int it = 0; it < B_IT; ++it) load_prepared_unit(c, k0, it, r);
     }
 
     // global -> registers (generic: any dtype, any K, element-wise, bounds-checked)
@@ -384,16 +420,27 @@ struct TileGemm {
       }
 #pragma unroll
       for (int it = 0; it < B_IT; ++it) {
-        if (B_UNITS % NTR == 0 || c.lds_b[it] >= 0) {
-          u32x4 t[PL];
-          split8<FMT, TERMS>(r.b[it], t, c.scale_b);
+        if constexpr (BPRE) {
+          if (B_UNITS % NTR == 0 || c.lds_b[it] >= 0) {
 #pragma unroll
-          for (int i = 0; i < PL; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
-        }
-        if (ISSUE) {
+            for (int i = 0; i < PL; ++i) {
+              const f32x4 v = {r.b[it][4 * i], r.b[it][4 * i + 1], r.b[it][4 * i + 2], r.b[it][4 * i + 3]};
+              sb[i * LL::kBTerm + c.lds_b[it]] = __builtin_bit_cast(u32x4, v);
+            }
+          }
+          if (ISSUE) load_prepared_unit(c, k_next, it, r);
+        } else {
+          if (B_UNITS % NTR == 0 || c.lds_b[it] >= 0) {
+            u32x4 t[PL];
+            split8<FMT, TERMS>(r.b[it], t, c.scale_b);
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], (k_next + e) * c.ldb_bytes, 0);
+            for (int i = 0; i < PL; ++i) sb[i * LL::kBTerm + c.lds_b[it]] = t[i];
+          }
+          if (ISSUE) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], (k_next + e) * c.ldb_bytes, 0);
+          }
         }
       }
     }
@@ -404,6 +451,7 @@ struct TileGemm {
     // already in registers while the consumers finish the current one and store its result.
     template <bool FAST>
     static __device__ __forceinline__ void loop(const GroupParams& p, u32x4* lds, int ktiles, int nitems) {
+      static_assert(FAST || !BPRE, "prepared B has no bounds-checked loader");
       const int rtid = threadIdx.x - TL::NCW * kWave - T0;
       const int tiles = p.tiles_m * p.tiles_n;
       const int gsteps = nitems * ktiles;
@@ -724,10 +772,10 @@ struct TileGemm {
   }
 };
 
-template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
+template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST, bool BPRE = false>
 __global__ __launch_bounds__(TL::NT) void cascmm_tile_kernel(const GroupParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char cascmm_smem[];
-  TileGemm<TL, IODT, FMT, TERMS, FULL>::template run<FAST>(p, (u32x4*)cascmm_smem);
+  TileGemm<TL, IODT, FMT, TERMS, FULL, BPRE>::template run<FAST>(p, (u32x4*)cascmm_smem);
 }
 
 }  // namespace cascmm

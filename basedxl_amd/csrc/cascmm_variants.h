@@ -19,11 +19,12 @@ struct VariantDesc {
   bool fast;  // needs fp32 operands, K % BK == 0, 16-byte aligned A rows
   bool grouped;  // one launch may run several same-shape problems and several tiles per workgroup
   int (*launch)(const GroupParams&, hipStream_t);
+  bool bpre = false;  // takes the right operand already split (cascmm_prepare_weight)
 };
 
-template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST>
+template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST, bool BPRE = false>
 int launch_tile(const GroupParams& p, hipStream_t stream) {
-  auto kfn = cascmm_tile_kernel<TL, IODT, FMT, TERMS, FULL, FAST>;
+  auto kfn = cascmm_tile_kernel<TL, IODT, FMT, TERMS, FULL, FAST, BPRE>;
   constexpr int lds = LdsLayout<TL, Lowp<FMT>::planes(TERMS)>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
@@ -122,6 +123,18 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   return CASCMM_OK;
 }
 
+// eight producer waves, every B column loaded singly (all producer threads share A and B evenly)
+#define CASCMM_TILE_VARIANT_PS(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)          \
+  {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>::NT,  \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, Lowp<FMT>::planes(TERMS)>::kBytes, FAST, true,  \
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, IODT, FMT, TERMS, FULL, FAST>}
+
+// right operand already split: every B column staged singly, fp32 A, fast path only
+#define CASCMM_TILE_VARIANT_BPRE(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, FMT, TERMS, FULL)                           \
+  {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>::NT, \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, Lowp<FMT>::planes(TERMS)>::kBytes, true, true,          \
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, CASCMM_DT_F32, FMT, TERMS, FULL, true, true>, true}
+
 // B-direct kernels: fp32 operands, fast path only
 #define CASCMM_BD_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                                \
   {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, 32 * WN, BK, TileBD<BM, WN, BK, DEPTH, NP>::NT, \
@@ -139,5 +152,6 @@ const VariantDesc* variants_bf16(int* n);
 const VariantDesc* variants_fp16(int* n);
 const VariantDesc* variants_fp8(int* n);
 const VariantDesc* variants_io16(int* n);
+const VariantDesc* variants_bpre(int* n);
 
 }  // namespace cascmm

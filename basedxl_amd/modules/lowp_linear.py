@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from ..cascaded_lowp_matmul import cascaded_lowp_matmul, tensor_scale_exp
+from ..cascaded_lowp_matmul import PreparedWeight, cascaded_lowp_matmul, tensor_scale_exp
 
 
 class BasedXLLowPLinear(nn.Module):
@@ -12,7 +12,8 @@ class BasedXLLowPLinear(nn.Module):
     (lowp_linear.py:12) and the forward pass is one cascade GEMM with the bias add fused
     into its store (the reference adds it in a second kernel, lowp_linear.py:17-19)."""
 
-    def __init__(self, submodule: nn.Linear, *, lowp: str = "bf16", terms: int = 2, products: str = "tri"):
+    def __init__(self, submodule: nn.Linear, *, lowp: str = "bf16", terms: int = 2, products: str = "tri",
+                 prepared: bool = False):
         super().__init__()
         self.in_features = submodule.in_features
         self.out_features = submodule.out_features
@@ -20,8 +21,18 @@ class BasedXLLowPLinear(nn.Module):
         self.bias = submodule.bias.detach().clone() if submodule.bias is not None else None
         self.lowp, self.terms, self.products = lowp, terms, products
         self._weight_exp = None   # fp8: tensor-scale exponent of the weight, found on first use
+        # prepared=True: the weight is also kept split (once, on first use on the GPU); inputs
+        # the prepared kernels do not take (not fp32, K not a multiple of 64) use the raw weight
+        self.prepared = prepared
+        self._prepared_weight = None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.prepared and x.is_cuda:
+            if self._prepared_weight is None or self._prepared_weight.device != self.weight.device:
+                self._prepared_weight = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms)
+            x2 = x.reshape(-1, self.in_features)
+            if self._prepared_weight.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous()):
+                return cascaded_lowp_matmul(x, self._prepared_weight, bias=self.bias, products=self.products)
         if self.lowp == "fp8" and (self._weight_exp is None or self._weight_exp.device != self.weight.device):
             self._weight_exp = tensor_scale_exp(self.weight)
         return cascaded_lowp_matmul(x, self.weight, bias=self.bias, lowp=self.lowp, terms=self.terms,

@@ -103,6 +103,34 @@ int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, v
                         const int32_t* tensor_exps,
                         void* workspace, size_t workspace_bytes, void* stream, int variant);
 
+/*
+ * Prepared weights.  A Linear layer's weight is constant, so its split can be done once: the
+ * counterpart of the one-time `W.T.contiguous().clone()` of basedxl/modules/lowp_linear.py:12.
+ * cascmm_prepare_weight writes B[K,N] (leading dimension ldb, element type `dtype`) as MFMA
+ * operand slots -- 16 bytes = 8 consecutive k of one column of one plane, [plane][ceil(K/8)][N];
+ * planes = terms (bf16, fp16) or ceil(terms/2) (fp8) -- into `out` (16-byte aligned, at least
+ * cascmm_prepared_bytes(K, N, fmt, terms) bytes, allocated by the caller).  fp8: *tensor_exp
+ * (device int32, NULL = 0) is the scale exponent applied before the split; pass the same value
+ * as e_B in tensor_exps of the GEMM.
+ * cascmm_gemm_prepared runs `count` (1..8) GEMMs C[i] = A[i] . B[i] (+ bias[i]) of one shape whose
+ * right operands are prepared buffers; arguments as cascmm_gemm_grouped, without ldb and
+ * workspace.  Only the fast kernels exist for it: A must be fp32 with 16-byte aligned rows
+ * (CASCMM_ERR_ALIGNMENT otherwise), K a multiple of 32 or 64 depending on the kernel
+ * (CASCMM_ERR_BAD_FORMAT when no kernel fits), the prepared buffer below 2 GiB
+ * (CASCMM_ERR_TOO_LARGE).  The results equal cascmm_gemm's bit for bit when the same kernel
+ * tile is used (same split, same order of accumulation).
+ */
+size_t cascmm_prepared_bytes(int64_t K, int64_t N, int fmt, int terms);
+int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                          const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream);
+int cascmm_gemm_prepared(int count, const void* const* A, const void* const* Bprep, void* const* C,
+                         const void* const* bias,
+                         int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                         int dtype, int fmt, int terms, int products,
+                         const int32_t* tensor_exps, void* stream, int variant);
+int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                                   int dtype, int fmt, int terms, int products);
+
 /* Bytes of device workspace cascmm_gemm can use for this problem (0 for most shapes).
  * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,
  * cascaded_lowp_matmul.py:155-156); the caller allocates, as it allocates `out` (:161). */

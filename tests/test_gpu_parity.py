@@ -10,7 +10,8 @@ import numpy as np
 import pytest
 import torch
 
-from basedxl_amd import _lib, cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, BasedXLLowPLinear
+from basedxl_amd import (_lib, cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, cascaded_lowp_matmul_prepared,
+                         PreparedWeight, BasedXLLowPLinear)
 from oracle import cascade as oc
 
 pytestmark = pytest.mark.gpu
@@ -34,7 +35,7 @@ def _gpu(t):
 
 def _variants_for(tag):
     """fp32-operand variants whose name contains tag (the 16-bit-operand ones end in _ioh / _iob)"""
-    return [(i, n) for i, n in enumerate(_lib.variant_names()) if tag in n and "_io" not in n]
+    return [(i, n) for i, n in enumerate(_lib.variant_names()) if tag in n and "_io" not in n and "_bpre" not in n]
 
 
 # ---------------------------------------------------------------------------------------
@@ -137,8 +138,8 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
     names = _lib.variant_names()
     ran = 0
     for vi, name in enumerate(names):
-        if "_io" in name:
-            continue  # 16-bit operands in memory: test_sixteen_bit_operands_*
+        if "_io" in name or "_bpre" in name:
+            continue  # 16-bit operands in memory / prepared weights: tested on their own below
         fmt = [f for f in ("bf16", "fp16", "fp8") if f + "x" in name][0]
         terms = int(name.split(fmt + "x")[1][0])
         products = "full" if "_full" in name else "tri"
@@ -212,7 +213,7 @@ def test_sixteen_bit_operands_match_oracle(gpu_device, dtype, fmt, terms):
 
 def test_fast_variant_is_refused_for_unaligned_k(gpu_device):
     a, b = _gpu(torch.randn(32, 20)), _gpu(torch.randn(20, 32))
-    vi = [i for i, n in enumerate(_lib.variant_names()) if "bf16x2_tri" in n and "generic" not in n][0]
+    vi = [i for i, n in enumerate(_lib.variant_names()) if "bf16x2_tri" in n and "generic" not in n and "_bpre" not in n][0]
     with pytest.raises(_lib.CascmmError, match="variant"):
         cascaded_lowp_matmul(a, b, variant=vi)
 
@@ -408,6 +409,87 @@ def test_lowp_linear_module_fp8_caches_the_weight_scale(gpu_device):
         torch.allclose(outs[0].reshape(-1, 320) + mod.bias, y1.reshape(-1, 320), rtol=1e-5, atol=1e-5)
     got2 = oc.error_metrics(outs[1].cpu().reshape(-1, 320), oc.fp64_matmul(xa, w * 3.0))
     assert got2["rel_fro"] <= TOL * ref["rel_fro"]
+
+
+# ---------------------------------------------------------------------------------------
+# prepared (split once) weights
+# ---------------------------------------------------------------------------------------
+def _fmt_of(name):
+    fmt = [f for f in ("bf16", "fp16", "fp8") if f + "x" in name][0]
+    return fmt, int(name.split(fmt + "x")[1][0])
+
+
+@pytest.mark.parametrize("shape", [(154, 64, 48), (256, 192, 160), (300, 128, 200), (96, 128, 384), (257, 64, 164)])
+def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
+    M, K, N = shape
+    a, b, want = _int_case(M, K, N, 100, seed=M + K + N)
+    a7, b7, want7 = _int_case(M, K, N, 7, seed=M + K + N + 1)
+    ran = 0
+    for vi, name in enumerate(_lib.variant_names()):
+        if "_bpre" not in name or K % int(name.split("_")[0].split("x")[2]):
+            continue
+        fmt, terms = _fmt_of(name)
+        _say("int-exact prepared", shape, name)
+        w = PreparedWeight(_gpu(torch.tensor(b, dtype=torch.float32)), lowp=fmt, terms=terms)
+        out = cascaded_lowp_matmul(_gpu(torch.tensor(a, dtype=torch.float32)), w, variant=vi)
+        assert np.array_equal(out.cpu().numpy().astype(np.int64), want), (name, shape)
+        ran += 1
+    assert ran >= 4
+
+
+def test_prepared_weight_equals_raw_weight_bit_for_bit(gpu_device):
+    """Same tile, same consumer layout: the prepared path does the same split and accumulates
+    in the same order as the on-the-fly path, so the bits agree."""
+    names = _lib.variant_names()
+    a, b = oc.make_operands(1000, 640, 640, seed=31, w_std=0.02)
+    ad, bd = _gpu(a), _gpu(b)
+    bias = _gpu(torch.randn(640))
+    w = PreparedWeight(bd)
+    pairs = 0
+    for vi, name in enumerate(names):
+        if not name.endswith("bf16x2_tri_bpre"):
+            continue
+        raw = name[:-len("_bpre")]
+        if raw not in names:
+            continue
+        _say("prepared == raw", name)
+        got = cascaded_lowp_matmul(ad, w, bias=bias, variant=vi)
+        ref = cascaded_lowp_matmul(ad, bd, bias=bias, variant=names.index(raw))
+        assert torch.equal(got, ref), name
+        pairs += 1
+    assert pairs >= 2
+
+
+@pytest.mark.parametrize("fmt,terms", [("bf16", 2), ("bf16", 3), ("fp16", 3), ("fp8", 3)])
+def test_prepared_weights_meet_the_bound(gpu_device, fmt, terms):
+    a, b = oc.make_operands(2048, 1280, 1280, seed=32, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, fmt, terms, "tri"), exp)
+    w = PreparedWeight(_gpu(b), lowp=fmt, terms=terms)
+    got = oc.error_metrics(cascaded_lowp_matmul(_gpu(a), w).cpu(), exp)
+    _say("prepared", fmt, terms, got["rel_fro"], ref["rel_fro"])
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+    # three weights, one activation tensor, one launch
+    ws = [w, PreparedWeight(_gpu(b * 2.0), lowp=fmt, terms=terms), w]
+    outs = cascaded_lowp_matmul_prepared([_gpu(a)] * 3, ws)
+    got2 = oc.error_metrics(outs[1].cpu(), 2.0 * exp)
+    assert got2["rel_fro"] <= TOL * ref["rel_fro"]
+    assert torch.equal(outs[0], outs[2])
+
+
+def test_prepared_weight_rejects_what_its_kernels_cannot_take(gpu_device):
+    w = PreparedWeight(_gpu(torch.randn(40, 64)))      # K = 40: no prepared kernel steps by 8
+    with pytest.raises(_lib.CascmmError):
+        cascaded_lowp_matmul(_gpu(torch.randn(16, 40)), w)
+    lin = torch.nn.Linear(40, 64).to("cuda:0")          # the module falls back to the raw weight
+    mod = BasedXLLowPLinear(lin, prepared=True)
+    x = torch.randn(16, 40, device="cuda:0")
+    assert torch.equal(mod(x), BasedXLLowPLinear(lin)(x))
+    lin = torch.nn.Linear(640, 320).to("cuda:0")
+    x = torch.randn(2, 77, 640, device="cuda:0")
+    y = BasedXLLowPLinear(lin, prepared=True)(x)
+    torch.testing.assert_close(y, BasedXLLowPLinear(lin)(x), rtol=1e-5, atol=1e-5)
+    assert y.shape == (2, 77, 320)
 
 
 def test_grouped_launch_equals_separate_launches(gpu_device):
