@@ -1,0 +1,168 @@
+"""The Linear-layer workload of one SDXL UNet step, as a shape table plus a timing harness.
+
+The reference gets the UNet from diffusers (basedxl/model.py:17-22) and swaps its ``nn.Linear``
+children (basedxl/unet.py:81-87); diffusers and the checkpoint are not available offline, so
+this module carries the layer table itself (SDXL base architecture: channels 320/640/1280,
+transformer depth 2 at 640 channels and 10 at 1280, 5 + 6 Transformer2D blocks, cross-attention
+width 2048, 77 text tokens) and runs every distinct GEMM shape with random weights.  1x1
+convolutions (resnet shortcuts), which the reference does not route (unet.py:85), are listed as
+GEMMs over channels-last pixels and can be included with ``--convs``.
+
+    python -m basedxl_amd.unet_shapes [--half-latent] [--convs] [--cascades bf16x2,fp8x3] [--prepared]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+from dataclasses import dataclass
+from typing import List
+
+
+@dataclass(frozen=True)
+class LinearShape:
+    name: str
+    count: int      # occurrences per UNet step
+    M: int
+    K: int
+    N: int
+    group: int = 1  # GEMMs that share one activation tensor and can share one launch (to_q/k/v)
+    routed_by_reference: bool = True
+
+    @property
+    def flops(self) -> float:
+        return 2.0 * self.M * self.K * self.N * self.count * self.group
+
+
+def sdxl_linear_shapes(batch: int = 2, latent: int = 128, half_latent: bool = False, text_tokens: int = 77,
+                       convs: bool = False) -> List[LinearShape]:
+    """GEMM shapes of one UNet forward.  ``half_latent``: one GPU's share under 2-way patch
+    parallelism (image tokens halved; text tokens and embeddings are not split)."""
+    div = 2 if half_latent else 1
+    t64 = batch * (latent // 2) ** 2 // div      # tokens at the 640-channel stage
+    t32 = batch * (latent // 4) ** 2 // div      # tokens at the 1280-channel stage
+    t128 = batch * latent ** 2 // div
+    txt = batch * text_tokens
+    out: List[LinearShape] = []
+    for d, tok, blocks, t2d in ((640, t64, 10, 5), (1280, t32, 60, 6)):
+        out += [
+            LinearShape(f"attn1.to_q/k/v d={d}", blocks, tok, d, d, group=3),
+            LinearShape(f"attn1.to_out d={d}", blocks, tok, d, d),
+            LinearShape(f"attn2.to_q d={d}", blocks, tok, d, d),
+            LinearShape(f"attn2.to_k/v d={d}", blocks, txt, 2048, d, group=2),
+            LinearShape(f"attn2.to_out d={d}", blocks, tok, d, d),
+            LinearShape(f"ff.geglu_proj d={d}", blocks, tok, d, 8 * d),
+            LinearShape(f"ff.out d={d}", blocks, tok, 4 * d, d),
+            LinearShape(f"transformer.proj_in/out d={d}", 2 * t2d, tok, d, d),
+        ]
+    out += [
+        LinearShape("time_embedding.linear_1", 1, batch, 320, 1280),
+        LinearShape("time_embedding.linear_2 + add_embedding.linear_2", 2, batch, 1280, 1280),
+        LinearShape("add_embedding.linear_1", 1, batch, 2816, 1280),
+        LinearShape("resnet.time_emb_proj -> 320", 5, batch, 1280, 320),
+        LinearShape("resnet.time_emb_proj -> 640", 5, batch, 1280, 640),
+        LinearShape("resnet.time_emb_proj -> 1280", 7, batch, 1280, 1280),
+    ]
+    if convs:
+        c = dict(routed_by_reference=False)
+        out += [
+            LinearShape("conv_shortcut 320->640 @64^2", 1, t64, 320, 640, **c),
+            LinearShape("conv_shortcut 640->1280 @32^2", 1, t32, 640, 1280, **c),
+            LinearShape("conv_shortcut 2560->1280 @32^2", 2, t32, 2560, 1280, **c),
+            LinearShape("conv_shortcut 1920->1280 @32^2", 1, t32, 1920, 1280, **c),
+            LinearShape("conv_shortcut 1920->640 @64^2", 1, t64, 1920, 640, **c),
+            LinearShape("conv_shortcut 1280->640 @64^2", 1, t64, 1280, 640, **c),
+            LinearShape("conv_shortcut 960->640 @64^2", 1, t64, 960, 640, **c),
+            LinearShape("conv_shortcut 960->320 @128^2", 1, t128, 960, 320, **c),
+            LinearShape("conv_shortcut 640->320 @128^2", 2, t128, 640, 320, **c),
+        ]
+    return out
+
+
+def total_flops(shapes: List[LinearShape]) -> float:
+    return sum(s.flops for s in shapes)
+
+
+def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool = False, iters: int = 10,
+                seed: int = 0) -> List[dict]:
+    """Times every shape on cuda:0 (HIP-graph replay of `iters` launches, random fp32 operands:
+    activations N(0,1), weights 0.02 N(0,1)); returns one record per shape."""
+    import torch
+
+    from . import PreparedWeight, cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, cascaded_lowp_matmul_prepared
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    rows = []
+    for s in shapes:
+        a = torch.randn(s.M, s.K, generator=g).to(dev)
+        ws = [(torch.randn(s.K, s.N, generator=g) * 0.02).to(dev) for _ in range(s.group)]
+        outs = [torch.empty(s.M, s.N, device=dev) for _ in range(s.group)]
+        use_prepared = prepared and s.K % 64 == 0 and s.N % 4 == 0
+        if use_prepared:
+            pw = [PreparedWeight(w, lowp=lowp, terms=terms) for w in ws]
+
+            def run():
+                cascaded_lowp_matmul_prepared([a] * s.group, pw, outs=outs)
+        elif s.group > 1:
+            def run():
+                cascaded_lowp_matmul_grouped([a] * s.group, ws, outs=outs, lowp=lowp, terms=terms)
+        else:
+            def run():
+                cascaded_lowp_matmul(a, ws[0], out=outs[0], lowp=lowp, terms=terms)
+        for _ in range(2):
+            run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(iters):
+                run()
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(3):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (3 * iters)
+        rows.append({"name": s.name, "count": s.count, "group": s.group, "M": s.M, "K": s.K, "N": s.N,
+                     "launch_us": round(us, 2), "prepared": use_prepared,
+                     "tflops_fp32_equiv": round(2.0 * s.M * s.K * s.N * s.group / us * 1e-6, 1),
+                     "us_per_step": round(us * s.count, 1)})
+        del a, ws, outs
+    return rows
+
+
+def main(argv=None) -> None:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--batch", type=int, default=2)
+    ap.add_argument("--latent", type=int, default=128)
+    ap.add_argument("--half-latent", action="store_true")
+    ap.add_argument("--convs", action="store_true", help="include the 1x1 shortcut convolutions as GEMMs")
+    ap.add_argument("--cascades", default="bf16x2,fp8x3")
+    ap.add_argument("--prepared", action="store_true", help="split the weights once (PreparedWeight)")
+    ap.add_argument("--json", action="store_true")
+    args = ap.parse_args(argv)
+    shapes = sdxl_linear_shapes(args.batch, args.latent, args.half_latent, convs=args.convs)
+    flops = total_flops(shapes)
+    summary = {"batch": args.batch, "latent": args.latent, "half_latent": args.half_latent, "convs": args.convs,
+               "prepared": args.prepared, "gflop_fp32_equiv_per_step": round(flops * 1e-9, 1), "cascades": {}}
+    for casc in args.cascades.split(","):
+        lowp, terms = casc.split("x")
+        rows = time_shapes(shapes, lowp, int(terms), prepared=args.prepared)
+        total_us = sum(r["us_per_step"] for r in rows)
+        summary["cascades"][casc] = {"linear_ms_per_step": round(total_us * 1e-3, 3),
+                                     "tflops_fp32_equiv": round(flops / total_us * 1e-6, 1), "shapes": rows}
+        if not args.json:
+            print(f"== {casc}{' (prepared weights)' if args.prepared else ''}: {total_us * 1e-3:.3f} ms of Linear work per "
+                  f"UNet step, {flops / total_us * 1e-6:.1f} TFLOP/s fp32-equivalent")
+            for r in rows:
+                print(f"  {r['name']:50s} x{r['count']:3d}  [{r['M']:6d} x {r['K']:5d}] x [{r['K']:5d} x {r['N']:5d}]"
+                      f"{' x' + str(r['group']) if r['group'] > 1 else '   '}  {r['launch_us']:9.2f} us  "
+                      f"{r['tflops_fp32_equiv']:7.1f} TFLOP/s")
+    if args.json:
+        print(json.dumps(summary))
+
+
+if __name__ == "__main__":
+    main()

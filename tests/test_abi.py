@@ -92,3 +92,20 @@ def test_cpu_tensors_are_rejected_without_fallback():
         cascaded_lowp_matmul(torch.randn(4, 4), torch.randn(5, 4))
     with pytest.raises(AssertionError, match="Matrix B must be contiguous"):
         cascaded_lowp_matmul(torch.randn(4, 4), torch.randn(4, 4).t())
+
+
+def test_unet_shape_table_matches_the_architecture():
+    """The SDXL Linear workload: 70 transformer blocks, about 8.6 TFLOP of Linear work per step
+    at batch 2 and a 128x128 latent; the half-latent share halves the image-token GEMMs only."""
+    from basedxl_amd.unet_shapes import sdxl_linear_shapes, total_flops
+
+    full = sdxl_linear_shapes()
+    assert sum(s.count for s in full if s.name.startswith("attn1.to_out")) == 70
+    assert 8.0e12 < total_flops(full) < 9.5e12
+    half = sdxl_linear_shapes(half_latent=True)
+    kv = [s for s in half if s.name.startswith("attn2.to_k/v")]
+    assert all(s.M == 154 and s.K == 2048 for s in kv)
+    assert [s.M for s in half if s.name.startswith("attn1.to_out")] == [4096, 1024]
+    assert 0.5 * total_flops(full) < total_flops(half) < 0.52 * total_flops(full) + total_flops(kv)
+    convs = sdxl_linear_shapes(convs=True)
+    assert sum(s.count for s in convs if not s.routed_by_reference) == 11
