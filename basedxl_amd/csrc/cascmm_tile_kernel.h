@@ -177,8 +177,25 @@ struct TileGemm {
     static constexpr bool HAS_A = ROLE != kQuads, HAS_Q = ROLE != kRest, HAS_S = ROLE != kQuads;
     static constexpr int NTR = ROLE == kAll ? TL::NTP : TL::NTP / 2;    // threads of this role
     static constexpr int T0 = ROLE == kRest ? TL::NTP / 2 : 0;          // first producer thread of it
-    static constexpr int A_IT = HAS_A ? (A_UNITS + NTR - 1) / NTR : 0;
     static constexpr int Q_IT = HAS_Q ? (Q_UNITS + NTR - 1) / NTR : 0;
+    // Weighted deal of the A units: when only the first Q_UNITS threads of the role have an 8x4
+    // block of B (32 elements, as much as four A units), they get four A units fewer than the
+    // other threads, so that every wave stages the same number of elements per K step.
+    static constexpr int NQT = (HAS_A && HAS_Q && Q_UNITS < NTR) ? Q_UNITS : 0;   // threads with a B block
+    static constexpr int A_LO_NUM = A_UNITS - 4 * (NTR - NQT);
+    static constexpr bool WEIGHTED = NQT > 0 && A_LO_NUM >= 0 && A_LO_NUM % NTR == 0 && NQT % kWave == 0;
+    static constexpr int A_LO = WEIGHTED ? A_LO_NUM / NTR : 0, A_HI = A_LO + 4;
+    static constexpr int A_IT = !HAS_A ? 0 : WEIGHTED ? A_HI : (A_UNITS + NTR - 1) / NTR;
+    static constexpr bool A_ALL = !WEIGHTED && A_UNITS % NTR == 0;   // every thread has A_IT valid units
+    // A unit number of (thread, iteration), or a number >= A_UNITS when there is none
+    static __device__ __forceinline__ int a_unit(int rtid, int it) {
+      if constexpr (WEIGHTED) {
+        if (rtid < NQT) return it < A_LO ? it * NQT + rtid : A_UNITS;
+        return NQT * A_LO + it * (NTR - NQT) + (rtid - NQT);
+      } else {
+        return rtid + it * NTR;
+      }
+    }
     static constexpr int B_IT = HAS_S ? (B_UNITS + NTR - 1) / NTR : 0;
     static_assert((A_IT * 2 + Q_IT * 8 + B_IT * (BPRE ? PL : 8)) * D <= 60, "too many loads in flight for the vmcnt counter");
 
@@ -205,7 +222,7 @@ struct TileGemm {
     static __device__ __forceinline__ void init_lds(Ctx& c, int rtid) {
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
-        const int u = rtid + it * NTR;
+        const int u = a_unit(rtid, it);
         const int kg = u % TL::KG, r = u / TL::KG;
         c.lds_a[it] = u < A_UNITS ? kg * LL::kAPlane + (r ^ LL::swz(kg)) : -1;
       }
@@ -252,7 +269,7 @@ struct TileGemm {
       const int last_row = p.M - 1 - m0, last_col = p.N - 1 - n0;
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
-        int u = rtid + it * NTR;
+        int u = a_unit(rtid, it);
         u = u < A_UNITS ? u : A_UNITS - 1;
         const int kg = u % TL::KG, r = u / TL::KG;
         const int rc = r < last_row ? r : last_row;
@@ -282,6 +299,7 @@ struct TileGemm {
       const int soff_a = k0 * ES;
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
+        if (WEIGHTED && c.lds_a[it] < 0) continue;   // (uniform over a wave)
         const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
         const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
 #pragma unroll
@@ -329,7 +347,7 @@ struct TileGemm {
       const IoT* B = (const IoT*)p.B[prob];
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
-        int u = rtid + it * NTR;
+        int u = a_unit(rtid, it);
         u = u < A_UNITS ? u : A_UNITS - 1;
         const int kg = u % TL::KG;
         int row = m0 + u / TL::KG;
@@ -379,13 +397,13 @@ struct TileGemm {
       const int soff_a = k_next * ES;
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
-        if (A_UNITS % NTR == 0 || c.lds_a[it] >= 0) {
+        if (A_ALL || c.lds_a[it] >= 0) {
           u32x4 t[PL];
           split8<FMT, TERMS>(r.a[it], t, c.scale_a);
 #pragma unroll
           for (int i = 0; i < PL; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
         }
-        if (ISSUE) {
+        if (ISSUE && (!WEIGHTED || c.lds_a[it] >= 0)) {
           const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
           const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
 #pragma unroll
