@@ -412,6 +412,34 @@ def test_lowp_linear_module_fp8_caches_the_weight_scale(gpu_device):
 
 
 # ---------------------------------------------------------------------------------------
+# committed fixture (tests/golden/oracle_fixture.json)
+# ---------------------------------------------------------------------------------------
+def test_gpu_split_and_cascades_against_the_committed_fixture(gpu_device):
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "oracle_fixture.json")) as f:
+        fx = json.load(f)
+    x = torch.tensor(fx["split"]["x_bits"], dtype=torch.int32).view(torch.float32)
+    xd = _gpu(x)
+    l = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    for fmt, rec in fx["split"]["terms"].items():
+        out = torch.empty(3, x.numel(), dtype=torch.float32, device=xd.device)
+        assert l.cascmm_split_terms(xd.data_ptr(), out.data_ptr(), x.numel(), _lib.DT_F32, _lib.FMT_BY_NAME[fmt], 3,
+                                    rec["tensor_exp"], stream) == 0
+        got = out.cpu()
+        for i in range(3):
+            want = torch.tensor(rec["bits"][i], dtype=torch.int32).view(torch.float32)
+            both_zero = (got[i] == 0) & (want == 0)
+            assert bool(((got[i].view(torch.int32) == want.view(torch.int32)) | both_zero).all()), (fmt, i)
+    for rec in fx["cascade"]:
+        a, b = oc.make_operands(rec["M"], rec["K"], rec["N"], seed=rec["seed"], w_std=rec["w_std"])
+        out = cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp=rec["fmt"], terms=rec["terms"], products=rec["products"])
+        m = oc.error_metrics(out.cpu(), oc.fp64_matmul(a, b))
+        assert m["rel_fro"] <= TOL * rec["rel_fro"] and m["max_abs"] <= TOL * rec["max_abs"], rec
+
+
+# ---------------------------------------------------------------------------------------
 # prepared (split once) weights
 # ---------------------------------------------------------------------------------------
 def _fmt_of(name):

@@ -165,3 +165,32 @@ def test_metrics_on_a_known_case():
     assert m["rel_fro"] == pytest.approx(np.sqrt(1.25) / np.sqrt(21.0))
     assert len(m["rel_quantiles"]) == 5
     assert oc.fp32_equiv_tflops(1024, 1024, 1024, 1e-3) == pytest.approx(2.147483648)
+
+
+# ---------------------------------------------------------------------------------------
+# drift check against the committed fixture (tests/golden/make_oracle_fixture.py)
+# ---------------------------------------------------------------------------------------
+def _fixture():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "oracle_fixture.json")) as f:
+        return json.load(f)
+
+
+def test_oracle_split_reproduces_the_fixture_bit_for_bit():
+    fx = _fixture()["split"]
+    x = torch.tensor(fx["x_bits"], dtype=torch.int32).view(torch.float32)
+    for fmt, rec in fx["terms"].items():
+        assert oc.tensor_scale_exp(x, fmt) == rec["tensor_exp"]
+        terms, _ = oc.split_terms(x, fmt, 3, tensor_exp=rec["tensor_exp"])
+        for t, want in zip(terms, rec["bits"]):
+            assert t.view(torch.int32).tolist() == want, fmt
+
+
+def test_oracle_cascade_errors_match_the_fixture():
+    for rec in _fixture()["cascade"]:
+        a, b = oc.make_operands(rec["M"], rec["K"], rec["N"], seed=rec["seed"], w_std=rec["w_std"])
+        m = oc.error_metrics(oc.cascade_matmul_ref(a, b, rec["fmt"], rec["terms"], rec["products"]), oc.fp64_matmul(a, b))
+        # the fp32 matmuls inside the oracle may sum in another order on another torch build
+        assert m["rel_fro"] == pytest.approx(rec["rel_fro"], rel=0.02), rec
+        assert m["max_abs"] == pytest.approx(rec["max_abs"], rel=0.25), rec
