@@ -773,92 +773,6 @@ struct TileGemm {
     }
   }
 
-  // ---- fused variant: every wave both stages and multiplies ------------------------------------
-  // The workgroup has only the WM x WN waves (TL::NP must equal their number: the staging units
-  // are dealt to the same threads).  In K step g a wave multiplies LDS stage g&1 while it splits
-  // its share of step g+1 out of its prefetch ring into stage (g+1)&1 and refills the ring slot
-  // with the loads of step g+1+DEPTH; one barrier per step.  One instruction stream per SIMD:
-  // the compiler interleaves the split's VALU work and the LDS / buffer instructions with the
-  // MFMAs, which leave about six issue slots each.  The accumulators sit in the 256 extra
-  // (accumulation) registers a wave has when only four waves occupy the CU.
-  static __device__ __forceinline__ void run_fused(const GroupParams& p, u32x4* lds) {
-    static_assert(TL::WK == 1 && TL::NP == TL::WM * TL::WN, "fused kernel: one role per wave, no K split");
-    typedef Prod<kAll> P;
-    const int tid = threadIdx.x;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave / TL::WN) * TL::WTM, wn0 = (wave % TL::WN) * TL::WTN;
-    const int ktiles = p.K / TL::BK;   // fast path only: K % BK == 0
-    const int tiles = p.tiles_m * p.tiles_n;
-    const int total = p.count * tiles;
-    const int nitems = (total - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    const int gsteps = nitems * ktiles;
-    typename P::Ctx ctx;
-    P::init_lds(ctx, tid);
-    typename P::Regs ring[D];
-    int cur_item = -1;
-    auto target = [&](int g) {
-      const int j = g / ktiles;
-      if (j != cur_item) {
-        cur_item = j;
-        const int item = blockIdx.x + j * gridDim.x;
-        const int prob = item / tiles;
-        int tm, tn;
-        tile_coords(item - prob * tiles, p.tiles_m, p.tiles_n, tm, tn);
-        P::set_tile(ctx, p, prob, tm * TL::BM, tn * TL::BN, tid);
-      }
-      return (g - j * ktiles) * TL::BK;
-    };
-    // stage step gs (held in ring slot r) into its LDS buffer; refill the slot with step gs + D
-    auto produce = [&](int gs, typename P::Regs& r) {
-      if (gs + D < gsteps) {
-        const int k_next = target(gs + D);
-        P::template restage<true>(ctx, lds + (gs & 1) * LL::kStage, r, k_next);
-      } else {
-        P::template restage<false>(ctx, lds + (gs & 1) * LL::kStage, r, 0);
-      }
-    };
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-      if (d < gsteps) P::load_fast(ctx, target(d), ring[d]);
-    produce(0, ring[0]);
-    __syncthreads();
-
-    f32x16 acc[NCLS][TL::MT][TL::NTL];
-    auto clear = [&]() {
-#pragma unroll
-      for (int c = 0; c < NCLS; ++c)
-#pragma unroll
-        for (int mi = 0; mi < TL::MT; ++mi)
-#pragma unroll
-          for (int ni = 0; ni < TL::NTL; ++ni)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[c][mi][ni][e] = 0.f;
-    };
-    clear();
-    // one K step; slot = ring slot of step g + 1 (a compile-time index at every call site)
-    auto step = [&](int g, typename P::Regs& next) {
-      if (g + 1 < gsteps) produce(g + 1, next);
-      compute(lds + (g & 1) * LL::kStage, wm0, wn0, 0, acc);
-      if ((g + 1) % ktiles == 0) {
-        const int item = blockIdx.x + (g / ktiles) * gridDim.x;
-        const int prob = item / tiles;
-        int tm, tn;
-        tile_coords(item - prob * tiles, p.tiles_m, p.tiles_n, tm, tn);
-        finish(p, lds, prob, tm * TL::BM, tn * TL::BN, 0, wave, wm0, wn0, acc);
-        clear();
-      }
-      __syncthreads();
-    };
-    int g = 0;
-    for (; g + D <= gsteps; g += D) {
-#pragma unroll
-      for (int d = 0; d < D; ++d) step(g + d, ring[(d + 1) % D]);
-    }
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-      if (g + d < gsteps) step(g + d, ring[(d + 1) % D]);
-  }
-
   template <bool FAST>
   static __device__ __forceinline__ void run(const GroupParams& p, u32x4* lds) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -880,12 +794,6 @@ template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST, bool BPR
 __global__ __launch_bounds__(TL::NT) void cascmm_tile_kernel(const GroupParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char cascmm_smem[];
   TileGemm<TL, IODT, FMT, TERMS, FULL, BPRE>::template run<FAST>(p, (u32x4*)cascmm_smem);
-}
-
-template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool BPRE = false>
-__global__ __launch_bounds__(TL::NTP) void cascmm_fused_kernel(const GroupParams p) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char cascmm_smem[];
-  TileGemm<TL, IODT, FMT, TERMS, FULL, BPRE>::run_fused(p, (u32x4*)cascmm_smem);
 }
 
 }  // namespace cascmm

@@ -129,33 +129,6 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, Lowp<FMT>::planes(TERMS)>::kBytes, FAST, true,  \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, IODT, FMT, TERMS, FULL, FAST>}
 
-template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool BPRE = false>
-int launch_fused(const GroupParams& p, hipStream_t stream) {
-  auto kfn = cascmm_fused_kernel<TL, IODT, FMT, TERMS, FULL, BPRE>;
-  constexpr int lds = LdsLayout<TL, Lowp<FMT>::planes(TERMS)>::kBytes;
-  static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
-  static std::once_flag once;
-  static hipError_t attr_err = hipSuccess;
-  static int per_cu = 1;
-  std::call_once(once, [&] {
-    if (lds > 64 * 1024) attr_err = hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kfn, TL::NTP, lds) == hipSuccess && n > 0) per_cu = n;
-  });
-  if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
-  const int64_t total = (int64_t)p.count * p.tiles_m * p.tiles_n;
-  const int64_t resident = (int64_t)kNumCUs * per_cu;
-  const unsigned grid = (unsigned)(total < resident ? total : resident);
-  hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NTP), lds, stream, p);
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
-}
-
-// fused kernels (every wave stages and multiplies): WM x WN waves, fp32 operands, fast path
-#define CASCMM_FUSED_VARIANT(NAME, BM, BN, BK, WM, WN, DEPTH, QUADS, FMT, TERMS, FULL)                                    \
-  {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, 1, DEPTH, WM * WN, QUADS>::NTP, \
-   LdsLayout<Tile<BM, BN, BK, WM, WN, 1, DEPTH, WM * WN, QUADS>, Lowp<FMT>::planes(TERMS)>::kBytes, true, true,           \
-   &launch_fused<Tile<BM, BN, BK, WM, WN, 1, DEPTH, WM * WN, QUADS>, CASCMM_DT_F32, FMT, TERMS, FULL>}
-
 // right operand already split: every B column staged singly, fp32 A, fast path only
 #define CASCMM_TILE_VARIANT_BPRE(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, FMT, TERMS, FULL)                           \
   {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>::NT, \
