@@ -71,22 +71,30 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   return true;
 }
 
-// Cost model, fitted on MI355X sweeps.  A 64-deep K step of a full round of 256 tiles costs
-// about (BM*BN + 64*(BM+BN)) / 20000 microseconds: MFMA work grows with BM*BN, while loading,
-// splitting and staging the operands grows with BM+BN and weighs about as much at these tile
-// sizes.  A round that fills only part of the CUs runs its steps faster (less contention for
-// the caches), hence the discount.  Eight producer waves are ~6 % faster than four, the
-// B-direct kernels ~15 % slower.
+// Cost model.  The two-term bf16 kernels, which carry the SDXL workload, are costed from
+// constants measured on MI355X (sweep over the UNet's Linear shapes, HIP-graph replay): a launch
+// takes  rounds x (K/64 x step64 + fixed)  microseconds, where a partly filled last round counts
+// as  tail + (1 - tail) x fill  of a full one, with one `tail` for a launch that has no full
+// round (its tiles run faster: less contention for the caches) and one for later rounds.  Other kernels use the analytic form the constants were first fitted with: a
+// 64-deep K step of a full round costs about (BM*BN + 64*(BM+BN)) / 20000 microseconds (MFMA
+// work grows with BM*BN; loading, splitting and staging grow with BM+BN and weigh about as much
+// at these tile sizes).
+struct TunedCost { const char* name; double step64_us, fixed_us, tail_first, tail_later; };
+static const TunedCost kTuned[] = {
+    {"t64x160x64_w2x1x2_d2_bf16x2_tri", 1.249, 3.33, 1.0, 1.0},
+    {"t256x128x32_w4x1x1_d2_bf16x2_tri", 2.252, 7.55, 0.8, 0.8},
+    {"t128x128x32_w4x1x1_d3_bf16x2_tri", 1.333, 7.97, 1.0, 1.0},
+    {"t128x128x64_w2x1x2_d2_bf16x2_tri", 1.015, 10.30, 1.0, 1.0},
+    {"t64x128x64_w2x1x2_d3_bf16x2_tri", 0.893, 4.56, 1.0, 1.0},
+    {"t64x64x64_w2x2x1_d3_bf16x2_tri", 0.725, 0.59, 1.0, 1.0},
+    {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.076, 3.57, 1.0, 1.0},
+    {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.155, 7.58, 0.8, 0.8},
+};
+
 static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
   const double tiles = (double)count * (double)((q.M + v.BM - 1) / v.BM) * (double)((q.N + v.BN - 1) / v.BN);
   const double full = (double)(int64_t)(tiles / kNumCUs);
   const double rem = tiles - full * kNumCUs;
-  const double rounds = full + (rem > 0 ? 0.55 + 0.45 * rem / kNumCUs : 0.0);
-  double step = ((double)v.BM * v.BN + 64.0 * (v.BM + v.BN)) / 20000.0;
-  const char* name = v.name;
-  if (strstr(name, "_p8_")) step *= 0.94;
-  if (name[0] == 'b' && name[1] == 'd') step *= 1.15;
-  const double ksteps = (double)((q.K + 63) / 64);
   if (v.kind == KIND_SPLITK) {
     // Problems with too few tiles to occupy the chip: splitting K wins whenever the plain tile
     // kernels would leave more than half of the CUs idle; among the split-K variants the
@@ -94,7 +102,24 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
     if ((double)((q.M + 63) / 64) * (double)((q.N + 127) / 128) >= kNumCUs / 2) return 1e9;
     return 1e-6 * (double)(((q.M + v.BM - 1) / v.BM) * v.BM) + 1e-8 * v.BM;
   }
-  return rounds * step * ksteps + (v.fast ? 0.0 : 1e3);
+  for (const TunedCost& t : kTuned) {
+    if (strcmp(t.name, v.name) != 0) continue;
+    const double tail = full == 0 ? t.tail_first : t.tail_later;
+    const double rounds = full + (rem > 0 ? tail + (1.0 - tail) * rem / kNumCUs : 0.0);
+    // tiles that hang over the edge of C take the bounds-checked epilogue and load clamped
+    // columns: measured about a quarter slower (32768 x 640 x 320 on the 128-wide tile)
+    const double edge = (q.N % v.BN != 0 || q.M % v.BM != 0) ? 1.25 : 1.0;
+    return edge * rounds * ((double)q.K / 64.0 * t.step64_us + t.fixed_us);
+  }
+  const double rounds = full + (rem > 0 ? 0.55 + 0.45 * rem / kNumCUs : 0.0);
+  double step = ((double)v.BM * v.BN + 64.0 * (v.BM + v.BN)) / 20000.0;
+  const char* name = v.name;
+  if (strstr(name, "_p8_")) step *= 0.94;
+  const double ksteps = (double)((q.K + 63) / 64);
+  // the plain B-direct kernels were slower than the LDS-tiled ones on every shape measured:
+  // they stay selectable by index only
+  if (name[0] == 'b' && name[1] == 'd') return 1e6 + rounds * step * ksteps;
+  return rounds * (step * ksteps + 5.0) + (v.fast ? 0.0 : 1e3);
 }
 
 // ws_bytes: workspace the caller brought (split-K variants that need more are skipped)
