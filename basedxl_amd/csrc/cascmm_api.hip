@@ -81,17 +81,24 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
 // at these tile sizes).
 struct TunedCost { const char* name; double step64_us, fixed_us, tail_first, tail_later; };
 static const TunedCost kTuned[] = {
-    {"t64x160x64_w2x1x2_d2_bf16x2_tri", 1.249, 3.33, 1.0, 1.0},
-    {"t256x128x32_w4x1x1_d2_bf16x2_tri", 2.252, 7.55, 0.8, 0.8},
-    {"t128x128x32_w4x1x1_d3_bf16x2_tri", 1.333, 7.97, 1.0, 1.0},
-    {"t128x128x64_w2x1x2_d2_bf16x2_tri", 1.015, 10.30, 1.0, 1.0},
-    {"t64x128x64_w2x1x2_d3_bf16x2_tri", 0.893, 4.56, 1.0, 1.0},
-    {"t64x64x64_w2x2x1_d3_bf16x2_tri", 0.725, 0.59, 1.0, 1.0},
-    {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.076, 3.57, 1.0, 1.0},
-    {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.155, 7.58, 0.8, 0.8},
+    {"t64x160x64_w2x1x2_d2_bf16x2_tri", 1.164, 6.93, 1.0, 1.0},
+    {"t256x128x32_w4x1x1_d2_bf16x2_tri", 2.135, 11.48, 0.8, 0.8},
+    {"t128x128x32_w4x1x1_d3_bf16x2_tri", 1.320, 8.11, 1.0, 1.0},
+    {"t128x128x64_w2x1x2_d2_bf16x2_tri", 0.998, 10.46, 1.0, 1.0},
+    {"t64x128x64_w2x1x2_d3_bf16x2_tri", 0.917, 4.19, 1.0, 1.0},
+    {"t64x64x64_w2x2x1_d3_bf16x2_tri", 0.699, 1.98, 1.0, 1.0},
+    {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.128, 4.52, 0.75, 0.75},
+    {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.065, 8.41, 0.9, 0.9},
 };
 
-static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
+constexpr int kMaxTileSplits = 4;
+
+// ws_bytes: workspace the caller brought; *splits_out: K split the cost was computed for (the
+// LDS-tiled two-term bf16 kernels may split K over up to kMaxTileSplits work items per tile when a
+// single problem has too few tiles to occupy the chip and the workspace holds the partials)
+static double variant_cost(const VariantDesc& v, const Problem& q, int count, size_t ws_bytes = 0,
+                           int* splits_out = nullptr) {
+  if (splits_out) *splits_out = 1;
   const double tiles = (double)count * (double)((q.M + v.BM - 1) / v.BM) * (double)((q.N + v.BN - 1) / v.BN);
   const double full = (double)(int64_t)(tiles / kNumCUs);
   const double rem = tiles - full * kNumCUs;
@@ -109,7 +116,23 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
     // tiles that hang over the edge of C take the bounds-checked epilogue and load clamped
     // columns: measured about a quarter slower (32768 x 640 x 320 on the 128-wide tile)
     const double edge = (q.N % v.BN != 0 || q.M % v.BM != 0) ? 1.25 : 1.0;
-    return edge * rounds * ((double)q.K / 64.0 * t.step64_us + t.fixed_us);
+    double best = edge * rounds * ((double)q.K / 64.0 * t.step64_us + t.fixed_us);
+    if (count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0) {
+      const int64_t ksteps = (q.K + v.BK - 1) / v.BK;
+      for (int sp = 2; sp <= kMaxTileSplits; ++sp) {
+        if (ksteps % sp != 0 || ksteps / sp < 4 || tiles * sp > kNumCUs) continue;
+        if (ws_bytes < (size_t)sp * q.M * q.N * sizeof(float)) continue;
+        const double r = t.tail_first + (1.0 - t.tail_first) * tiles * sp / kNumCUs;
+        // the second pass: a launch plus writing and reading the partial results at about 4 TB/s
+        const double reduce_us = 2.0 + (double)(sp + 1) * q.M * q.N * 4.0 / 4.0e6;
+        const double c = edge * r * ((double)q.K / sp / 64.0 * t.step64_us + t.fixed_us) + reduce_us;
+        if (c < best) {
+          best = c;
+          if (splits_out) *splits_out = sp;
+        }
+      }
+    }
+    return best;
   }
   const double rounds = full + (rem > 0 ? 0.55 + 0.45 * rem / kNumCUs : 0.0);
   double step = ((double)v.BM * v.BN + 64.0 * (v.BM + v.BN)) / 20000.0;
@@ -123,18 +146,25 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count) {
 }
 
 // ws_bytes: workspace the caller brought (split-K variants that need more are skipped)
-static int select_variant(const Problem& q, bool fast, int count, size_t ws_bytes = (size_t)-1) {
+static int select_variant(const Problem& q, bool fast, int count, size_t ws_bytes = (size_t)-1,
+                          int* splits_out = nullptr) {
   const auto& t = table();
   int best = -1;
   double best_cost = 0;
+  if (splits_out) *splits_out = 1;
   for (int i = 0; i < (int)t.size(); ++i) {
     if (!variant_matches(t[i], q, fast)) continue;
     if (count > 1 && !t[i].grouped) continue;
     if (t[i].kind == KIND_SPLITK &&
         skinny_workspace_bytes(q.M, q.N, q.K, t[i].BM, t[i].BN, t[i].BK) > ws_bytes)
       continue;
-    const double c = variant_cost(t[i], q, count);
-    if (best < 0 || c < best_cost) { best = i; best_cost = c; }
+    int sp = 1;
+    const double c = variant_cost(t[i], q, count, ws_bytes, &sp);
+    if (best < 0 || c < best_cost) {
+      best = i;
+      best_cost = c;
+      if (splits_out) *splits_out = sp;
+    }
   }
   return best < 0 ? (int)CASCMM_ERR_BAD_FORMAT : best;
 }
@@ -322,10 +352,14 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   }
 
   const auto& t = table();
+  int splits = 1;
   if (variant < 0) {
-    variant = select_variant(q, fast, count, workspace ? workspace_bytes : 0);
+    variant = select_variant(q, fast, count, workspace ? workspace_bytes : 0, &splits);
     if (variant < 0) return variant;
   } else {
+    splits = (variant >> 16) > 0 ? (variant >> 16) : 1;   // forced: kernel index | K splits << 16
+    variant &= 0xFFFF;
+    if (splits > kMaxTileSplits) return CASCMM_ERR_BAD_VARIANT;
     if (variant >= (int)t.size()) return CASCMM_ERR_BAD_VARIANT;
     if (!variant_matches(t[variant], q, fast)) return CASCMM_ERR_BAD_VARIANT;
   }
@@ -341,6 +375,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   p.count = count;
   p.workspace = workspace;
   p.workspace_bytes = workspace_bytes;
+  p.k_splits = v.kind == KIND_TILE ? splits : 1;
   p.tensor_exps = q.fmt == CASCMM_FMT_FP8 ? tensor_exps : nullptr;
   for (int i = 0; i < count; ++i) {
     p.A[i] = A[i]; p.B[i] = B[i]; p.C[i] = C[i]; p.bias[i] = bias ? bias[i] : nullptr;
@@ -431,6 +466,17 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
     if (v.kind != KIND_SPLITK || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
     const size_t n = skinny_workspace_bytes(M, N, K, v.BM, v.BN, v.BK);
     need = n > need ? n : need;
+  }
+  // K split of the LDS-tiled kernels: up to kMaxTileSplits partial results when some kernel
+  // would run the problem with at most half the CUs busy
+  if (dtype == CASCMM_DT_F32 && N % 4 == 0) {
+    for (const auto& v : table()) {
+      if (v.kind != KIND_TILE || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
+      int sp = 1;
+      variant_cost(v, q, 1, (size_t)-1, &sp);
+      const size_t n = sp > 1 ? (size_t)kMaxTileSplits * M * N * sizeof(float) : 0;
+      need = n > need ? n : need;
+    }
   }
   return need;
 }

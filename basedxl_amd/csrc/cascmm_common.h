@@ -226,8 +226,9 @@ struct GroupParams {
   const void* B[kMaxGroup];
   void* C[kMaxGroup];
   const void* bias[kMaxGroup];
-  void* workspace;          // split-K partials (skinny path)
+  void* workspace;          // split-K partials: fp32 [k_splits][M][N]
   size_t workspace_bytes;
+  int k_splits;             // LDS-tiled kernels: work item = (split, problem, tile); 0 or 1 = no split
   const int32_t* tensor_exps;  // fp8: {e_A, e_B} of problem i at [2i], [2i + 1]; NULL = all zero
 };
 

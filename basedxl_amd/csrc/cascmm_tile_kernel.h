@@ -477,12 +477,15 @@ struct TileGemm {
       init_lds(ctx, rtid);
       Regs ring[D];
       // loads for global step g (only ever called with g < gsteps): retarget on a new item
-      int cur_item = -1, prob = 0, m0 = 0, n0 = 0;
+      int cur_item = -1, prob = 0, m0 = 0, n0 = 0, kbase = 0;
       auto target = [&](int g) {
         const int j = g / ktiles;
         if (j != cur_item) {
           cur_item = j;
-          const int item = blockIdx.x + j * gridDim.x;
+          int item = blockIdx.x + j * gridDim.x;
+          const int split = item / (p.count * tiles);   // K split: items are (split, problem, tile)
+          item -= split * (p.count * tiles);
+          kbase = split * ktiles * TL::BK;
           prob = item / tiles;
           int tm, tn;
           tile_coords(item - prob * tiles, p.tiles_m, p.tiles_n, tm, tn);
@@ -490,7 +493,7 @@ struct TileGemm {
           n0 = tn * TL::BN;
           set_tile(ctx, p, prob, m0, n0, rtid);
         }
-        return (g - j * ktiles) * TL::BK;
+        return kbase + (g - j * ktiles) * TL::BK;
       };
       auto issue = [&](int g, Regs& r) {
         const int k0 = target(g);
@@ -589,7 +592,9 @@ struct TileGemm {
     constexpr int kChunkSteps = (AC::kChunkK / TL::BK) > 0 ? (AC::kChunkK / TL::BK) : 1;
     int g = 0;
     for (int j = 0; j < nitems; ++j) {
-      const int item = blockIdx.x + j * gridDim.x;
+      int item = blockIdx.x + j * gridDim.x;
+      const int split = item / (p.count * tiles);
+      item -= split * (p.count * tiles);
       const int prob = item / tiles;
       int tm, tn;
       tile_coords(item - prob * tiles, p.tiles_m, p.tiles_n, tm, tn);
@@ -639,12 +644,12 @@ struct TileGemm {
 #pragma unroll
           for (int ni = 0; ni < TL::NTL; ++ni) acc[0][mi][ni] += master[mi][ni];
       }
-      finish(p, lds, prob, m0, n0, wk, wmn, wm0, wn0, acc);
+      finish(p, lds, prob, split, m0, n0, wk, wmn, wm0, wn0, acc);
     }
   }
 
   // ---- end of an item: fold, reduce the K halves, store -----------------------------------------
-  static __device__ __forceinline__ void finish(const GroupParams& p, u32x4* lds, int prob, int m0, int n0, int wk, int wmn,
+  static __device__ __forceinline__ void finish(const GroupParams& p, u32x4* lds, int prob, int split, int m0, int n0, int wk, int wmn,
                                                 int wm0, int wn0, f32x16 (&acc)[NCLS][TL::MT][TL::NTL]) {
     // fold the scale classes (smallest first), then the cross-wave-group reduction (WK == 2):
     // group 1 parks its tile in LDS, group 0 adds it
@@ -700,18 +705,26 @@ struct TileGemm {
     // epilogue: of every 32x32 tile a lane holds column lane%32 and rows 8*q + 4*(lane/32) + e
     IoT* C = (IoT*)p.C[prob];
     const IoT* bias = (const IoT*)p.bias[prob];
-    const bool interior = (m0 + TL::BM <= p.M) && (n0 + TL::BN <= p.N) && p.ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
+    int64_t ldc = p.ldc;
+    if (p.k_splits > 1) {
+      // K split (fp32 only): this item's partial result goes to the workspace, [split][M][N];
+      // splitk_reduce_kernel adds the splits in order and applies the bias
+      C = (IoT*)p.workspace + ((int64_t)(prob * p.k_splits + split) * p.M) * p.N;
+      bias = nullptr;
+      ldc = p.N;
+    }
+    const bool interior = (m0 + TL::BM <= p.M) && (n0 + TL::BN <= p.N) && ldc * (int64_t)(TL::BM * ES) < 0x7FFFFFFF;
     // Column blocks of this wave that hold permuted columns come in runs of RUN blocks of one
     // 128-column group: block b of the tile (b = wn0/32 + ni), lane l31 <-> column
     // 128*(b/4) + 4*l31 + b%4.
     constexpr int NQ = (TL::BNQ == 0) ? 0 : (TL::WN == 1 ? TL::BNQ / 32 : TL::NTL);
     constexpr int RUN = (NQ % 4 == 0) ? 4 : 2;
     const int b0 = wn0 >> 5;
-    if (IODT == CASCMM_DT_F32 && interior && (p.ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0 &&
+    if (IODT == CASCMM_DT_F32 && interior && (ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0 &&
         (bias == nullptr || (((uintptr_t)bias) & 15) == 0)) {
       // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask
-      const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * p.ldc + n0, 0x7FFFFFFF);
-      const int ldc_bytes = (int)p.ldc * ES;
+      const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * ldc + n0, 0x7FFFFFFF);
+      const int ldc_bytes = (int)ldc * ES;
 #pragma unroll
       for (int r0 = 0; r0 < NQ; r0 += RUN) {
         const int b = b0 + r0;
@@ -762,12 +775,12 @@ struct TileGemm {
 #pragma unroll
       for (int mi = 0; mi < TL::MT; ++mi) {
         const int row0 = m0 + wm0 + mi * 32 + g * 4;
-        IoT* dst = C + (int64_t)row0 * p.ldc + col;
+        IoT* dst = C + (int64_t)row0 * ldc + col;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            if (row0 + q * 8 + e < p.M) IoType<IODT>::store(dst + (int64_t)(q * 8 + e) * p.ldc, res[mi][ni][4 * q + e] + bv);
+            if (row0 + q * 8 + e < p.M) IoType<IODT>::store(dst + (int64_t)(q * 8 + e) * ldc, res[mi][ni][4 * q + e] + bv);
           }
       }
     }
@@ -776,8 +789,9 @@ struct TileGemm {
   template <bool FAST>
   static __device__ __forceinline__ void run(const GroupParams& p, u32x4* lds) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ktiles = (p.K + TL::BK - 1) / TL::BK;
-    const int total = p.count * p.tiles_m * p.tiles_n;
+    const int splits = p.k_splits > 1 ? p.k_splits : 1;
+    const int ktiles = (p.K + TL::BK - 1) / TL::BK / splits;   // K steps of one item (the host picks a divisor)
+    const int total = splits * p.count * p.tiles_m * p.tiles_n;
     const int nitems = (total - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;  // grid <= total
     if (wave < TL::NCW) {
       consumer(p, lds, ktiles, nitems, wave);

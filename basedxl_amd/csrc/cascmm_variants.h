@@ -42,11 +42,27 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kfn, TL::NT, lds) == hipSuccess && n > 0) per_cu = n;
   });
-  const int64_t total = (int64_t)p.count * p.tiles_m * p.tiles_n;
+  const int splits = p.k_splits > 1 ? p.k_splits : 1;
+  if (splits > 1) {
+    // K split: fp32 only, one problem, partial results [split][M][N] in the workspace
+    if (IODT != CASCMM_DT_F32 || p.count != 1 || p.N % 4 != 0 || ((p.K + TL::BK - 1) / TL::BK) % splits != 0)
+      return CASCMM_ERR_BAD_VARIANT;
+    if (!p.workspace || p.workspace_bytes < (size_t)splits * p.M * p.N * sizeof(float)) return CASCMM_ERR_WORKSPACE;
+    if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
+  }
+  const int64_t total = (int64_t)splits * p.count * p.tiles_m * p.tiles_n;
   const int64_t resident = (int64_t)kNumCUs * per_cu;
   const unsigned grid = (unsigned)(total < resident ? total : resident);
   hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+  if (splits > 1) {
+    const int64_t elems = (int64_t)p.M * p.N;
+    const int vec_out = p.ldc % 4 == 0 && (uintptr_t)p.C[0] % 16 == 0 && (uintptr_t)p.bias[0] % 16 == 0;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, stream,
+                       (const float*)p.workspace, splits, p.M, p.N, (const float*)p.bias[0], (float*)p.C[0], p.ldc, vec_out);
+    if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+  }
+  return CASCMM_OK;
 }
 
 #define CASCMM_TILE_VARIANT(NAME, BM, BN, BK, WM, WN, WK, DEPTH, IODT, FMT, TERMS, FULL, FAST)         \

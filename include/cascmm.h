@@ -65,9 +65,9 @@ enum cascmm_status {
  *   tensor_exps: fp8 only -- device pointer to two int32 {e_A, e_B}: the operands are
  *       scaled by 2^e before rounding (see cascmm_tensor_exp); NULL means {0, 0}.  (Grouped
  *       launch: 2 * count values, problem i at [2i], [2i + 1].)
- *   workspace: used only when cascmm_workspace_bytes(...) > 0 (the split-K path for skinny
- *       shapes: fp32 partial results); 16-byte aligned, contents need no initialisation.  When it
- *       is NULL or too small, a kernel that needs none is selected instead.
+ *   workspace: used only when cascmm_workspace_bytes(...) > 0 (K split for problems with too
+ *       few tiles to occupy the chip: fp32 partial results); 16-byte aligned, contents need no
+ *       initialisation.  When it is NULL or too small, a kernel that needs none is selected.
  *   M, N or K equal to 0 is valid (K == 0 writes bias or zeros).
  */
 int cascmm_gemm(const void* A, const void* B, void* C, const void* bias,
@@ -78,7 +78,9 @@ int cascmm_gemm(const void* A, const void* B, void* C, const void* bias,
                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* Same with the kernel variant forced (index into the variant table, see
- * cascmm_variant_count / cascmm_variant_name); variant < 0 selects automatically.
+ * cascmm_variant_count / cascmm_variant_name); variant < 0 selects automatically.  A forced
+ * LDS-tiled kernel runs without K split unless `variant` carries a split count S in 2..4 as
+ * index | S << 16 (needs S * M * N * 4 bytes of workspace and S dividing the kernel's K steps).
  * No counterpart in the reference, whose Triton autotuner picks among its two configs
  * (cascaded_lowp_matmul.py:29-51); used by the tests and the tuning sweep. */
 int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,

@@ -412,6 +412,51 @@ def test_lowp_linear_module_fp8_caches_the_weight_scale(gpu_device):
 
 
 # ---------------------------------------------------------------------------------------
+# K split of the LDS-tiled kernels (problems with too few tiles to occupy the chip)
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(300, 768, 200), (1024, 1280, 1280), (130, 384, 84)])
+def test_tile_k_split_is_exact_and_ordered(gpu_device, shape):
+    """Forced kernel index | splits << 16: integer operands stay exact for every split count that
+    divides the K steps, and the result does not change from launch to launch (the partial
+    results are added in split order by a second kernel)."""
+    M, K, N = shape
+    a, b, want = _int_case(M, K, N, 30, seed=M + K)
+    at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
+    bias = _gpu(torch.arange(N, dtype=torch.float32))
+    ran = 0
+    for vi, name in _variants_for("bf16x2_tri"):
+        if name.startswith(("bd", "skinny")):
+            continue
+        bk = int(name.split("_")[0].split("x")[2])
+        steps = -(-K // bk)
+        if "generic" not in name and K % bk:
+            continue
+        for sp in (2, 3, 4):
+            if steps % sp:
+                continue
+            _say("k-split", shape, name, sp)
+            out = cascaded_lowp_matmul(at, bt, bias=bias, variant=vi | (sp << 16))
+            assert np.array_equal(out.cpu().numpy().astype(np.int64), want + np.arange(N)), (name, sp)
+            assert torch.equal(out, cascaded_lowp_matmul(at, bt, bias=bias, variant=vi | (sp << 16)))
+            ran += 1
+    assert ran >= 6
+
+
+def test_automatic_k_split_meets_the_bound(gpu_device):
+    """1024 x 1280 x 1280 (the 1280-channel stage of the half-latent share): 80-160 tiles; the
+    automatic choice may split K; the error bound and launch-to-launch identity hold either way."""
+    a, b = oc.make_operands(1024, 5120, 1280, seed=41, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exp)
+    ad, bd = _gpu(a), _gpu(b)
+    first = cascaded_lowp_matmul(ad, bd).clone()
+    got = oc.error_metrics(first.cpu(), exp)
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+    for _ in range(3):
+        assert torch.equal(cascaded_lowp_matmul(ad, bd), first)
+
+
+# ---------------------------------------------------------------------------------------
 # committed fixture (tests/golden/oracle_fixture.json)
 # ---------------------------------------------------------------------------------------
 def test_gpu_split_and_cascades_against_the_committed_fixture(gpu_device):
