@@ -6,8 +6,9 @@ The operands are split on the fly into ``terms`` low-precision terms (``lowp``),
 partial products run on MFMA with fp32 accumulation and are summed in registers.
 
 Differences from the reference wrapper, all behind keyword-only arguments with defaults:
-  * ``lowp`` / ``terms`` / ``products`` choose the cascade (default: two bf16 terms, the
-    three products hi.hi + hi.lo + lo.hi);
+  * ``lowp`` / ``terms`` / ``products`` choose the cascade (default for fp32 tensors: two bf16
+    terms, the three products hi.hi + hi.lo + lo.hi; fp16 / bf16 tensors, which the reference
+    runs its UNet in, default to one term of their own format: exact operands, fp32 accumulation);
   * ``bias`` fuses the ``x + bias`` that basedxl/modules/lowp_linear.py:17-19 does separately;
   * there is no torch.matmul fallback for small shapes (:155-156): every shape, including
     M = 154 text tokens, runs the HIP kernels, and a batched ``b`` loops over its batch.
@@ -58,16 +59,29 @@ def tensor_scale_exp(x: torch.Tensor) -> torch.Tensor:
     return e
 
 
+def default_cascade(dtype: torch.dtype) -> Tuple[str, int]:
+    """The cascade used when the caller names none: two bf16 terms for fp32 tensors; fp16 / bf16
+    tensors are multiplied as one term of their own format (exact operands, fp32 accumulation)."""
+    if dtype == torch.float16:
+        return "fp16", 1
+    if dtype == torch.bfloat16:
+        return "bf16", 1
+    return "bf16", 2
+
+
 class PreparedWeight:
     """A constant right operand ``w`` ([K, N]: the ``[in, out]`` weight of
     basedxl/modules/lowp_linear.py:12) split once on the GPU into the terms of a cascade and
     kept as MFMA operand slots; ``cascaded_lowp_matmul(a, prepared)`` then splits only ``a``.
     The arithmetic is the same as with the raw weight (same split, same products)."""
 
-    def __init__(self, w: torch.Tensor, *, lowp: str = "bf16", terms: int = 2):
+    def __init__(self, w: torch.Tensor, *, lowp: Optional[str] = None, terms: Optional[int] = None):
         _check_device_tensor(w, "w")
         if w.dim() != 2 or w.dtype not in _DTYPES:
             raise ValueError("PreparedWeight needs a 2-D fp32 / fp16 / bf16 tensor")
+        d_lowp, d_terms = default_cascade(w.dtype)
+        lowp = d_lowp if lowp is None else lowp
+        terms = d_terms if terms is None else terms
         if lowp not in _lib.FMT_BY_NAME:
             raise ValueError(f"lowp must be one of {sorted(_lib.FMT_BY_NAME)}, got {lowp!r}")
         self.K, self.N = int(w.shape[0]), int(w.shape[1])
@@ -86,10 +100,15 @@ class PreparedWeight:
                                            self.slots.data_ptr(), self.slots.numel(), stream), "cascmm_prepare_weight")
 
     def usable_with(self, a2: torch.Tensor) -> bool:
-        """Whether the prepared kernels take this left operand: fp32, K a multiple of 64, rows
-        16-byte aligned (anything else goes through the raw weight)."""
-        return (a2.dtype == torch.float32 and self.K % 64 == 0 and self.N % 4 == 0 and a2.data_ptr() % 16 == 0
-                and (a2.shape[0] <= 1 or a2.stride(0) % 4 == 0))
+        """Whether the prepared kernels take this left operand: fp32 (or fp16 / bf16 tensors with a
+        weight of the same dtype kept as one term of that format), K a multiple of 64, rows 16-byte
+        aligned (anything else goes through the raw weight)."""
+        if self.K % 64 != 0 or self.N % 4 != 0 or a2.data_ptr() % 16 != 0:
+            return False
+        if a2.dtype == torch.float32:
+            return a2.shape[0] <= 1 or a2.stride(0) % 4 == 0
+        return (a2.dtype == self.dtype and self.terms == 1 and default_cascade(a2.dtype)[0] == self.lowp
+                and (a2.shape[0] <= 1 or a2.stride(0) % 8 == 0))
 
 
 def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, products: str = "tri", variant: int = -1):
@@ -109,8 +128,10 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
             raise TypeError("w_list must hold PreparedWeight objects")
         assert a.shape[-1] == w.K, "Incompatible dimensions"
         _check_device_tensor(a, "a")
-        if (w.K, w.N, w.fmt, w.terms) != (w0.K, w0.N, w0.fmt, w0.terms) or a.dtype != torch.float32:
-            raise ValueError("grouped problems must share one shape, cascade and fp32 activations")
+        if (w.K, w.N, w.fmt, w.terms) != (w0.K, w0.N, w0.fmt, w0.terms) or a.dtype != a_list[0].dtype:
+            raise ValueError("grouped problems must share one shape, cascade and activation dtype")
+        if a.dtype not in _DTYPES:
+            raise TypeError(f"unsupported dtype {a.dtype}")
         a2s.append(_rows(a.reshape(-1, w.K)))
     M, K, N = a2s[0].shape[0], w0.K, w0.N
     lda = a2s[0].stride(0) if M > 1 else max(K, 1)
@@ -118,12 +139,13 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
         if a2.shape[0] != M or (M > 1 and a2.stride(0) != lda):
             raise ValueError("grouped problems must share M and the row stride of a")
     dev = a_list[0].device
+    adt = a_list[0].dtype
     if outs is None:
-        outs = [torch.empty((M, N), device=dev, dtype=torch.float32) for _ in range(n)]
+        outs = [torch.empty((M, N), device=dev, dtype=adt) for _ in range(n)]
     for o in outs:
         _check_device_tensor(o, "out")
-        if o.numel() != M * N or not o.is_contiguous() or o.dtype != torch.float32:
-            raise ValueError("every out must be a contiguous fp32 [M, N] tensor")
+        if o.numel() != M * N or not o.is_contiguous() or o.dtype != adt:
+            raise ValueError("every out must be a contiguous [M, N] tensor of the dtype of a")
     if biases is not None:
         biases = [None if bb is None else bb.contiguous() for bb in biases]
     arr = ctypes.c_void_p * n
@@ -136,10 +158,10 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
     if w0.fmt == _lib.FMT_FP8:
         exps = torch.empty(2 * n, dtype=torch.int32, device=dev)
         for i in range(n):
-            _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _lib.DT_F32, exps.data_ptr() + 8 * i,
+            _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _DTYPES[adt], exps.data_ptr() + 8 * i,
                                                     stream), "cascmm_tensor_exp(A)")
             exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
-    st = _lib.lib().cascmm_gemm_prepared(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), _lib.DT_F32, w0.fmt, w0.terms,
+    st = _lib.lib().cascmm_gemm_prepared(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), _DTYPES[adt], w0.fmt, w0.terms,
                                          _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None,
                                          stream, variant)
     _lib.check(st, "cascmm_gemm_prepared")
@@ -176,7 +198,8 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
     _lib.check(st, "cascmm_gemm")
 
 
-def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp: str = "bf16", terms: int = 2,
+def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp: Optional[str] = None,
+                                 terms: Optional[int] = None,
                                  products: str = "tri", variant: int = -1):
     """Several independent cascade GEMMs of one shape in ONE kernel launch.
 
@@ -191,6 +214,9 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
     n = len(a_list)
     if n == 0 or n != len(b_list) or n > 8:
         raise ValueError("need 1..8 problems, one b per a")
+    d_lowp, d_terms = default_cascade(a_list[0].dtype)
+    lowp = d_lowp if lowp is None else lowp
+    terms = d_terms if terms is None else terms
     if lowp not in _lib.FMT_BY_NAME or products not in _lib.PROD_BY_NAME:
         raise ValueError("bad lowp / products")
     fmt, prod = _lib.FMT_BY_NAME[lowp], _lib.PROD_BY_NAME[products]
@@ -258,13 +284,17 @@ def cascaded_lowp_matmul(
     *,
     out: Optional[torch.Tensor] = None,
     dump_ptx: bool = False,
-    lowp: str = "bf16",
-    terms: int = 2,
+    lowp: Optional[str] = None,
+    terms: Optional[int] = None,
     products: str = "tri",
     bias: Optional[torch.Tensor] = None,
     variant: int = -1,
     b_exp: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
+    if lowp is None or terms is None:
+        d_lowp, d_terms = default_cascade(a.dtype)
+        lowp = d_lowp if lowp is None else lowp
+        terms = d_terms if terms is None else terms
     if isinstance(b, PreparedWeight):
         res = out.view(-1, b.N) if out is not None else None
         return cascaded_lowp_matmul_prepared([a], [b], outs=None if res is None else [res],

@@ -58,6 +58,12 @@ static int check_problem(const Problem& q) {
 
 // what the fast (buffer-load, 16-byte accesses, no K tail) kernels need apart from K % BK == 0
 static bool fast_ok(const Problem& q, const void* A, const void* B) {
+  if (q.dtype != CASCMM_DT_F32) {
+    // 16-bit operands: only with a prepared right operand, as one term of their own format
+    return q.bpre && q.terms == 1 &&
+           ((q.dtype == CASCMM_DT_F16 && q.fmt == CASCMM_FMT_FP16) || (q.dtype == CASCMM_DT_BF16 && q.fmt == CASCMM_FMT_BF16)) &&
+           q.lda % 8 == 0 && (A == nullptr || aligned_to(A, 16)) && q.lda * 2 * 512 < INT32_MAX;
+  }
   return q.dtype == CASCMM_DT_F32 && q.lda % 4 == 0 && (A == nullptr || aligned_to(A, 16)) &&
          q.ldb % 4 == 0 && q.N % 4 == 0 && (B == nullptr || aligned_to(B, 16)) &&
          q.lda * 4 * 512 < INT32_MAX && q.ldb * 4 * 136 < INT32_MAX;  // 32-bit byte offsets inside a tile
@@ -311,6 +317,21 @@ static int launch_prepare_fmt(const void* B, int K, int N, int64_t ldb, int fmt,
   return CASCMM_ERR_BAD_FORMAT;
 }
 
+// 16-bit tensors multiplied as one term of their own format can use the prepared-operand kernels
+// when the caller brought room for the re-laid B
+static bool onthefly_prepare_ok(const Problem& q, int count, const void* const* A, const void* const* B,
+                                const void* workspace, size_t workspace_bytes) {
+  if (q.bpre || count != 1 || q.dtype == CASCMM_DT_F32 || q.terms != 1 || q.K % 64 != 0 || !A[0] || !B[0]) return false;
+  if (!((q.dtype == CASCMM_DT_F16 && q.fmt == CASCMM_FMT_FP16) || (q.dtype == CASCMM_DT_BF16 && q.fmt == CASCMM_FMT_BF16)))
+    return false;
+  if (q.lda % 8 != 0 || !aligned_to(A[0], 16) || !aligned_to(B[0], 2)) return false;
+  const int64_t need = prepared_bytes(q.K, q.N, q.fmt, 1);
+  return workspace && aligned_to(workspace, 16) && need <= INT32_MAX && workspace_bytes >= (size_t)need;
+}
+
+extern "C" int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                                     const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream);
+
 // One launch for `count` problems of one shape (count == 1: a plain GEMM).
 static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
                      const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
@@ -337,6 +358,18 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
         hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
     }
     return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  }
+  if (onthefly_prepare_ok(q, count, A, B, workspace, workspace_bytes)) {
+    // fp16 x fp16 (bf16 x bf16) tensors as one term: re-lay B as operand slots in the workspace
+    // (one pass over B), then the copy-only kernels
+    st = cascmm_prepare_weight(B[0], q.K, q.N, q.ldb, q.dtype, q.fmt, 1, nullptr, workspace, workspace_bytes, (void*)stream);
+    if (st != CASCMM_OK) return st;
+    Problem qp = q;
+    qp.bpre = true;
+    qp.ldb = q.N;
+    const void* bp = workspace;
+    const int r = gemm_impl(1, A, &bp, C, bias, qp, tensor_exps, nullptr, 0, stream, variant < 0 ? -1 : variant);
+    if (r != CASCMM_ERR_BAD_FORMAT && r != CASCMM_ERR_BAD_VARIANT) return r;
   }
   bool fast = true;
   for (int i = 0; i < count; ++i) {
@@ -466,6 +499,12 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
     if (v.kind != KIND_SPLITK || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
     const size_t n = skinny_workspace_bytes(M, N, K, v.BM, v.BN, v.BK);
     need = n > need ? n : need;
+  }
+  // 16-bit tensors as one term of their own format: room for B re-laid as operand slots
+  if (((dtype == CASCMM_DT_F16 && fmt == CASCMM_FMT_FP16) || (dtype == CASCMM_DT_BF16 && fmt == CASCMM_FMT_BF16)) &&
+      terms == 1 && K % 64 == 0) {
+    const int64_t n = prepared_bytes(K, N, fmt, 1);
+    if (n <= INT32_MAX && (size_t)n > need) need = (size_t)n;
   }
   // K split of the LDS-tiled kernels: up to kMaxTileSplits partial results when some kernel
   // would run the problem with at most half the CUs busy

@@ -19,6 +19,15 @@ static const VariantDesc kTable[] = {
     CASCMM_TILE_VARIANT_BPRE("t128x128x32_w4x2x1_d2_bf16x3_tri_bpre", 128, 128, 32, 4, 2, 1, 2, 4, BF, 3, false),
     CASCMM_TILE_VARIANT_BPRE("t128x128x32_w4x2x1_d2_fp16x3_tri_bpre", 128, 128, 32, 4, 2, 1, 2, 4, FP, 3, false),
     CASCMM_TILE_VARIANT_BPRE("t128x128x32_w4x2x1_d2_fp8x3_tri_bpre", 128, 128, 32, 4, 2, 1, 2, 4, F8, 3, false),
+    // 16-bit tensors (what the reference runs its UNet in): a plain fp16 / bf16 GEMM with fp32 accumulation
+    CASCMM_TILE_VARIANT_BPRE16("t256x128x64_w4x1x1_d2_fp16x1_bpre_ioh", 256, 128, 64, 4, 1, 1, 2, 4, CASCMM_DT_F16, FP),
+    CASCMM_TILE_VARIANT_BPRE16("t128x128x64_w2x2x1_d3_fp16x1_bpre_ioh", 128, 128, 64, 2, 2, 1, 3, 4, CASCMM_DT_F16, FP),
+    CASCMM_TILE_VARIANT_BPRE16("t64x160x64_w2x1x2_d3_fp16x1_bpre_ioh", 64, 160, 64, 2, 1, 2, 3, 4, CASCMM_DT_F16, FP),
+    CASCMM_TILE_VARIANT_BPRE16("t64x64x64_w2x2x1_d3_fp16x1_bpre_ioh", 64, 64, 64, 2, 2, 1, 3, 4, CASCMM_DT_F16, FP),
+    CASCMM_TILE_VARIANT_BPRE16("t256x128x64_w4x1x1_d2_bf16x1_bpre_iob", 256, 128, 64, 4, 1, 1, 2, 4, CASCMM_DT_BF16, BF),
+    CASCMM_TILE_VARIANT_BPRE16("t128x128x64_w2x2x1_d3_bf16x1_bpre_iob", 128, 128, 64, 2, 2, 1, 3, 4, CASCMM_DT_BF16, BF),
+    CASCMM_TILE_VARIANT_BPRE16("t64x160x64_w2x1x2_d3_bf16x1_bpre_iob", 64, 160, 64, 2, 1, 2, 3, 4, CASCMM_DT_BF16, BF),
+    CASCMM_TILE_VARIANT_BPRE16("t64x64x64_w2x2x1_d3_bf16x1_bpre_iob", 64, 64, 64, 2, 2, 1, 3, 4, CASCMM_DT_BF16, BF),
 };
 
 const VariantDesc* variants_bpre(int* n) {

@@ -122,6 +122,7 @@ __device__ void llvm_raw_buffer_store_f32(float v, i32x4 rsrc, int voffset, int 
 __device__ void llvm_raw_buffer_store_v4f32(f32x4 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v4f32");
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 __device__ void llvm_raw_buffer_store_v2f32(f32x2 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v2f32");
+__device__ void llvm_raw_buffer_store_i16(short v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.i16");
 
 // gfx9-family raw buffer descriptor: 48-bit base, stride 0, byte count, 32-bit data format
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
@@ -153,6 +154,9 @@ struct TileGemm {
   static constexpr int B_UNITS = TL::KG * TL::BNS;         // 8(k) x 1(n) columns of B
   static constexpr int D = TL::DEPTH;
   static_assert(!BPRE || TL::BNQ == 0, "prepared B is staged column by column");
+  // 16-bit operands on the fast path: A is fp16 (bf16) data multiplied as one fp16 (bf16) term, so
+  // 8 consecutive elements of a row ARE the operand slot: the producers copy 16 bytes, no split
+  static constexpr bool RAW16 = IODT != CASCMM_DT_F32;
   static constexpr int BREGS = BPRE ? 4 * PL : 8;            // registers of one B unit in the ring
   static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // quads per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
@@ -301,11 +305,12 @@ struct TileGemm {
       for (int it = 0; it < A_IT; ++it) {
         if (WEIGHTED && c.lds_a[it] < 0) continue;   // (uniform over a wave)
         const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
-        const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          r.a[it][e] = v0[e];
-          r.a[it][4 + e] = v1[e];
+        for (int e = 0; e < 4; ++e) r.a[it][e] = v0[e];
+        if constexpr (!RAW16) {
+          const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r.a[it][4 + e] = v1[e];
         }
       }
       if constexpr (BPRE) {
@@ -391,25 +396,31 @@ struct TileGemm {
     // that unit's registers for K step k_next (ISSUE).  Spreading the loads between the VALU
     // batches keeps the texture-address unit busy while the splits run; issued in one burst
     // they would stall the wave on the full address FIFO with no VALU work to overlap.
-    template <bool ISSUE>
+    template <bool ISSUE, bool RAW = false>
     static __device__ __forceinline__ void restage(const Ctx& c, u32x4* stage, Regs& r, int k_next) {
       u32x4* sb = stage + PL * LL::kATerm;
       const int soff_a = k_next * ES;
 #pragma unroll
       for (int it = 0; it < A_IT; ++it) {
         if (A_ALL || c.lds_a[it] >= 0) {
-          u32x4 t[PL];
-          split8<FMT, TERMS>(r.a[it], t, c.scale_a);
+          if constexpr (RAW) {
+            const f32x4 v = {r.a[it][0], r.a[it][1], r.a[it][2], r.a[it][3]};
+            stage[c.lds_a[it]] = __builtin_bit_cast(u32x4, v);
+          } else {
+            u32x4 t[PL];
+            split8<FMT, TERMS>(r.a[it], t, c.scale_a);
 #pragma unroll
-          for (int i = 0; i < PL; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+            for (int i = 0; i < PL; ++i) stage[i * LL::kATerm + c.lds_a[it]] = t[i];
+          }
         }
         if (ISSUE && (!WEIGHTED || c.lds_a[it] >= 0)) {
           const f32x4 v0 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it], soff_a, 0);
-          const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            r.a[it][e] = v0[e];
-            r.a[it][4 + e] = v1[e];
+          for (int e = 0; e < 4; ++e) r.a[it][e] = v0[e];
+          if constexpr (!RAW) {
+            const f32x4 v1 = llvm_raw_buffer_load_v4f32(c.ra, c.voff_a[it] + 16, soff_a, 0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.a[it][4 + e] = v1[e];
           }
         }
       }
@@ -470,6 +481,10 @@ struct TileGemm {
     template <bool FAST>
     static __device__ __forceinline__ void loop(const GroupParams& p, u32x4* lds, int ktiles, int nitems) {
       static_assert(FAST || !BPRE, "prepared B has no bounds-checked loader");
+      constexpr bool RAW = FAST && RAW16;
+      static_assert(!RAW || (BPRE && TERMS == 1 &&
+                             ((IODT == CASCMM_DT_F16 && FMT == CASCMM_FMT_FP16) || (IODT == CASCMM_DT_BF16 && FMT == CASCMM_FMT_BF16))),
+                    "16-bit operands on the fast path: one term of their own format, prepared B");
       const int rtid = threadIdx.x - TL::NCW * kWave - T0;
       const int tiles = p.tiles_m * p.tiles_n;
       const int gsteps = nitems * ktiles;
@@ -518,9 +533,9 @@ struct TileGemm {
         for (int d = 0; d < D; ++d) {
           if (FAST) {
             const int k_next = target(g + d + D);
-            restage<true>(ctx, lds + ((g + d) & 1) * LL::kStage, ring[d], k_next);
+            restage<true, RAW>(ctx, lds + ((g + d) & 1) * LL::kStage, ring[d], k_next);
           } else {
-            restage<false>(ctx, lds + ((g + d) & 1) * LL::kStage, ring[d], 0);
+            restage<false, RAW>(ctx, lds + ((g + d) & 1) * LL::kStage, ring[d], 0);
             issue(g + d + D, ring[d]);
           }
           __syncthreads();
@@ -533,9 +548,9 @@ struct TileGemm {
         if (g + dd < gsteps) {
           if (FAST && g + dd + D < gsteps) {
             const int k_next = target(g + dd + D);
-            restage<true>(ctx, lds + ((g + dd) & 1) * LL::kStage, ring[d], k_next);
+            restage<true, RAW>(ctx, lds + ((g + dd) & 1) * LL::kStage, ring[d], k_next);
           } else {
-            restage<false>(ctx, lds + ((g + dd) & 1) * LL::kStage, ring[d], 0);
+            restage<false, RAW>(ctx, lds + ((g + dd) & 1) * LL::kStage, ring[d], 0);
             if (g + dd + D < gsteps) issue(g + dd + D, ring[d]);
           }
           __syncthreads();
@@ -763,6 +778,27 @@ struct TileGemm {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               llvm_raw_buffer_store_f32(res[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+      }
+      return;
+    }
+    if constexpr (IODT != CASCMM_DT_F32 && NQ == 0) if (interior) {
+      // 16-bit output, whole tile inside C: 2-byte buffer stores, the row as a scalar offset
+      const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * ldc + n0, 0x7FFFFFFF);
+      const int ldc_bytes = (int)ldc * ES;
+#pragma unroll
+      for (int ni = 0; ni < TL::NTL; ++ni) {
+        const int col = wn0 + ni * 32 + l31;
+        const int voff = g * 4 * ldc_bytes + col * ES;
+        const float bv = bias ? IoType<IODT>::load(bias + n0 + col) : 0.f;
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const IoT h = (IoT)(res[mi][ni][4 * q + e] + bv);
+              llvm_raw_buffer_store_i16(__builtin_bit_cast(short, h), rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+            }
       }
       return;
     }

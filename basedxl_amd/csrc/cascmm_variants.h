@@ -151,6 +151,13 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, Lowp<FMT>::planes(TERMS)>::kBytes, true, true,          \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, CASCMM_DT_F32, FMT, TERMS, FULL, true, true>, true}
 
+// fp16 (bf16) operands in memory multiplied as one fp16 (bf16) term, right operand prepared: the
+// producers only copy
+#define CASCMM_TILE_VARIANT_BPRE16(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT)                       \
+  {NAME, KIND_TILE, IODT, FMT, 1, false, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>::NT,     \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, 1>::kBytes, true, true,                         \
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, IODT, FMT, 1, false, true, true>, true}
+
 // B-direct kernels: fp32 operands, fast path only
 #define CASCMM_BD_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                                \
   {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, 32 * WN, BK, TileBD<BM, WN, BK, DEPTH, NP>::NT, \

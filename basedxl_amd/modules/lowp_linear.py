@@ -4,7 +4,9 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
-from ..cascaded_lowp_matmul import PreparedWeight, cascaded_lowp_matmul, tensor_scale_exp
+from typing import Optional
+
+from ..cascaded_lowp_matmul import PreparedWeight, cascaded_lowp_matmul, default_cascade, tensor_scale_exp
 
 
 class BasedXLLowPLinear(nn.Module):
@@ -12,14 +14,15 @@ class BasedXLLowPLinear(nn.Module):
     (lowp_linear.py:12) and the forward pass is one cascade GEMM with the bias add fused
     into its store (the reference adds it in a second kernel, lowp_linear.py:17-19)."""
 
-    def __init__(self, submodule: nn.Linear, *, lowp: str = "bf16", terms: int = 2, products: str = "tri",
-                 prepared: bool = False):
+    def __init__(self, submodule: nn.Linear, *, lowp: Optional[str] = None, terms: Optional[int] = None,
+                 products: str = "tri", prepared: bool = False):
         super().__init__()
         self.in_features = submodule.in_features
         self.out_features = submodule.out_features
         self.weight = submodule.weight.detach().T.contiguous().clone()
         self.bias = submodule.bias.detach().clone() if submodule.bias is not None else None
-        self.lowp, self.terms, self.products = lowp, terms, products
+        d_lowp, d_terms = default_cascade(self.weight.dtype)   # fp32: bf16 x 2; fp16 / bf16: their own format x 1
+        self.lowp, self.terms, self.products = d_lowp if lowp is None else lowp, d_terms if terms is None else terms, products
         self._weight_exp = None   # fp8: tensor-scale exponent of the weight, found on first use
         # prepared=True: the weight is also kept split (once, on first use on the GPU); inputs
         # the prepared kernels do not take (not fp32, K not a multiple of 64) use the raw weight

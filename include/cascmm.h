@@ -31,8 +31,12 @@ extern "C" {
 #define CASCMM_VERSION 100 /* major*10000 + minor*100 + patch */
 
 /* element type of A, B, C and bias as stored in memory (C has the type of A, like
- * `torch.empty((M, N), dtype=a.dtype)` at cascaded_lowp_matmul.py:161).  The fast kernels take
- * fp32; fp16 / bf16 run on bounds-checked kernels (bf16 or fp16 terms, 1 or 2 of them, tri). */
+ * `torch.empty((M, N), dtype=a.dtype)` at cascaded_lowp_matmul.py:161).  The cascade kernels
+ * take fp32.  fp16 (bf16) tensors multiplied as ONE fp16 (bf16) term have fast kernels too:
+ * through cascmm_gemm_prepared, or through cascmm_gemm when K % 64 == 0, the rows of A are
+ * 16-byte aligned and the workspace holds cascmm_workspace_bytes(...) (B is re-laid there
+ * first).  Other combinations with 16-bit tensors run on bounds-checked kernels (bf16 or
+ * fp16 terms, 1 or 2 of them, tri). */
 enum cascmm_dtype { CASCMM_DT_F32 = 0, CASCMM_DT_F16 = 1, CASCMM_DT_BF16 = 2 };
 
 /* low-precision format of the cascade terms */

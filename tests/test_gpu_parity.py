@@ -173,7 +173,7 @@ def test_sixteen_bit_operands_integer_exact(gpu_device, dtype, shape):
     tag = "_ioh" if dtype == torch.float16 else "_iob"
     ran = 0
     for vi, name in enumerate(_lib.variant_names()):
-        if tag not in name:
+        if tag not in name or "_bpre" in name:
             continue
         fmt = [f for f in ("bf16", "fp16", "fp8") if f + "x" in name][0]
         terms = int(name.split(fmt + "x")[1][0])
@@ -209,6 +209,49 @@ def test_sixteen_bit_operands_match_oracle(gpu_device, dtype, fmt, terms):
     assert float((got_nb == want_nb).float().mean()) > 0.98
     assert bool(((got_nb.float() - want_nb.float()).abs() <= torch.maximum(want_nb.float().abs(), torch.tensor(1e-3))
                  * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7)).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_sixteen_bit_fast_path(gpu_device, dtype):
+    """fp16 / bf16 tensors with the default cascade (one term of their own format): B is re-laid
+    as operand slots (on the fly into the workspace, or once with PreparedWeight) and the
+    copy-only kernels run.  Integers exact on every such kernel; random operands equal the
+    oracle's wrapper up to one unit in the last place of the 16-bit output."""
+    tag = "_bpre_ioh" if dtype == torch.float16 else "_bpre_iob"
+    names = _lib.variant_names()
+    hi = 3 if dtype == torch.float16 else 1
+    for (M, K, N) in [(256, 192, 160), (300, 128, 200), (130, 64, 84)]:
+        a, b, want = _int_case(M, K, N, hi, seed=M + N + 5)
+        at, bt = _gpu(torch.tensor(a, dtype=dtype)), _gpu(torch.tensor(b, dtype=dtype))
+        w = PreparedWeight(bt)
+        for vi, name in enumerate(names):
+            if tag not in name:
+                continue
+            _say("16-bit fast", (M, K, N), name)
+            out = cascaded_lowp_matmul(at, w, variant=vi)
+            assert out.dtype == dtype
+            assert np.array_equal(out.float().cpu().numpy().astype(np.int64), want), (name, M, K, N)
+        auto = cascaded_lowp_matmul(at, bt)          # two plain tensors: prepared on the fly
+        assert np.array_equal(auto.float().cpu().numpy().astype(np.int64), want)
+    g = torch.Generator().manual_seed(23)
+    a = torch.randn(2, 512, 640, generator=g).to(dtype)
+    b = (torch.randn(640, 320, generator=g) * 0.05).to(dtype)
+    bias = torch.randn(320, generator=g).to(dtype)
+    fmt = "fp16" if dtype == torch.float16 else "bf16"
+    want32 = oc.cascade_matmul_ref(a.reshape(-1, 640).float(), b.float(), fmt, 1, "tri") + bias.float()
+    # one unit in the last place of the 16-bit output (outputs near zero: of 0.02, far above the
+    # 1e-6 by which fp32 sums in different orders differ)
+    ulp = lambda t: torch.maximum(t.float().abs(), torch.tensor(2e-2)) * (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7)
+    for bb in (_gpu(b), PreparedWeight(_gpu(b))):
+        got = cascaded_lowp_matmul(_gpu(a), bb, bias=_gpu(bias)).cpu().reshape(-1, 320)
+        want = want32.to(dtype)
+        assert bool(((got.float() - want.float()).abs() <= ulp(want)).all())
+        assert float((got == want).float().mean()) > 0.98
+    lin = torch.nn.Linear(640, 320).to("cuda:0").to(dtype)
+    x = _gpu(a)
+    y0, y1 = BasedXLLowPLinear(lin)(x), BasedXLLowPLinear(lin, prepared=True)(x)
+    assert y0.dtype == dtype and y1.shape == (2, 512, 320)
+    assert bool(((y0.float() - y1.float()).abs() <= ulp(y0)).all())
 
 
 def test_fast_variant_is_refused_for_unaligned_k(gpu_device):
@@ -499,7 +542,7 @@ def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
     a7, b7, want7 = _int_case(M, K, N, 7, seed=M + K + N + 1)
     ran = 0
     for vi, name in enumerate(_lib.variant_names()):
-        if "_bpre" not in name or K % int(name.split("_")[0].split("x")[2]):
+        if "_bpre" not in name or "_io" in name or K % int(name.split("_")[0].split("x")[2]):
             continue
         fmt, terms = _fmt_of(name)
         _say("int-exact prepared", shape, name)
