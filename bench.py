@@ -91,6 +91,9 @@ def main():
                          "plus to_out on its own (default), all four in one grouped launch, or four separate launches")
     ap.add_argument("--streams", type=int, default=1,
                     help="number of HIP streams the four independent GEMMs of a step are spread over")
+    ap.add_argument("--rotate", type=int, default=1,
+                    help="number of distinct input/weight/output buffer sets the steps cycle through (1 = the same "
+                         "70 MB every step, resident in the Infinity Cache; 8 = 560 MB, every step reads HBM-cold data)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -110,12 +113,20 @@ def main():
     outs = [torch.empty(M, N, device=dev, dtype=torch.float32) for _ in range(N_PROJ)]
 
     ins = [x, x, x, y]
+    # --rotate R: R - 1 further copies of every buffer; step i uses set i % R
+    sets = [(ins, ws, outs)]
+    for _ in range(max(1, args.rotate) - 1):
+        x2, y2 = x.clone(), y.clone()
+        sets.append(([x2, x2, x2, y2], [w.clone() for w in ws], [torch.empty_like(o) for o in outs]))
+    step_no = [0]
     extra = [torch.cuda.Stream() for _ in range(max(0, min(args.streams, N_PROJ) - 1))]
 
     def step():
         # the four projections are independent GEMMs; with --streams > 1 they are enqueued on
         # several streams (forked from and joined back into the current one) so that the tail
         # of one kernel overlaps the start of the next
+        ins, ws, outs = sets[step_no[0] % len(sets)]
+        step_no[0] += 1
         if args.group == "qkv+o":
             cascaded_lowp_matmul_grouped(ins[:3], ws[:3], outs=outs[:3])
             cascaded_lowp_matmul(ins[3], ws[3], out=outs[3])
@@ -160,6 +171,9 @@ def main():
         # one graph holds `per_graph` consecutive steps, as a UNet forward would hold hundreds of
         # layers: the cost of starting a graph is not charged to every step
         per_graph = max(d for d in range(1, 11) if args.steps % d == 0)
+        if len(sets) > 1:   # every set appears in the graph
+            per_graph = len(sets) if args.steps % len(sets) == 0 else per_graph
+        step_no[0] = 0
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             for _ in range(per_graph):
@@ -255,7 +269,9 @@ def main():
                          "all": "1 grouped launch per step (4 GEMMs)", "none": "4 launches per step"}[args.group],
             "launches_per_step": launches_per_step,
             "kernel": vname, "seed": SEED,
-            "cache_regime": "same buffers every step (70 MB working set, resident in the 256 MB Infinity Cache)",
+            "cache_regime": ("same buffers every step (70 MB working set, resident in the 256 MB Infinity Cache)"
+                             if len(sets) == 1 else
+                             f"{len(sets)} buffer sets in rotation ({70 * len(sets)} MB: inputs and weights come from HBM)"),
         },
         "roofline": {
             "bound": "mfma",

@@ -650,3 +650,20 @@ def test_more_tiles_than_resident_workgroups(gpu_device):
         _say("many-tiles", name)
         got = cascaded_lowp_matmul(at, bt, variant=vi).cpu().numpy().astype(np.int64)
         assert np.array_equal(got, want), name
+
+
+# ---------------------------------------------------------------------------------------
+# the shape harness and the error-study script run
+# ---------------------------------------------------------------------------------------
+def test_unet_shape_harness_and_error_script_run(gpu_device, capsys):
+    from basedxl_amd import measure_error, unet_shapes
+
+    shapes = [s for s in unet_shapes.sdxl_linear_shapes(batch=1, latent=32, half_latent=True)
+              if s.name.startswith(("attn1.to_q/k/v d=640", "attn2.to_k/v d=640", "time_embedding.linear_1"))]
+    for prepared in (False, True):
+        rows = unet_shapes.time_shapes(shapes, "bf16", 2, prepared=prepared, iters=2)
+        assert len(rows) == 3 and all(r["launch_us"] > 0 for r in rows)
+    a = torch.randn(96, 128, device="cuda:0")
+    b = torch.randn(128, 64, device="cuda:0")
+    m = measure_error.metrics(cascaded_lowp_matmul(a, b), a.double() @ b.double())
+    assert 1e-7 < m["rel_fro"] < 1e-4 and len(m["quantiles"]) == 5
