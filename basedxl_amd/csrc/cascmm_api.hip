@@ -66,7 +66,8 @@ static bool fast_ok(const Problem& q, const void* A, const void* B) {
   }
   return q.dtype == CASCMM_DT_F32 && q.lda % 4 == 0 && (A == nullptr || aligned_to(A, 16)) &&
          q.ldb % 4 == 0 && q.N % 4 == 0 && (B == nullptr || aligned_to(B, 16)) &&
-         q.lda * 4 * 512 < INT32_MAX && q.ldb * 4 * 136 < INT32_MAX;  // 32-bit byte offsets inside a tile
+         q.lda * 4 * 512 < INT32_MAX && q.ldb * 4 * 136 < INT32_MAX &&  // 32-bit byte offsets inside a tile
+         (q.bpre || q.K * q.ldb * 4 < INT32_MAX);  // ... and down a column block of B (buffer offsets are 32-bit)
 }
 
 static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {

@@ -109,3 +109,14 @@ def test_unet_shape_table_matches_the_architecture():
     assert 0.5 * total_flops(full) < total_flops(half) < 0.52 * total_flops(full) + total_flops(kv)
     convs = sdxl_linear_shapes(convs=True)
     assert sum(s.count for s in convs if not s.routed_by_reference) == 11
+
+
+def test_fast_kernels_are_not_chosen_when_offsets_would_overflow():
+    """The fast kernels address B with 32-bit byte offsets from the top of a column block: a B of
+    2 GiB or more must go to the bounds-checked kernels (64-bit addressing)."""
+    l = _lib.lib()
+    names = _lib.variant_names()
+    ok = l.cascmm_select_variant(4096, 16384, 16384, 16384, 16384, 16384, 0, 0, 2, 0)
+    big = l.cascmm_select_variant(4096, 32768, 32768, 32768, 32768, 32768, 0, 0, 2, 0)
+    assert ok >= 0 and "generic" not in names[ok]
+    assert big >= 0 and "generic" in names[big]
