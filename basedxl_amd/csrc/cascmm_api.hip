@@ -330,9 +330,6 @@ static bool onthefly_prepare_ok(const Problem& q, int count, const void* const* 
   return workspace && aligned_to(workspace, 16) && need <= INT32_MAX && workspace_bytes >= (size_t)need;
 }
 
-extern "C" int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
-                                     const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream);
-
 // One launch for `count` problems of one shape (count == 1: a plain GEMM).
 static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
                      const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,

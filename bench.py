@@ -32,7 +32,7 @@ TERMS, PRODUCTS_PER_ELEMENT = 2, 3  # bf16 hi/lo, tri product set
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
 # summary under profiles/ gives the commands and the calibration); keyed by (--group, GEMMs).
-TRAFFIC_BYTES_PER_LAUNCH = {("qkv+o", 3): 2 * 21929.1 * 1024 + 30720.0 * 1024}
+TRAFFIC_BYTES_PER_LAUNCH = {("qkv+o", 3): 2 * 21945.3 * 1024 + 30720.0 * 1024}
 SEED = 1
 
 
