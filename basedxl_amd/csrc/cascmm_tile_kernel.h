@@ -491,13 +491,13 @@ struct TileGemm {
       Ctx ctx;
       init_lds(ctx, rtid);
       Regs ring[D];
-      // loads for global step g (only ever called with g < gsteps): retarget on a new item
-      int cur_item = -1, prob = 0, m0 = 0, n0 = 0, kbase = 0;
-      auto target = [&](int g) {
-        const int j = g / ktiles;
-        if (j != cur_item) {
-          cur_item = j;
-          int item = blockIdx.x + j * gridDim.x;
+      // Loads for the next global step: target() is called once per global step, in order
+      // (0, 1, 2 ... gsteps - 1), and keeps its position in counters, so the K loop holds no
+      // integer division; the item is decoded (and the descriptors retargeted) on its first step.
+      int next_item = 0, next_kt = 0, prob = 0, m0 = 0, n0 = 0, kbase = 0;
+      auto target = [&](int /* g */) {
+        if (next_kt == 0) {
+          int item = blockIdx.x + next_item * gridDim.x;
           const int split = item / (p.count * tiles);   // K split: items are (split, problem, tile)
           item -= split * (p.count * tiles);
           kbase = split * ktiles * TL::BK;
@@ -508,7 +508,12 @@ struct TileGemm {
           n0 = tn * TL::BN;
           set_tile(ctx, p, prob, m0, n0, rtid);
         }
-        return kbase + (g - j * ktiles) * TL::BK;
+        const int k0 = kbase + next_kt * TL::BK;
+        if (++next_kt == ktiles) {
+          next_kt = 0;
+          ++next_item;
+        }
+        return k0;
       };
       auto issue = [&](int g, Regs& r) {
         const int k0 = target(g);
@@ -516,12 +521,16 @@ struct TileGemm {
         else load_generic(p, prob, m0, n0, k0, rtid, r);
       };
       // after the last step of an item the consumers reduce their K halves through LDS (WK == 2):
-      // three barriers during which nothing may be staged
-      auto item_end = [&](int g) {
-        if (TL::WK > 1 && (g + 1) % ktiles == 0) {
-          __syncthreads();
-          __syncthreads();
-          __syncthreads();
+      // three barriers during which nothing may be staged (called once per staged step, in order)
+      int staged_kt = 0;
+      auto item_end = [&](int /* g */) {
+        if (TL::WK > 1) {
+          if (++staged_kt == ktiles) {
+            staged_kt = 0;
+            __syncthreads();
+            __syncthreads();
+            __syncthreads();
+          }
         }
       };
 #pragma unroll
