@@ -169,7 +169,8 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
 
 
 def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optional[torch.Tensor],
-             fmt: int, terms: int, products: int, variant: int, b_exp: Optional[torch.Tensor] = None) -> None:
+             fmt: int, terms: int, products: int, variant: int, b_exp: Optional[torch.Tensor] = None,
+             tensor_exps: Optional[torch.Tensor] = None) -> None:
     M, K = a2.shape
     N = b2.shape[1]
     dt = _DTYPES[a2.dtype]
@@ -178,7 +179,12 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
     ws_bytes = l.cascmm_workspace_bytes(M, N, K, dt, fmt, terms, products)
     ws = _workspace(a2.device, stream, ws_bytes)
     exps = None
-    if fmt == _lib.FMT_FP8:
+    if fmt == _lib.FMT_FP8 and tensor_exps is not None:
+        # static scales: {e_A, e_B} chosen by the caller (calibrated once), no pass over the operands
+        if tensor_exps.dtype != torch.int32 or tensor_exps.numel() != 2 or not tensor_exps.is_cuda:
+            raise ValueError("tensor_exps must be a device int32 tensor {e_A, e_B}")
+        exps = tensor_exps.contiguous()
+    elif fmt == _lib.FMT_FP8:
         exps = torch.empty(2, dtype=torch.int32, device=a2.device)
         _lib.check(l.cascmm_tensor_exp(a2.data_ptr(), M, K, a2.stride(0), dt, exps.data_ptr(), stream),
                    "cascmm_tensor_exp(A)")
@@ -290,6 +296,7 @@ def cascaded_lowp_matmul(
     bias: Optional[torch.Tensor] = None,
     variant: int = -1,
     b_exp: Optional[torch.Tensor] = None,
+    tensor_exps: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     if lowp is None or terms is None:
         d_lowp, d_terms = default_cascade(a.dtype)
@@ -354,7 +361,7 @@ def cascaded_lowp_matmul(
     if N > 1 and out2.stride(1) != 1:
         raise ValueError("out must have unit stride along N")
 
-    _gemm_2d(a2, b, out2, bias, fmt, terms, prod, variant, b_exp)
+    _gemm_2d(a2, b, out2, bias, fmt, terms, prod, variant, b_exp, tensor_exps)
 
     if dump_ptx:
         # the reference writes the kernel's PTX (cascaded_lowp_matmul.py:170-171); there is no

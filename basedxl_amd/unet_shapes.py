@@ -83,7 +83,7 @@ def total_flops(shapes: List[LinearShape]) -> float:
 
 
 def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool = False, iters: int = 10,
-                seed: int = 0) -> List[dict]:
+                seed: int = 0, static_scales: bool = False) -> List[dict]:
     """Times every shape on cuda:0 (HIP-graph replay of `iters` launches, random fp32 operands:
     activations N(0,1), weights 0.02 N(0,1)); returns one record per shape."""
     import torch
@@ -98,7 +98,16 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
         ws = [(torch.randn(s.K, s.N, generator=g) * 0.02).to(dev) for _ in range(s.group)]
         outs = [torch.empty(s.M, s.N, device=dev) for _ in range(s.group)]
         use_prepared = prepared and s.K % 64 == 0 and s.N % 4 == 0
-        if use_prepared:
+        if lowp == "fp8" and static_scales:
+            # fp8 tensor scales found once (as a calibrated deployment would), not in every call
+            from . import tensor_scale_exp
+            ea = tensor_scale_exp(a)
+            exps = [torch.cat([ea, tensor_scale_exp(w)]) for w in ws]
+
+            def run():
+                for i in range(s.group):
+                    cascaded_lowp_matmul(a, ws[i], out=outs[i], lowp=lowp, terms=terms, tensor_exps=exps[i])
+        elif use_prepared:
             pw = [PreparedWeight(w, lowp=lowp, terms=terms) for w in ws]
 
             def run():
@@ -141,6 +150,7 @@ def main(argv=None) -> None:
     ap.add_argument("--convs", action="store_true", help="include the 1x1 shortcut convolutions as GEMMs")
     ap.add_argument("--cascades", default="bf16x2,fp8x3")
     ap.add_argument("--prepared", action="store_true", help="split the weights once (PreparedWeight)")
+    ap.add_argument("--static-scales", action="store_true", help="fp8: tensor scales found once, not in every call")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args(argv)
     shapes = sdxl_linear_shapes(args.batch, args.latent, args.half_latent, convs=args.convs)
@@ -149,7 +159,7 @@ def main(argv=None) -> None:
                "prepared": args.prepared, "gflop_fp32_equiv_per_step": round(flops * 1e-9, 1), "cascades": {}}
     for casc in args.cascades.split(","):
         lowp, terms = casc.split("x")
-        rows = time_shapes(shapes, lowp, int(terms), prepared=args.prepared)
+        rows = time_shapes(shapes, lowp, int(terms), prepared=args.prepared, static_scales=args.static_scales)
         total_us = sum(r["us_per_step"] for r in rows)
         summary["cascades"][casc] = {"linear_ms_per_step": round(total_us * 1e-3, 3),
                                      "tflops_fp32_equiv": round(flops / total_us * 1e-6, 1), "shapes": rows}

@@ -446,6 +446,11 @@ def test_lowp_linear_module_fp8_caches_the_weight_scale(gpu_device):
     ref = oc.error_metrics(oc.cascade_matmul_ref(xa, w, "fp8", 3, "tri") + lin.bias.detach().cpu(), exp)
     got = oc.error_metrics(y1.cpu().reshape(-1, 320), exp)
     assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+    # static scales: the caller's exponents are used as they are (here: the ones the device found)
+    from basedxl_amd import tensor_scale_exp
+    exps = torch.cat([tensor_scale_exp(x), mod._weight_exp])
+    y3 = cascaded_lowp_matmul(x, mod.weight, bias=mod.bias, lowp="fp8", terms=3, tensor_exps=exps)
+    assert torch.equal(y3, y1)
     # grouped launch with fp8 computes the exponents of every problem on the device
     outs = cascaded_lowp_matmul_grouped([x, x], [mod.weight, mod.weight * 3.0], lowp="fp8", terms=3)
     assert torch.equal(outs[0].reshape(-1, 320) + mod.bias, y1.reshape(-1, 320)) or \
