@@ -672,3 +672,25 @@ def test_unet_shape_harness_and_error_script_run(gpu_device, capsys):
     b = torch.randn(128, 64, device="cuda:0")
     m = measure_error.metrics(cascaded_lowp_matmul(a, b), a.double() @ b.double())
     assert 1e-7 < m["rel_fro"] < 1e-4 and len(m["quantiles"]) == 5
+
+
+def test_wrapper_shapes_like_the_reference(gpu_device):
+    """M = prod(a.shape[:-1]) (cascaded_lowp_matmul.py:150-151), result reshaped to [*batch, N] (:173):
+    a 1-D ``a`` gives a 1-D result, a 4-D ``a`` keeps its leading dims, ``out`` of the flattened
+    shape is accepted and returned as a view."""
+    g = torch.Generator().manual_seed(51)
+    b = _gpu(torch.randn(64, 48, generator=g))
+    v = _gpu(torch.randn(64, generator=g))
+    r = cascaded_lowp_matmul(v, b)
+    assert r.shape == (48,)
+    torch.testing.assert_close(r, (v.double() @ b.double()).float(), rtol=1e-4, atol=1e-4)
+    a4 = _gpu(torch.randn(2, 3, 5, 64, generator=g))
+    r4 = cascaded_lowp_matmul(a4, b)
+    assert r4.shape == (2, 3, 5, 48)
+    torch.testing.assert_close(r4, (a4.double() @ b.double()).float(), rtol=1e-4, atol=1e-4)
+    out = torch.empty(30, 48, device="cuda:0")
+    r5 = cascaded_lowp_matmul(a4, b, out=out)
+    assert r5.shape == (2, 3, 5, 48) and r5.data_ptr() == out.data_ptr()
+    assert torch.equal(r5.reshape(30, 48), r4.reshape(30, 48))
+    at = _gpu(torch.randn(64, 40, generator=g)).t()          # [40, 64] with a column stride: made contiguous like :158
+    torch.testing.assert_close(cascaded_lowp_matmul(at, b), (at.double() @ b.double()).float(), rtol=1e-4, atol=1e-4)
