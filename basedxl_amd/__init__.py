@@ -1,8 +1,9 @@
 """MI355X-native cascaded low-precision matmul (the Linear-layer hot path of basedxl)."""
 from .cascaded_lowp_matmul import (cascaded_lowp_matmul, cascaded_lowp_matmul_grouped,  # noqa: F401
                                    cascaded_lowp_matmul_prepared, PreparedWeight, tensor_scale_exp)
-from .modules.lowp_linear import BasedXLLowPLinear, patch_linear_layers  # noqa: F401
+from .modules import (BasedXLFusedKV, BasedXLLowPConv1x1, BasedXLLowPLinear, patch_linear_layers,  # noqa: F401
+                      patch_pointwise_convs)
 
 __all__ = ["cascaded_lowp_matmul", "cascaded_lowp_matmul_grouped", "cascaded_lowp_matmul_prepared", "PreparedWeight", "tensor_scale_exp",
-           "BasedXLLowPLinear",
-           "patch_linear_layers"]
+           "BasedXLLowPLinear", "BasedXLLowPConv1x1", "BasedXLFusedKV",
+           "patch_linear_layers", "patch_pointwise_convs"]
