@@ -73,9 +73,14 @@ class PreparedWeight:
     """A constant right operand ``w`` ([K, N]: the ``[in, out]`` weight of
     basedxl/modules/lowp_linear.py:12) split once on the GPU into the terms of a cascade and
     kept as MFMA operand slots; ``cascaded_lowp_matmul(a, prepared)`` then splits only ``a``.
-    The arithmetic is the same as with the raw weight (same split, same products)."""
+    The arithmetic is the same as with the raw weight (same split, same products).
 
-    def __init__(self, w: torch.Tensor, *, lowp: Optional[str] = None, terms: Optional[int] = None):
+    ``glu=True``: ``w`` is the ``[in, 2 * inner]`` weight of a gated projection (diffusers' GEGLU:
+    ``h = x @ w + b; y = h[:, :inner] * gelu(h[:, inner:])``); its columns are stored so that a
+    kernel holds a value column and its gate column together, and the product with it returns
+    ``y`` ([..., inner]) directly, the gate applied in the GEMM's store (fp32 only, inner % 32 == 0)."""
+
+    def __init__(self, w: torch.Tensor, *, lowp: Optional[str] = None, terms: Optional[int] = None, glu: bool = False):
         _check_device_tensor(w, "w")
         if w.dim() != 2 or w.dtype not in _DTYPES:
             raise ValueError("PreparedWeight needs a 2-D fp32 / fp16 / bf16 tensor")
@@ -88,22 +93,28 @@ class PreparedWeight:
         self.shape = (self.K, self.N)
         self.lowp, self.terms, self.fmt = lowp, int(terms), _lib.FMT_BY_NAME[lowp]
         self.dtype, self.device = w.dtype, w.device
+        self.glu = bool(glu)
+        if self.glu and (w.dtype != torch.float32 or self.N % 64 != 0):
+            raise ValueError("glu=True needs an fp32 weight whose width is a multiple of 64")
+        self.out_features = self.N // 2 if self.glu else self.N
         w2 = _rows(w)
         l = _lib.lib()
         stream = torch.cuda.current_stream(w.device).cuda_stream
         self.exp = tensor_scale_exp(w2) if self.fmt == _lib.FMT_FP8 else None
         nbytes = l.cascmm_prepared_bytes(self.K, self.N, self.fmt, self.terms)
         self.slots = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=w.device)
-        _lib.check(l.cascmm_prepare_weight(w2.data_ptr(), self.K, self.N, w2.stride(0) if self.K > 1 else max(self.N, 1),
-                                           _DTYPES[w.dtype], self.fmt, self.terms,
-                                           self.exp.data_ptr() if self.exp is not None else None,
-                                           self.slots.data_ptr(), self.slots.numel(), stream), "cascmm_prepare_weight")
+        prepare = l.cascmm_prepare_weight_glu if self.glu else l.cascmm_prepare_weight
+        _lib.check(prepare(w2.data_ptr(), self.K, self.N, w2.stride(0) if self.K > 1 else max(self.N, 1),
+                           _DTYPES[w.dtype], self.fmt, self.terms, self.exp.data_ptr() if self.exp is not None else None,
+                           self.slots.data_ptr(), self.slots.numel(), stream), "cascmm_prepare_weight")
 
     def usable_with(self, a2: torch.Tensor) -> bool:
         """Whether the prepared kernels take this left operand: fp32 (or fp16 / bf16 tensors with a
         weight of the same dtype kept as one term of that format), K a multiple of 64, rows 16-byte
         aligned (anything else goes through the raw weight)."""
         if self.K % 64 != 0 or self.N % 4 != 0 or a2.data_ptr() % 16 != 0:
+            return False
+        if self.glu and a2.dtype != torch.float32:
             return False
         if a2.dtype == torch.float32:
             return a2.shape[0] <= 1 or a2.stride(0) % 4 == 0
@@ -128,12 +139,13 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
             raise TypeError("w_list must hold PreparedWeight objects")
         assert a.shape[-1] == w.K, "Incompatible dimensions"
         _check_device_tensor(a, "a")
-        if (w.K, w.N, w.fmt, w.terms) != (w0.K, w0.N, w0.fmt, w0.terms) or a.dtype != a_list[0].dtype:
+        if (w.K, w.N, w.fmt, w.terms, w.glu) != (w0.K, w0.N, w0.fmt, w0.terms, w0.glu) or a.dtype != a_list[0].dtype:
             raise ValueError("grouped problems must share one shape, cascade and activation dtype")
         if a.dtype not in _DTYPES:
             raise TypeError(f"unsupported dtype {a.dtype}")
         a2s.append(_rows(a.reshape(-1, w.K)))
     M, K, N = a2s[0].shape[0], w0.K, w0.N
+    NO = w0.out_features                       # columns of the result (N / 2 for a gated weight)
     lda = a2s[0].stride(0) if M > 1 else max(K, 1)
     for a2 in a2s:
         if a2.shape[0] != M or (M > 1 and a2.stride(0) != lda):
@@ -141,10 +153,10 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
     dev = a_list[0].device
     adt = a_list[0].dtype
     if outs is None:
-        outs = [torch.empty((M, N), device=dev, dtype=adt) for _ in range(n)]
+        outs = [torch.empty((M, NO), device=dev, dtype=adt) for _ in range(n)]
     for o in outs:
         _check_device_tensor(o, "out")
-        if o.numel() != M * N or not o.is_contiguous() or o.dtype != adt:
+        if o.numel() != M * NO or not o.is_contiguous() or o.dtype != adt:
             raise ValueError("every out must be a contiguous [M, N] tensor of the dtype of a")
     if biases is not None:
         biases = [None if bb is None else bb.contiguous() for bb in biases]
@@ -161,11 +173,11 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
             _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _DTYPES[adt], exps.data_ptr() + 8 * i,
                                                     stream), "cascmm_tensor_exp(A)")
             exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
-    st = _lib.lib().cascmm_gemm_prepared(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), _DTYPES[adt], w0.fmt, w0.terms,
-                                         _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None,
-                                         stream, variant)
+    gemm = _lib.lib().cascmm_gemm_prepared_glu if w0.glu else _lib.lib().cascmm_gemm_prepared
+    st = gemm(n, pa, pb, pc, pbias, M, N, K, lda, max(NO, 1), _DTYPES[adt], w0.fmt, w0.terms,
+              _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None, stream, variant)
     _lib.check(st, "cascmm_gemm_prepared")
-    return [o.reshape(*a.shape[:-1], N) for o, a in zip(outs, a_list)]
+    return [o.reshape(*a.shape[:-1], NO) for o, a in zip(outs, a_list)]
 
 
 def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optional[torch.Tensor],
@@ -303,7 +315,7 @@ def cascaded_lowp_matmul(
         lowp = d_lowp if lowp is None else lowp
         terms = d_terms if terms is None else terms
     if isinstance(b, PreparedWeight):
-        res = out.view(-1, b.N) if out is not None else None
+        res = out.view(-1, b.out_features) if out is not None else None
         return cascaded_lowp_matmul_prepared([a], [b], outs=None if res is None else [res],
                                              biases=None if bias is None else [bias], products=products,
                                              variant=variant)[0]

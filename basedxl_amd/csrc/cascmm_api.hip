@@ -37,6 +37,7 @@ struct Problem {
   int64_t M, N, K, lda, ldb, ldc;
   int dtype, fmt, terms, products;
   bool bpre = false;  // B is a prepared (already split) weight buffer
+  bool glu = false;   // gated epilogue: B prepared by cascmm_prepare_weight_glu, C has N / 2 columns
 };
 
 // bytes of a prepared weight: planes x ceil(K/8) x N operand slots of 16 bytes
@@ -52,7 +53,7 @@ static int check_problem(const Problem& q) {
   if (q.products != CASCMM_PROD_TRI && q.products != CASCMM_PROD_FULL) return CASCMM_ERR_BAD_FORMAT;
   if (q.M < 0 || q.N < 0 || q.K < 0) return CASCMM_ERR_BAD_SHAPE;
   if (q.M > INT32_MAX || q.N > INT32_MAX || q.K > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
-  if (q.lda < q.K || q.ldb < q.N || q.ldc < q.N) return CASCMM_ERR_BAD_SHAPE;
+  if (q.lda < q.K || q.ldb < q.N || q.ldc < (q.glu ? q.N / 2 : q.N)) return CASCMM_ERR_BAD_SHAPE;
   return CASCMM_OK;
 }
 
@@ -75,6 +76,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full || v.bpre != q.bpre) return false;
   if (v.fast && (!fast || q.K % v.BK != 0)) return false;
   if (v.kind == KIND_SPLITK && (q.M > 5 * v.BM || q.K < 4 * v.BK)) return false;  // skinny: few row tiles, deep K
+  if (q.glu && !v.glu) return false;
   return true;
 }
 
@@ -96,6 +98,14 @@ static const TunedCost kTuned[] = {
     {"t64x64x64_w2x2x1_d3_bf16x2_tri", 0.699, 1.98, 1.0, 1.0},
     {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.128, 4.52, 0.75, 0.75},
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.065, 8.41, 0.9, 0.9},
+    // right operand prepared (sweep over M in 1024..8192 of the UNet's (K, N) pairs)
+    {"t64x160x64_w2x1x2_d2_bf16x2_tri_bpre", 0.817, 5.30, 1.00, 0.80},
+    {"t64x160x64_w2x1x2_d3_bf16x2_tri_bpre", 0.811, 5.90, 1.00, 0.90},
+    {"t128x128x64_w2x2x1_d2_bf16x2_tri_bpre", 1.105, 6.41, 0.90, 0.70},
+    {"t128x160x32_w2x1x2_d3_bf16x2_tri_bpre", 1.332, 8.84, 0.80, 0.50},
+    {"t256x128x32_w4x1x1_d2_bf16x2_tri_bpre", 1.926, 8.80, 0.80, 0.90},
+    {"t64x64x64_w2x2x1_d3_bf16x2_tri_bpre", 0.484, 1.88, 1.00, 1.00},
+    {"t64x256x32_w1x4x1_d3_bf16x2_tri_bpre", 1.128, 5.55, 0.90, 0.60},
 };
 
 constexpr int kMaxTileSplits = 4;
@@ -124,7 +134,7 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count, si
     // columns: measured about a quarter slower (32768 x 640 x 320 on the 128-wide tile)
     const double edge = (q.N % v.BN != 0 || q.M % v.BM != 0) ? 1.25 : 1.0;
     double best = edge * rounds * ((double)q.K / 64.0 * t.step64_us + t.fixed_us);
-    if (count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0) {
+    if (count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0 && !q.glu) {
       const int64_t ksteps = (q.K + v.BK - 1) / v.BK;
       for (int sp = 2; sp <= kMaxTileSplits; ++sp) {
         if (ksteps % sp != 0 || ksteps / sp < 4 || tiles * sp > kNumCUs) continue;
@@ -273,17 +283,20 @@ static int launch_split(const void* x, float* out, int64_t n, int terms, int ten
 // out[(plane * K/8 + kg) * N + n].
 template <int IODT, int FMT, int TERMS>
 __global__ __launch_bounds__(256) void prepare_weight_kernel(const void* B, int K, int N, int64_t ldb,
-                                                            const int32_t* tensor_exp, u32x4* out) {
+                                                            const int32_t* tensor_exp, u32x4* out, int glu) {
   typedef typename IoType<IODT>::T T;
   const int kgs = (K + 7) / 8;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (int64_t)kgs * N) return;
   const int kg = (int)(i / N), n = (int)(i - (int64_t)kg * N);
+  // gated layout: prepared columns alternate 32 value columns (first half of B) and their 32
+  // gate columns (second half)
+  const int src = glu ? (n >> 6) * 32 + (n & 31) + ((n >> 5) & 1) * (N >> 1) : n;
   float r[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const int k = kg * 8 + e;
-    r[e] = k < K ? IoType<IODT>::load((const T*)B + (int64_t)k * ldb + n) : 0.f;
+    r[e] = k < K ? IoType<IODT>::load((const T*)B + (int64_t)k * ldb + src) : 0.f;
   }
   constexpr int PL = Lowp<FMT>::planes(TERMS);
   u32x4 t[PL];
@@ -297,13 +310,14 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(const void* B, int 
 }
 
 template <int IODT, int FMT>
-static int launch_prepare(const void* B, int K, int N, int64_t ldb, int terms, const int32_t* e, u32x4* out, hipStream_t s) {
+static int launch_prepare(const void* B, int K, int N, int64_t ldb, int terms, const int32_t* e, u32x4* out, hipStream_t s,
+                          int glu) {
   const int64_t total = (int64_t)((K + 7) / 8) * N;
   const unsigned grid = (unsigned)((total + 255) / 256);
   switch (terms) {
-    case 1: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out); break;
-    case 2: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out); break;
-    case 3: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out); break;
+    case 1: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
+    case 2: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
+    case 3: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
     default: return CASCMM_ERR_BAD_FORMAT;
   }
   return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
@@ -311,10 +325,10 @@ static int launch_prepare(const void* B, int K, int N, int64_t ldb, int terms, c
 
 template <int IODT>
 static int launch_prepare_fmt(const void* B, int K, int N, int64_t ldb, int fmt, int terms, const int32_t* e, u32x4* out,
-                              hipStream_t s) {
-  if (fmt == CASCMM_FMT_BF16) return launch_prepare<IODT, CASCMM_FMT_BF16>(B, K, N, ldb, terms, e, out, s);
-  if (fmt == CASCMM_FMT_FP16) return launch_prepare<IODT, CASCMM_FMT_FP16>(B, K, N, ldb, terms, e, out, s);
-  if (fmt == CASCMM_FMT_FP8) return launch_prepare<IODT, CASCMM_FMT_FP8>(B, K, N, ldb, terms, e, out, s);
+                              hipStream_t s, int glu) {
+  if (fmt == CASCMM_FMT_BF16) return launch_prepare<IODT, CASCMM_FMT_BF16>(B, K, N, ldb, terms, e, out, s, glu);
+  if (fmt == CASCMM_FMT_FP16) return launch_prepare<IODT, CASCMM_FMT_FP16>(B, K, N, ldb, terms, e, out, s, glu);
+  if (fmt == CASCMM_FMT_FP8) return launch_prepare<IODT, CASCMM_FMT_FP8>(B, K, N, ldb, terms, e, out, s, glu);
   return CASCMM_ERR_BAD_FORMAT;
 }
 
@@ -343,6 +357,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
     if (!C[i]) return CASCMM_ERR_NULL_POINTER;
     if (!aligned_to(C[i], es) || (bias && !aligned_to(bias[i], es))) return CASCMM_ERR_ALIGNMENT;
   }
+  if (q.glu && (!q.bpre || q.dtype != CASCMM_DT_F32 || q.N % 64 != 0 || q.K == 0)) return CASCMM_ERR_BAD_SHAPE;
   if (q.K == 0) {
     const int64_t total = q.M * q.N;
     const unsigned grid = (unsigned)((total + 255) / 256);
@@ -408,6 +423,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   p.workspace_bytes = workspace_bytes;
   p.k_splits = v.kind == KIND_TILE ? splits : 1;
   p.tensor_exps = q.fmt == CASCMM_FMT_FP8 ? tensor_exps : nullptr;
+  p.glu = q.glu ? 1 : 0;
   for (int i = 0; i < count; ++i) {
     p.A[i] = A[i]; p.B[i] = B[i]; p.C[i] = C[i]; p.bias[i] = bias ? bias[i] : nullptr;
   }
@@ -451,9 +467,9 @@ size_t cascmm_prepared_bytes(int64_t K, int64_t N, int fmt, int terms) {
   return (size_t)prepared_bytes(K, N, fmt, terms);
 }
 
-int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
-                          const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream) {
-  if (K < 0 || N < 0 || ldb < N) return CASCMM_ERR_BAD_SHAPE;
+static int prepare_weight_impl(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                               const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream, int glu) {
+  if (K < 0 || N < 0 || ldb < N || (glu && N % 64 != 0)) return CASCMM_ERR_BAD_SHAPE;
   if (K > INT32_MAX || N > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
   if (terms < 1 || terms > 3) return CASCMM_ERR_BAD_FORMAT;
   if (fmt != CASCMM_FMT_BF16 && fmt != CASCMM_FMT_FP16 && fmt != CASCMM_FMT_FP8) return CASCMM_ERR_BAD_FORMAT;
@@ -462,10 +478,31 @@ int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int 
   if (!aligned_to(out, 16)) return CASCMM_ERR_ALIGNMENT;
   if (out_bytes < (size_t)prepared_bytes(K, N, fmt, terms)) return CASCMM_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == CASCMM_DT_F32) return launch_prepare_fmt<CASCMM_DT_F32>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s);
-  if (dtype == CASCMM_DT_F16) return launch_prepare_fmt<CASCMM_DT_F16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s);
-  if (dtype == CASCMM_DT_BF16) return launch_prepare_fmt<CASCMM_DT_BF16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s);
+  if (dtype == CASCMM_DT_F32) return launch_prepare_fmt<CASCMM_DT_F32>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s, glu);
+  if (dtype == CASCMM_DT_F16) return launch_prepare_fmt<CASCMM_DT_F16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s, glu);
+  if (dtype == CASCMM_DT_BF16) return launch_prepare_fmt<CASCMM_DT_BF16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s, glu);
   return CASCMM_ERR_BAD_DTYPE;
+}
+
+int cascmm_prepare_weight(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                          const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream) {
+  return prepare_weight_impl(B, K, N, ldb, dtype, fmt, terms, tensor_exp, out, out_bytes, stream, 0);
+}
+
+int cascmm_prepare_weight_glu(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                              const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream) {
+  return prepare_weight_impl(B, K, N, ldb, dtype, fmt, terms, tensor_exp, out, out_bytes, stream, 1);
+}
+
+int cascmm_gemm_prepared_glu(int count, const void* const* A, const void* const* Bprep, void* const* C,
+                             const void* const* bias, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                             int dtype, int fmt, int terms, int products, const int32_t* tensor_exps, void* stream,
+                             int variant) {
+  if (!A || !Bprep || !C) return CASCMM_ERR_NULL_POINTER;
+  Problem q{M, N, K, lda, N, ldc, dtype, fmt, terms, products};
+  q.bpre = true;
+  q.glu = true;
+  return gemm_impl(count, A, Bprep, C, bias, q, tensor_exps, nullptr, 0, (hipStream_t)stream, variant);
 }
 
 int cascmm_gemm_prepared(int count, const void* const* A, const void* const* Bprep, void* const* C,
@@ -484,7 +521,7 @@ int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, i
   q.bpre = true;
   const int st = check_problem(q);
   if (st != CASCMM_OK) return st;
-  return select_variant(q, fast_ok(q, nullptr, nullptr), count);
+  return select_variant(q, fast_ok(q, nullptr, nullptr), count, 0);   // cascmm_gemm_prepared brings no workspace: no K split
 }
 
 size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms, int products) {

@@ -230,6 +230,10 @@ struct GroupParams {
   size_t workspace_bytes;
   int k_splits;             // LDS-tiled kernels: work item = (split, problem, tile); 0 or 1 = no split
   const int32_t* tensor_exps;  // fp8: {e_A, e_B} of problem i at [2i], [2i + 1]; NULL = all zero
+  // Gated epilogue (prepared-weight kernels): the N columns of B alternate 32 "value" and 32
+  // "gate" columns; C has N/2 columns, C[m][32 j + l] = (h[m][64 j + l] + bias[32 j + l]) *
+  // gelu(h[m][64 j + 32 + l] + bias[N/2 + 32 j + l]) with h = A x B.
+  int glu;
 };
 
 }  // namespace cascmm

@@ -158,6 +158,33 @@ struct TileGemm {
   // 8 consecutive elements of a row ARE the operand slot: the producers copy 16 bytes, no split
   static constexpr bool RAW16 = IODT != CASCMM_DT_F32;
   static constexpr int BREGS = BPRE ? 4 * PL : 8;            // registers of one B unit in the ring
+  // the gated epilogue needs prepared B (columns in any order at no cost), fp32 results and a
+  // consumer wave that owns whole value / gate pairs of 32-column blocks
+  static constexpr bool kGluCapable = BPRE && IODT == CASCMM_DT_F32 && TL::BNQ == 0 && TL::NTL % 2 == 0;
+  // value x gelu(gate), gelu(g) = 0.5 g (1 + erf(g / sqrt 2)) = 0.5 g erfc(-g / sqrt 2).
+  // With x = |g| / sqrt 2 <= 4:  t = erfc(x) = 2^P(x), P a degree-11 fit of log2 erfc on [0, 4]
+  // (|P - log2 erfc| < 4e-8, so t is good to a few 1e-6 RELATIVE down to erfc(4) = 1.5e-8), and
+  // 1 + erf(g / sqrt 2) = t for g < 0, 2 - t otherwise: no cancellation in the negative tail, no
+  // branch, one v_exp_f32.  Evaluated in fp32 the gate is within 4e-7 (one ulp at its largest)
+  // of the exact gelu, like the textbook formula on a correctly rounded erff.
+  static __device__ __forceinline__ float gated(float v, float g) {
+    const float ax = __builtin_fabsf(g) * 0.70710678118654752f;
+    const float x = __builtin_fminf(ax, 4.0f);
+    float p = 1.133601089e-07f;
+    p = __builtin_fmaf(p, x, -2.984485036e-06f);
+    p = __builtin_fmaf(p, x, 3.493388431e-05f);
+    p = __builtin_fmaf(p, x, -2.373710740e-04f);
+    p = __builtin_fmaf(p, x, 1.004358870e-03f);
+    p = __builtin_fmaf(p, x, -2.405994106e-03f);
+    p = __builtin_fmaf(p, x, 7.954029570e-05f);
+    p = __builtin_fmaf(p, x, 2.782256342e-02f);
+    p = __builtin_fmaf(p, x, -1.483802944e-01f);
+    p = __builtin_fmaf(p, x, -9.184222221e-01f);
+    p = __builtin_fmaf(p, x, -1.627909303e+00f);
+    p = __builtin_fmaf(p, x, 3.292588246e-08f);
+    const float t = ax > 4.0f ? 0.f : __builtin_amdgcn_exp2f(p);   // beyond: erfc < 1.6e-8, taken as 0
+    return v * (0.5f * g * (g < 0.f ? t : 2.f - t));
+  }
   static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // quads per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
 
@@ -744,6 +771,49 @@ struct TileGemm {
     constexpr int NQ = (TL::BNQ == 0) ? 0 : (TL::WN == 1 ? TL::BNQ / 32 : TL::NTL);
     constexpr int RUN = (NQ % 4 == 0) ? 4 : 2;
     const int b0 = wn0 >> 5;
+    if constexpr (kGluCapable) if (p.glu) {
+      // gated epilogue: blocks 2j (value) and 2j + 1 (gate) of this wave, same lane and register,
+      // make block j of the output, whose row has N/2 columns
+      const int half = p.N >> 1;
+      const int oc0 = (n0 + wn0) >> 1;   // first output column of this wave
+      if (interior) {
+        const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * ldc, 0x7FFFFFFF);
+        const int ldc_bytes = (int)ldc * ES;
+#pragma unroll
+        for (int nj = 0; nj < TL::NTL / 2; ++nj) {
+          const int col = oc0 + nj * 32 + l31;
+          const int voff = g * 4 * ldc_bytes + col * ES;
+          const float bv = bias ? bias[col] : 0.f, bg = bias ? bias[half + col] : 0.f;
+#pragma unroll
+          for (int mi = 0; mi < TL::MT; ++mi)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                llvm_raw_buffer_store_f32(gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg), rc, voff,
+                                          (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+        }
+        return;
+      }
+#pragma unroll
+      for (int nj = 0; nj < TL::NTL / 2; ++nj) {
+        const int col = oc0 + nj * 32 + l31;
+        if (col >= half) continue;
+        const float bv = bias ? bias[col] : 0.f, bg = bias ? bias[half + col] : 0.f;
+#pragma unroll
+        for (int mi = 0; mi < TL::MT; ++mi) {
+          const int row0 = m0 + wm0 + mi * 32 + g * 4;
+          IoT* dst = C + (int64_t)row0 * ldc + col;
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (row0 + q * 8 + e < p.M)
+                dst[(int64_t)(q * 8 + e) * ldc] = gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg);
+        }
+      }
+      return;
+    }
     if (IODT == CASCMM_DT_F32 && interior && (ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0 &&
         (bias == nullptr || (((uintptr_t)bias) & 15) == 0)) {
       // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask

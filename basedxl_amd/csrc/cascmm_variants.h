@@ -20,6 +20,7 @@ struct VariantDesc {
   bool grouped;  // one launch may run several same-shape problems and several tiles per workgroup
   int (*launch)(const GroupParams&, hipStream_t);
   bool bpre = false;  // takes the right operand already split (cascmm_prepare_weight)
+  bool glu = false;   // has the gated epilogue (a consumer wave owns whole value / gate block pairs)
 };
 
 template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST, bool BPRE = false>
@@ -45,6 +46,7 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
   const int splits = p.k_splits > 1 ? p.k_splits : 1;
   if (splits > 1) {
     // K split: fp32 only, one problem, partial results [split][M][N] in the workspace
+    if (p.glu) return CASCMM_ERR_BAD_VARIANT;
     if (IODT != CASCMM_DT_F32 || p.count != 1 || p.N % 4 != 0 || ((p.K + TL::BK - 1) / TL::BK) % splits != 0)
       return CASCMM_ERR_BAD_VARIANT;
     if (!p.workspace || p.workspace_bytes < (size_t)splits * p.M * p.N * sizeof(float)) return CASCMM_ERR_WORKSPACE;
@@ -149,7 +151,8 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
 #define CASCMM_TILE_VARIANT_BPRE(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, FMT, TERMS, FULL)                           \
   {NAME, KIND_TILE, CASCMM_DT_F32, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>::NT, \
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, Lowp<FMT>::planes(TERMS)>::kBytes, true, true,          \
-   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, CASCMM_DT_F32, FMT, TERMS, FULL, true, true>, true}
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, CASCMM_DT_F32, FMT, TERMS, FULL, true, true>, true,    \
+   ((BN) / (WN)) % 64 == 0}
 
 // fp16 (bf16) operands in memory multiplied as one fp16 (bf16) term, right operand prepared: the
 // producers only copy

@@ -9,6 +9,7 @@ convolutions (resnet shortcuts), which the reference does not route (unet.py:85)
 GEMMs over channels-last pixels and can be included with ``--convs``.
 
     python -m basedxl_amd.unet_shapes [--half-latent] [--convs] [--cascades bf16x2,fp8x3] [--prepared]
+                                      [--geglu off|unfused|fused]
 """
 from __future__ import annotations
 
@@ -27,6 +28,7 @@ class LinearShape:
     N: int
     group: int = 1  # GEMMs that share one activation tensor and can share one launch (to_q/k/v)
     routed_by_reference: bool = True
+    gated: bool = False  # the projection of a GEGLU block: value * gelu(gate) follows
 
     @property
     def flops(self) -> float:
@@ -50,7 +52,7 @@ def sdxl_linear_shapes(batch: int = 2, latent: int = 128, half_latent: bool = Fa
             LinearShape(f"attn2.to_q d={d}", blocks, tok, d, d),
             LinearShape(f"attn2.to_k/v d={d}", blocks, txt, 2048, d, group=2),
             LinearShape(f"attn2.to_out d={d}", blocks, tok, d, d),
-            LinearShape(f"ff.geglu_proj d={d}", blocks, tok, d, 8 * d),
+            LinearShape(f"ff.geglu_proj d={d}", blocks, tok, d, 8 * d, gated=True),
             LinearShape(f"ff.out d={d}", blocks, tok, 4 * d, d),
             LinearShape(f"transformer.proj_in/out d={d}", 2 * t2d, tok, d, d),
         ]
@@ -83,9 +85,11 @@ def total_flops(shapes: List[LinearShape]) -> float:
 
 
 def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool = False, iters: int = 10,
-                seed: int = 0, static_scales: bool = False) -> List[dict]:
+                seed: int = 0, static_scales: bool = False, geglu: str = "off") -> List[dict]:
     """Times every shape on cuda:0 (HIP-graph replay of `iters` launches, random fp32 operands:
-    activations N(0,1), weights 0.02 N(0,1)); returns one record per shape."""
+    activations N(0,1), weights 0.02 N(0,1)); returns one record per shape.  ``geglu``: what is
+    timed for the gated projections: "off" the GEMM alone, "unfused" the GEMM plus torch's
+    ``value * gelu(gate)``, "fused" the kernel that applies the gate in its store."""
     import torch
 
     from . import PreparedWeight, cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, cascaded_lowp_matmul_prepared
@@ -98,7 +102,15 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
         ws = [(torch.randn(s.K, s.N, generator=g) * 0.02).to(dev) for _ in range(s.group)]
         outs = [torch.empty(s.M, s.N, device=dev) for _ in range(s.group)]
         use_prepared = prepared and s.K % 64 == 0 and s.N % 4 == 0
-        if lowp == "fp8" and static_scales:
+        gate = geglu if s.gated else "off"
+        if gate == "fused":
+            pw = PreparedWeight(ws[0], lowp=lowp, terms=terms, glu=True)
+            gated_out = torch.empty(s.M, s.N // 2, device=dev)
+            use_prepared = True
+
+            def run():
+                cascaded_lowp_matmul(a, pw, out=gated_out)
+        elif lowp == "fp8" and static_scales:
             # fp8 tensor scales found once (as a calibrated deployment would), not in every call
             from . import tensor_scale_exp
             ea = tensor_scale_exp(a)
@@ -118,6 +130,12 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
         else:
             def run():
                 cascaded_lowp_matmul(a, ws[0], out=outs[0], lowp=lowp, terms=terms)
+        if gate == "unfused":
+            gemm, gated_out = run, torch.empty(s.M, s.N // 2, device=dev)
+
+            def run():
+                gemm()
+                torch.mul(outs[0][:, : s.N // 2], torch.nn.functional.gelu(outs[0][:, s.N // 2:]), out=gated_out)
         for _ in range(2):
             run()
         torch.cuda.synchronize()
@@ -125,8 +143,13 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
         with torch.cuda.graph(graph):
             for _ in range(iters):
                 run()
-        graph.replay()
-        torch.cuda.synchronize()
+        # the GPU leaves its idle clocks only after some 0.3 s of work (and drops back between
+        # shapes while the host builds the next operands): replay untimed until it has
+        import time
+        t_end = time.perf_counter() + (0.3 if not rows else 0.05)
+        while time.perf_counter() < t_end:
+            graph.replay()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(3):
@@ -135,7 +158,7 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / (3 * iters)
         rows.append({"name": s.name, "count": s.count, "group": s.group, "M": s.M, "K": s.K, "N": s.N,
-                     "launch_us": round(us, 2), "prepared": use_prepared,
+                     "launch_us": round(us, 2), "prepared": use_prepared, "gate": gate,
                      "tflops_fp32_equiv": round(2.0 * s.M * s.K * s.N * s.group / us * 1e-6, 1),
                      "us_per_step": round(us * s.count, 1)})
         del a, ws, outs
@@ -151,6 +174,8 @@ def main(argv=None) -> None:
     ap.add_argument("--cascades", default="bf16x2,fp8x3")
     ap.add_argument("--prepared", action="store_true", help="split the weights once (PreparedWeight)")
     ap.add_argument("--static-scales", action="store_true", help="fp8: tensor scales found once, not in every call")
+    ap.add_argument("--geglu", choices=["off", "unfused", "fused"], default="off",
+                    help="gated projections: time the GEMM alone, with torch's gate after it, or the fused kernel")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args(argv)
     shapes = sdxl_linear_shapes(args.batch, args.latent, args.half_latent, convs=args.convs)
@@ -159,7 +184,8 @@ def main(argv=None) -> None:
                "prepared": args.prepared, "gflop_fp32_equiv_per_step": round(flops * 1e-9, 1), "cascades": {}}
     for casc in args.cascades.split(","):
         lowp, terms = casc.split("x")
-        rows = time_shapes(shapes, lowp, int(terms), prepared=args.prepared, static_scales=args.static_scales)
+        rows = time_shapes(shapes, lowp, int(terms), prepared=args.prepared, static_scales=args.static_scales,
+                           geglu=args.geglu)
         total_us = sum(r["us_per_step"] for r in rows)
         summary["cascades"][casc] = {"linear_ms_per_step": round(total_us * 1e-3, 3),
                                      "tflops_fp32_equiv": round(flops / total_us * 1e-6, 1), "shapes": rows}

@@ -137,6 +137,27 @@ int cascmm_gemm_prepared(int count, const void* const* A, const void* const* Bpr
 int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
                                    int dtype, int fmt, int terms, int products);
 
+/*
+ * Gated projection (GEGLU) in one kernel.  The feed-forward block of the UNet's transformer layers
+ * (diffusers' `GEGLU`, a module of the third-party model the reference patches at
+ * basedxl/unet.py:81-87: `proj` is one of the nn.Linear layers it routes) computes
+ *     h = x . W + b   (N = 2 * Nh columns);   y = h[:, :Nh] * gelu(h[:, Nh:])   (exact, erf form)
+ * and writes h, reads it back and writes y.  Here the product and the gate share one kernel:
+ * cascmm_prepare_weight_glu prepares W [K, N] like cascmm_prepare_weight but with the columns
+ * reordered so that 32 value columns and their 32 gate columns alternate (N % 64 == 0), and
+ * cascmm_gemm_prepared_glu, with the arguments of cascmm_gemm_prepared, writes
+ *     C[m][j] = (h[m][j] + bias[j]) * gelu(h[m][Nh + j] + bias[Nh + j]),   C [M, Nh], ldc >= Nh,
+ * with `bias` (N entries, or NULL) in the ORIGINAL column order.  fp32 only; N is the width of
+ * the projection (2 * Nh).  CASCMM_ERR_BAD_FORMAT when no kernel with the gated store fits.
+ */
+int cascmm_prepare_weight_glu(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
+                              const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream);
+int cascmm_gemm_prepared_glu(int count, const void* const* A, const void* const* Bprep, void* const* C,
+                             const void* const* bias,
+                             int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
+                             int dtype, int fmt, int terms, int products,
+                             const int32_t* tensor_exps, void* stream, int variant);
+
 /* Bytes of device workspace cascmm_gemm can use for this problem (0 for most shapes).
  * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,
  * cascaded_lowp_matmul.py:155-156); the caller allocates, as it allocates `out` (:161). */

@@ -16,6 +16,12 @@ What is restated here and from where
   that collapse to a plain library matmul, and error bands against an fp64 product.
 * Wrapper semantics (batch flattening, the two asserts, output dtype/shape) follow
   basedxl/triton/cascaded_lowp_matmul.py:139-173.
+* The gated projection (``gated_projection_ref``) restates diffusers' ``GEGLU.forward``
+  (``hidden_states, gate = proj(x).chunk(2, dim=-1); return hidden_states * gelu(gate)``,
+  gelu in the exact erf form).  diffusers is a third-party dependency of the reference
+  (README.md:17 installs it unpinned; model.py:3-4 imports it) and is absent here, so its
+  published formula is restated; pins: math.erf in double precision on a grid, torch's own
+  gelu (a library routine) and the identities gelu(x) - gelu(-x) = x, gelu(0) = 0.
 * Error metrics follow extras/measure_cascaded_lowp_matmul_error.py:8-9,21,27-31 and the
   TFLOP/s formula follows basedxl/triton/cascaded_lowp_matmul.py:237-238.
 
@@ -161,6 +167,23 @@ def cascaded_lowp_matmul_ref(a: torch.Tensor, b: torch.Tensor, *,
         out.copy_(res.reshape(out.shape))
         return out.reshape(res.shape)
     return res
+
+
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    """Exact GELU, x * Phi(x) = 0.5 x (1 + erf(x / sqrt 2)), evaluated in the dtype of ``x``."""
+    return 0.5 * x * (1.0 + torch.erf(x * (1.0 / math.sqrt(2.0))))
+
+
+def gated_projection_ref(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, fmt: str = "bf16",
+                         terms: int = 2, products: str = "tri") -> torch.Tensor:
+    """``h = a . w (+ bias)`` through the cascade, then ``h[:, :inner] * gelu(h[:, inner:])``
+    in fp32: what diffusers' GEGLU computes around its ``proj`` Linear."""
+    assert w.shape[1] % 2 == 0
+    h = cascade_matmul_ref(a, w, fmt, terms, products)
+    if bias is not None:
+        h = h + bias
+    inner = w.shape[1] // 2
+    return h[:, :inner] * gelu_erf(h[:, inner:])
 
 
 # --------------------------------------------------------------------------------------

@@ -129,3 +129,120 @@ def test_fused_kv_equals_separate_projections_and_caches(gpu_device):
     assert mod.kv_cache is None
     k4, _ = BasedXLFusedKV(to_k, to_v)(ctx)
     assert torch.equal(k4, k)
+
+
+# ---------------------------------------------------------------------------------- gated projection
+
+
+def test_geglu_module_holds_the_transposed_weight():
+    from basedxl_amd import BasedXLLowPGEGLU
+
+    proj = torch.nn.Linear(64, 128)
+    mod = BasedXLLowPGEGLU(proj)
+    assert mod.inner == 64 and mod.weight.shape == (64, 128) and torch.equal(mod.weight, proj.weight.detach().T)
+    with pytest.raises(ValueError):
+        BasedXLLowPGEGLU(torch.nn.Linear(64, 127))
+
+
+def _glu_variants():
+    from basedxl_amd import _lib
+
+    l = _lib.lib()
+    return [i for i in range(l.cascmm_variant_count()) if l.cascmm_variant_name(i).decode().endswith("_tri_bpre")]
+
+
+@pytest.mark.gpu
+def test_gated_kernels_integer_exact_value_and_gate_pairing(gpu_device):
+    """Small-integer operands: h is exact, so every kernel with the gated store must give
+    value * gelu(gate) of the integer product up to the erf evaluation, on a shape with ragged row
+    and column tiles; kernels without the gated store must refuse."""
+    from basedxl_amd import PreparedWeight, _lib, cascaded_lowp_matmul
+
+    g = torch.Generator().manual_seed(41)
+    M, K, inner = 200, 128, 96
+    a = torch.randint(-3, 4, (M, K), generator=g).float()
+    w = torch.randint(-2, 3, (K, 2 * inner), generator=g).float()
+    bias = torch.randint(-2, 3, (2 * inner,), generator=g).float()
+    h = (a.long() @ w.long() + bias.long()).double()
+    want = h[:, :inner] * torch.nn.functional.gelu(h[:, inner:])
+    ran = 0
+    for lowp, terms in (("bf16", 2), ("bf16", 3), ("fp16", 3)):
+        pw = PreparedWeight(w.to("cuda:0"), lowp=lowp, terms=terms, glu=True)
+        for v in _glu_variants():
+            name = _lib.lib().cascmm_variant_name(v).decode()
+            if f"_{lowp}x{terms}_" not in name:
+                continue
+            try:
+                y = cascaded_lowp_matmul(a.to("cuda:0"), pw, bias=bias.to("cuda:0"), variant=v)
+            except RuntimeError as e:
+                assert "variant" in str(e).lower(), (name, str(e))
+                continue
+            assert y.shape == (M, inner), name
+            # fp32 gate: 1 + erf(g / sqrt 2) cancels for g << 0, an absolute error of about |value * g| * 2^-24
+            torch.testing.assert_close(y.cpu().double(), want, rtol=1e-5, atol=2e-5, msg=lambda m: f"{name}: {m}")
+            ran += 1
+    assert ran >= 5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,inner", [(4096, 640, 2560), (1024, 1280, 5120), (77, 640, 2560)])
+def test_geglu_module_matches_oracle_and_unfused_path(gpu_device, M, K, inner):
+    from basedxl_amd import BasedXLLowPGEGLU, BasedXLLowPLinear
+
+    torch.manual_seed(42)
+    proj = torch.nn.Linear(K, 2 * inner).to("cuda:0")
+    with torch.no_grad():
+        proj.weight.mul_(0.02 * K ** 0.5)     # weights of std ~0.02 like the UNet's
+    x = torch.randn(2, M // 2 if M % 2 == 0 else M, K, device="cuda:0")
+    if M % 2:
+        x = x[:1]
+    y = BasedXLLowPGEGLU(proj)(x)
+    assert y.shape == (*x.shape[:-1], inner)
+    # same cascade through the plain prepared path, gate applied by torch: only the erf evaluation
+    # and (when another tile is chosen) the accumulation order differ
+    h = BasedXLLowPLinear(proj, prepared=True)(x)
+    unfused = h[..., :inner] * torch.nn.functional.gelu(h[..., inner:])
+    torch.testing.assert_close(y, unfused, rtol=2e-5, atol=2e-5)
+    x2, wt, b = x.cpu().reshape(-1, K), proj.weight.detach().cpu().T.contiguous(), proj.bias.detach().cpu()
+    want = oc.gated_projection_ref(x2, wt, b)
+    h64 = oc.fp64_matmul(x2, wt) + b.double()
+    exp = h64[:, :inner] * oc.gelu_erf(h64[:, inner:])
+    got, ref = oc.error_metrics(y.cpu().reshape(-1, inner), exp), oc.error_metrics(want, exp)
+    assert got["rel_fro"] <= 1.25 * ref["rel_fro"] and got["max_abs"] <= 1.25 * ref["max_abs"], (got, ref)
+
+
+@pytest.mark.gpu
+def test_geglu_module_falls_back_to_three_kernels(gpu_device):
+    """Shapes the fused kernel does not take (inner not a multiple of 32) give the same function."""
+    from basedxl_amd import BasedXLLowPGEGLU
+
+    torch.manual_seed(43)
+    proj = torch.nn.Linear(64, 2 * 40).to("cuda:0")
+    x = torch.randn(50, 64, device="cuda:0")
+    y = BasedXLLowPGEGLU(proj)(x)
+    want = oc.gated_projection_ref(x.cpu(), proj.weight.detach().cpu().T.contiguous(), proj.bias.detach().cpu())
+    torch.testing.assert_close(y.cpu(), want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_gate_function_against_double_precision(gpu_device):
+    """The gate on its own: with A = I and value columns of ones, the kernel's output is
+    gelu(w[r, inner + j]) for gates on a grid of 2^-6 steps over [-12, 12] (exact in two bf16
+    terms).  Against 0.5 g erfc(-g / sqrt 2) in double precision: within one fp32 ulp of the gate
+    (4e-7 + 2e-7 |g|), and with RELATIVE accuracy in the negative tail, where the textbook
+    0.5 g (1 + erf) cancels."""
+    import math
+
+    from basedxl_amd import PreparedWeight, cascaded_lowp_matmul
+
+    inner = 64
+    gates = (torch.arange(64 * inner, dtype=torch.float64) * (1536.0 / (64 * inner - 1))).round() / 64.0 - 12.0
+    w = torch.ones(64, 2 * inner)
+    w[:, inner:] = gates.float().reshape(64, inner)
+    y = cascaded_lowp_matmul(torch.eye(64, device="cuda:0"), PreparedWeight(w.to("cuda:0"), glu=True)).cpu().double()
+    g = w[:, inner:].double()
+    want = torch.tensor([0.5 * v * math.erfc(-v / math.sqrt(2.0)) for v in g.flatten().tolist()], dtype=torch.float64).reshape(64, inner)
+    err = (y - want).abs()
+    assert bool((err <= 4e-7 + 2e-7 * g.abs()).all()), float(err.max())
+    neg = g < 0
+    assert bool((err[neg] <= 1e-5 * want[neg].abs() + 5e-8).all()), float((err[neg] / want[neg].abs().clamp_min(1e-30)).max())

@@ -194,3 +194,39 @@ def test_oracle_cascade_errors_match_the_fixture():
         # the fp32 matmuls inside the oracle may sum in another order on another torch build
         assert m["rel_fro"] == pytest.approx(rec["rel_fro"], rel=0.02), rec
         assert m["max_abs"] == pytest.approx(rec["max_abs"], rel=0.25), rec
+
+
+def test_gelu_erf_against_double_precision_erf_and_identities():
+    """The oracle's gate: double-precision math.erf on a grid (an independent evaluation), torch's
+    own gelu (library routine), and what the definition x * Phi(x) fixes: gelu(0) = 0,
+    gelu(x) - gelu(-x) = x, gelu(x) -> x and gelu(-x) -> 0 for large x."""
+    import math
+
+    xs = torch.linspace(-6.0, 6.0, 481, dtype=torch.float64)
+    want = torch.tensor([0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0))) for v in xs.tolist()], dtype=torch.float64)
+    got64 = oc.gelu_erf(xs)
+    assert torch.allclose(got64, want, rtol=1e-13, atol=1e-15)
+    got32 = oc.gelu_erf(xs.float())
+    assert torch.allclose(got32.double(), want, rtol=0, atol=1e-6)   # ulp(6) = 4.8e-7
+    assert torch.allclose(got32, torch.nn.functional.gelu(xs.float()), rtol=0, atol=1e-6)
+    assert oc.gelu_erf(torch.zeros(3)).abs().max() == 0
+    x = torch.linspace(0.0, 5.0, 101, dtype=torch.float64)
+    assert torch.allclose(oc.gelu_erf(x) - oc.gelu_erf(-x), x, rtol=0, atol=1e-15)
+    assert oc.gelu_erf(torch.tensor([40.0]))[0] == 40.0 and oc.gelu_erf(torch.tensor([-40.0]))[0] == 0.0
+
+
+def test_gated_projection_is_the_cascade_followed_by_the_gate():
+    """Integer operands make the cascade exact, so the gated projection must equal the gate applied
+    to the integer product (computed in int64), bias included; the value half must come from the
+    first half of the columns and the gate from the second (a swapped pair changes the result)."""
+    g = torch.Generator().manual_seed(5)
+    a = torch.randint(-4, 5, (9, 16), generator=g).float()
+    w = torch.randint(-3, 4, (16, 12), generator=g).float()
+    bias = torch.randint(-2, 3, (12,), generator=g).float()
+    h = (a.long() @ w.long() + bias.long()).double()
+    want = h[:, :6] * torch.nn.functional.gelu(h[:, 6:])
+    got = oc.gated_projection_ref(a, w, bias)
+    assert got.shape == (9, 6)
+    assert torch.allclose(got.double(), want, rtol=1e-6, atol=1e-6)
+    swapped = h[:, 6:] * torch.nn.functional.gelu(h[:, :6])
+    assert not torch.allclose(got.double(), swapped, rtol=1e-3, atol=1e-3)
