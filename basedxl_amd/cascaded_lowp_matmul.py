@@ -78,7 +78,7 @@ class PreparedWeight:
     ``glu=True``: ``w`` is the ``[in, 2 * inner]`` weight of a gated projection (diffusers' GEGLU:
     ``h = x @ w + b; y = h[:, :inner] * gelu(h[:, inner:])``); its columns are stored so that a
     kernel holds a value column and its gate column together, and the product with it returns
-    ``y`` ([..., inner]) directly, the gate applied in the GEMM's store (fp32 only, inner % 32 == 0)."""
+    ``y`` ([..., inner]) directly, the gate applied in the GEMM's store (inner % 32 == 0)."""
 
     def __init__(self, w: torch.Tensor, *, lowp: Optional[str] = None, terms: Optional[int] = None, glu: bool = False):
         _check_device_tensor(w, "w")
@@ -94,8 +94,8 @@ class PreparedWeight:
         self.lowp, self.terms, self.fmt = lowp, int(terms), _lib.FMT_BY_NAME[lowp]
         self.dtype, self.device = w.dtype, w.device
         self.glu = bool(glu)
-        if self.glu and (w.dtype != torch.float32 or self.N % 64 != 0):
-            raise ValueError("glu=True needs an fp32 weight whose width is a multiple of 64")
+        if self.glu and self.N % 64 != 0:
+            raise ValueError("glu=True needs a weight whose width is a multiple of 64")
         self.out_features = self.N // 2 if self.glu else self.N
         w2 = _rows(w)
         l = _lib.lib()
@@ -113,8 +113,6 @@ class PreparedWeight:
         weight of the same dtype kept as one term of that format), K a multiple of 64, rows 16-byte
         aligned (anything else goes through the raw weight)."""
         if self.K % 64 != 0 or self.N % 4 != 0 or a2.data_ptr() % 16 != 0:
-            return False
-        if self.glu and a2.dtype != torch.float32:
             return False
         if a2.dtype == torch.float32:
             return a2.shape[0] <= 1 or a2.stride(0) % 4 == 0

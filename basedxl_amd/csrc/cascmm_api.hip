@@ -357,7 +357,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
     if (!C[i]) return CASCMM_ERR_NULL_POINTER;
     if (!aligned_to(C[i], es) || (bias && !aligned_to(bias[i], es))) return CASCMM_ERR_ALIGNMENT;
   }
-  if (q.glu && (!q.bpre || q.dtype != CASCMM_DT_F32 || q.N % 64 != 0 || q.K == 0)) return CASCMM_ERR_BAD_SHAPE;
+  if (q.glu && (!q.bpre || q.N % 64 != 0 || q.K == 0)) return CASCMM_ERR_BAD_SHAPE;
   if (q.K == 0) {
     const int64_t total = q.M * q.N;
     const unsigned grid = (unsigned)((total + 255) / 256);

@@ -158,9 +158,9 @@ struct TileGemm {
   // 8 consecutive elements of a row ARE the operand slot: the producers copy 16 bytes, no split
   static constexpr bool RAW16 = IODT != CASCMM_DT_F32;
   static constexpr int BREGS = BPRE ? 4 * PL : 8;            // registers of one B unit in the ring
-  // the gated epilogue needs prepared B (columns in any order at no cost), fp32 results and a
-  // consumer wave that owns whole value / gate pairs of 32-column blocks
-  static constexpr bool kGluCapable = BPRE && IODT == CASCMM_DT_F32 && TL::BNQ == 0 && TL::NTL % 2 == 0;
+  // the gated epilogue needs prepared B (columns in any order at no cost) and a consumer wave that
+  // owns whole value / gate pairs of 32-column blocks
+  static constexpr bool kGluCapable = BPRE && TL::BNQ == 0 && TL::NTL % 2 == 0;
   // value x gelu(gate), gelu(g) = 0.5 g (1 + erf(g / sqrt 2)) = 0.5 g erfc(-g / sqrt 2).
   // With x = |g| / sqrt 2 <= 4:  t = erfc(x) = 2^P(x), P a degree-11 fit of log2 erfc on [0, 4]
   // (|P - log2 erfc| < 4e-8, so t is good to a few 1e-6 RELATIVE down to erfc(4) = 1.5e-8), and
@@ -783,15 +783,18 @@ struct TileGemm {
         for (int nj = 0; nj < TL::NTL / 2; ++nj) {
           const int col = oc0 + nj * 32 + l31;
           const int voff = g * 4 * ldc_bytes + col * ES;
-          const float bv = bias ? bias[col] : 0.f, bg = bias ? bias[half + col] : 0.f;
+          const float bv = bias ? IoType<IODT>::load(bias + col) : 0.f, bg = bias ? IoType<IODT>::load(bias + half + col) : 0.f;
 #pragma unroll
           for (int mi = 0; mi < TL::MT; ++mi)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
-                llvm_raw_buffer_store_f32(gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg), rc, voff,
-                                          (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+              for (int e = 0; e < 4; ++e) {
+                const float y = gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg);
+                const int soff = (mi * 32 + q * 8 + e) * ldc_bytes;
+                if constexpr (IODT == CASCMM_DT_F32) llvm_raw_buffer_store_f32(y, rc, voff, soff, 0);
+                else llvm_raw_buffer_store_i16(__builtin_bit_cast(short, (IoT)y), rc, voff, soff, 0);
+              }
         }
         return;
       }
@@ -799,7 +802,7 @@ struct TileGemm {
       for (int nj = 0; nj < TL::NTL / 2; ++nj) {
         const int col = oc0 + nj * 32 + l31;
         if (col >= half) continue;
-        const float bv = bias ? bias[col] : 0.f, bg = bias ? bias[half + col] : 0.f;
+        const float bv = bias ? IoType<IODT>::load(bias + col) : 0.f, bg = bias ? IoType<IODT>::load(bias + half + col) : 0.f;
 #pragma unroll
         for (int mi = 0; mi < TL::MT; ++mi) {
           const int row0 = m0 + wm0 + mi * 32 + g * 4;
@@ -809,7 +812,8 @@ struct TileGemm {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               if (row0 + q * 8 + e < p.M)
-                dst[(int64_t)(q * 8 + e) * ldc] = gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg);
+                IoType<IODT>::store(dst + (int64_t)(q * 8 + e) * ldc,
+                                    gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg));
         }
       }
       return;

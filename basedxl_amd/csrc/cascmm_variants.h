@@ -159,7 +159,8 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
 #define CASCMM_TILE_VARIANT_BPRE16(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT)                       \
   {NAME, KIND_TILE, IODT, FMT, 1, false, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>::NT,     \
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, 1>::kBytes, true, true,                         \
-   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, IODT, FMT, 1, false, true, true>, true}
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, false>, IODT, FMT, 1, false, true, true>, true,      \
+   ((BN) / (WN)) % 64 == 0}
 
 // B-direct kernels: fp32 operands, fast path only
 #define CASCMM_BD_VARIANT(NAME, BM, WN, BK, DEPTH, NP, FMT, TERMS, FULL)                                \

@@ -21,8 +21,8 @@ class BasedXLLowPGEGLU(nn.Module):
     """Wraps the ``proj`` Linear ([in] -> [2 * inner]) of a GEGLU block; ``forward(x)`` returns
     ``value * gelu(gate)`` ([..., inner]), gelu in its exact (erf) form.
 
-    The fused kernel takes fp32 activations on the GPU with ``in % 64 == 0`` and ``inner % 32 == 0``;
-    anything else runs the cascade GEMM on the raw weight followed by torch's gate (the same
+    The fused kernel takes fp32 activations (any cascade) or fp16 / bf16 activations (as one term of
+    their own format) on the GPU with ``in % 64 == 0`` and ``inner % 32 == 0``; anything else runs the cascade GEMM on the raw weight followed by torch's gate (the same
     arithmetic in three kernels)."""
 
     def __init__(self, proj: nn.Linear, *, lowp: Optional[str] = None, terms: Optional[int] = None,
@@ -38,8 +38,10 @@ class BasedXLLowPGEGLU(nn.Module):
         self._prepared: Optional[PreparedWeight] = None
 
     def _fusable(self, x: torch.Tensor) -> bool:
-        return (x.is_cuda and x.dtype == torch.float32 and self.weight.dtype == torch.float32
-                and self.in_features % 64 == 0 and self.inner % 32 == 0)
+        if not x.is_cuda or x.dtype != self.weight.dtype or self.in_features % 64 != 0 or self.inner % 32 != 0:
+            return False
+        # 16-bit tensors have prepared kernels only for one term of their own format
+        return x.dtype == torch.float32 or (self.lowp, self.terms) == default_cascade(x.dtype)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self._fusable(x):

@@ -147,8 +147,10 @@ int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, i
  * reordered so that 32 value columns and their 32 gate columns alternate (N % 64 == 0), and
  * cascmm_gemm_prepared_glu, with the arguments of cascmm_gemm_prepared, writes
  *     C[m][j] = (h[m][j] + bias[j]) * gelu(h[m][Nh + j] + bias[Nh + j]),   C [M, Nh], ldc >= Nh,
- * with `bias` (N entries, or NULL) in the ORIGINAL column order.  fp32 only; N is the width of
- * the projection (2 * Nh).  CASCMM_ERR_BAD_FORMAT when no kernel with the gated store fits.
+ * with `bias` (N entries, or NULL) in the ORIGINAL column order; N is the width of the projection
+ * (2 * Nh).  Element types as cascmm_gemm_prepared (fp32, or fp16 / bf16 tensors as one term of
+ * their own format; the gate is computed in fp32 on the unrounded accumulators and the result
+ * rounded once).  CASCMM_ERR_BAD_FORMAT when no kernel with the gated store fits.
  */
 int cascmm_prepare_weight_glu(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
                               const int32_t* tensor_exp, void* out, size_t out_bytes, void* stream);

@@ -246,3 +246,25 @@ def test_gate_function_against_double_precision(gpu_device):
     assert bool((err <= 4e-7 + 2e-7 * g.abs()).all()), float(err.max())
     neg = g < 0
     assert bool((err[neg] <= 1e-5 * want[neg].abs() + 5e-8).all()), float((err[neg] / want[neg].abs().clamp_min(1e-30)).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,fmt,ulp", [(torch.float16, "fp16", 2.0 ** -10), (torch.bfloat16, "bf16", 2.0 ** -7)])
+def test_geglu_module_sixteen_bit_tensors(gpu_device, dtype, fmt, ulp):
+    """fp16 / bf16 tensors (what the reference runs its UNet in): the gate is applied in fp32 to the
+    unrounded accumulators and the result rounded once, so it must sit within one unit in the last
+    place of the oracle's fp32 result (the 16-bit operands as one exact term each)."""
+    from basedxl_amd import BasedXLLowPGEGLU
+
+    torch.manual_seed(44)
+    M, K, inner = 384, 640, 1280
+    proj = torch.nn.Linear(K, 2 * inner).to("cuda:0").to(dtype)
+    x = torch.randn(M, K, device="cuda:0").to(dtype)
+    mod = BasedXLLowPGEGLU(proj)
+    y = mod(x)
+    assert mod._prepared is not None and mod._prepared.glu        # the fused kernel ran, not the fallback
+    assert y.dtype == dtype and y.shape == (M, inner)
+    want = oc.gated_projection_ref(x.cpu().float(), proj.weight.detach().cpu().float().T.contiguous(),
+                                   proj.bias.detach().cpu().float(), fmt, 1)
+    err = (y.cpu().float() - want).abs()
+    assert bool((err <= ulp * want.abs() + 1e-6).all()), float((err / want.abs().clamp_min(1e-6)).max())
