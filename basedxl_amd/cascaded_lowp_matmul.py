@@ -278,9 +278,16 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
                        "cascmm_tensor_exp(A)")
             _lib.check(_lib.lib().cascmm_tensor_exp(b_list[i].data_ptr(), K, N, max(N, 1), dt,
                                                     exps.data_ptr() + 8 * i + 4, stream), "cascmm_tensor_exp(B)")
+    # 16-bit tensors as one term of their own format: room for every right operand re-laid as operand slots
+    ws = None
+    if a_list[0].dtype != torch.float32:
+        need = _lib.lib().cascmm_workspace_bytes(M, N, K, _DTYPES[a_list[0].dtype], fmt, terms, prod)
+        ws = _workspace(dev, stream, n * need) if need else None
     st = _lib.lib().cascmm_gemm_grouped(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), max(N, 1),
                                         _DTYPES[a_list[0].dtype], fmt, terms, prod,
-                                        exps.data_ptr() if exps is not None else None, None, 0, stream, variant)
+                                        exps.data_ptr() if exps is not None else None,
+                                        ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+                                        stream, variant)
     _lib.check(st, "cascmm_gemm_grouped")
     return [o.reshape(*a.shape[:-1], N) for o, a in zip(outs, a_list)]
 

@@ -334,14 +334,17 @@ static int launch_prepare_fmt(const void* B, int K, int N, int64_t ldb, int fmt,
 
 // 16-bit tensors multiplied as one term of their own format can use the prepared-operand kernels
 // when the caller brought room for the re-laid B
+// (a grouped launch needs `count` such buffers, one behind the other)
 static bool onthefly_prepare_ok(const Problem& q, int count, const void* const* A, const void* const* B,
                                 const void* workspace, size_t workspace_bytes) {
-  if (q.bpre || count != 1 || q.dtype == CASCMM_DT_F32 || q.terms != 1 || q.K % 64 != 0 || !A[0] || !B[0]) return false;
+  if (q.bpre || q.dtype == CASCMM_DT_F32 || q.terms != 1 || q.K % 64 != 0) return false;
   if (!((q.dtype == CASCMM_DT_F16 && q.fmt == CASCMM_FMT_FP16) || (q.dtype == CASCMM_DT_BF16 && q.fmt == CASCMM_FMT_BF16)))
     return false;
-  if (q.lda % 8 != 0 || !aligned_to(A[0], 16) || !aligned_to(B[0], 2)) return false;
+  if (q.lda % 8 != 0) return false;
+  for (int i = 0; i < count; ++i)
+    if (!A[i] || !B[i] || !aligned_to(A[i], 16) || !aligned_to(B[i], 2)) return false;
   const int64_t need = prepared_bytes(q.K, q.N, q.fmt, 1);
-  return workspace && aligned_to(workspace, 16) && need <= INT32_MAX && workspace_bytes >= (size_t)need;
+  return workspace && aligned_to(workspace, 16) && need <= INT32_MAX && workspace_bytes >= (size_t)need * count;
 }
 
 // One launch for `count` problems of one shape (count == 1: a plain GEMM).
@@ -375,13 +378,25 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   if (onthefly_prepare_ok(q, count, A, B, workspace, workspace_bytes)) {
     // fp16 x fp16 (bf16 x bf16) tensors as one term: re-lay B as operand slots in the workspace
     // (one pass over B), then the copy-only kernels
-    st = cascmm_prepare_weight(B[0], q.K, q.N, q.ldb, q.dtype, q.fmt, 1, nullptr, workspace, workspace_bytes, (void*)stream);
-    if (st != CASCMM_OK) return st;
+    const size_t each = (size_t)prepared_bytes(q.K, q.N, q.fmt, 1);
+    const void* bp[kMaxGroup];
+    for (int i = 0; i < count; ++i) {
+      void* dst = (char*)workspace + (size_t)i * each;
+      bp[i] = dst;
+      int same = -1;   // the same weight twice in one group is prepared once
+      for (int j = 0; j < i && same < 0; ++j)
+        if (B[j] == B[i]) same = j;
+      if (same >= 0) {
+        bp[i] = bp[same];
+        continue;
+      }
+      st = cascmm_prepare_weight(B[i], q.K, q.N, q.ldb, q.dtype, q.fmt, 1, nullptr, dst, each, (void*)stream);
+      if (st != CASCMM_OK) return st;
+    }
     Problem qp = q;
     qp.bpre = true;
     qp.ldb = q.N;
-    const void* bp = workspace;
-    const int r = gemm_impl(1, A, &bp, C, bias, qp, tensor_exps, nullptr, 0, stream, variant < 0 ? -1 : variant);
+    const int r = gemm_impl(count, A, bp, C, bias, qp, tensor_exps, nullptr, 0, stream, variant < 0 ? -1 : variant);
     if (r != CASCMM_ERR_BAD_FORMAT && r != CASCMM_ERR_BAD_VARIANT) return r;
   }
   bool fast = true;

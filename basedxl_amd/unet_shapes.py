@@ -85,27 +85,38 @@ def total_flops(shapes: List[LinearShape]) -> float:
 
 
 def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool = False, iters: int = 10,
-                seed: int = 0, static_scales: bool = False, geglu: str = "off") -> List[dict]:
+                seed: int = 0, static_scales: bool = False, geglu: str = "off", dtype: str = "fp32",
+                torch_matmul: bool = False) -> List[dict]:
     """Times every shape on cuda:0 (HIP-graph replay of `iters` launches, random fp32 operands:
     activations N(0,1), weights 0.02 N(0,1)); returns one record per shape.  ``geglu``: what is
     timed for the gated projections: "off" the GEMM alone, "unfused" the GEMM plus torch's
-    ``value * gelu(gate)``, "fused" the kernel that applies the gate in its store."""
+    ``value * gelu(gate)``, "fused" the kernel that applies the gate in its store.  ``dtype``: element
+    type of the tensors ("fp16" is what the reference runs its UNet in); ``torch_matmul``: time
+    ``torch.matmul`` (the vendor GEMM library) on the same tensors instead of the cascade kernels."""
     import torch
 
     from . import PreparedWeight, cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, cascaded_lowp_matmul_prepared
 
     dev = torch.device("cuda:0")
+    tdt = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}[dtype]
     g = torch.Generator(device="cpu").manual_seed(seed)
     rows = []
     for s in shapes:
-        a = torch.randn(s.M, s.K, generator=g).to(dev)
-        ws = [(torch.randn(s.K, s.N, generator=g) * 0.02).to(dev) for _ in range(s.group)]
-        outs = [torch.empty(s.M, s.N, device=dev) for _ in range(s.group)]
+        a = torch.randn(s.M, s.K, generator=g).to(dev).to(tdt)
+        ws = [(torch.randn(s.K, s.N, generator=g) * 0.02).to(dev).to(tdt) for _ in range(s.group)]
+        outs = [torch.empty(s.M, s.N, device=dev, dtype=tdt) for _ in range(s.group)]
         use_prepared = prepared and s.K % 64 == 0 and s.N % 4 == 0
         gate = geglu if s.gated else "off"
-        if gate == "fused":
+        if torch_matmul:
+            use_prepared = False
+            gate = "unfused" if gate == "fused" else gate
+
+            def run():
+                for i in range(s.group):
+                    torch.matmul(a, ws[i], out=outs[i])
+        elif gate == "fused":
             pw = PreparedWeight(ws[0], lowp=lowp, terms=terms, glu=True)
-            gated_out = torch.empty(s.M, s.N // 2, device=dev)
+            gated_out = torch.empty(s.M, s.N // 2, device=dev, dtype=tdt)
             use_prepared = True
 
             def run():
@@ -131,7 +142,7 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
             def run():
                 cascaded_lowp_matmul(a, ws[0], out=outs[0], lowp=lowp, terms=terms)
         if gate == "unfused":
-            gemm, gated_out = run, torch.empty(s.M, s.N // 2, device=dev)
+            gemm, gated_out = run, torch.empty(s.M, s.N // 2, device=dev, dtype=tdt)
 
             def run():
                 gemm()
@@ -176,6 +187,9 @@ def main(argv=None) -> None:
     ap.add_argument("--static-scales", action="store_true", help="fp8: tensor scales found once, not in every call")
     ap.add_argument("--geglu", choices=["off", "unfused", "fused"], default="off",
                     help="gated projections: time the GEMM alone, with torch's gate after it, or the fused kernel")
+    ap.add_argument("--dtype", choices=["fp32", "fp16", "bf16"], default="fp32",
+                    help="element type of activations, weights and results (use --cascades fp16x1 / bf16x1 with 16-bit tensors)")
+    ap.add_argument("--torch-matmul", action="store_true", help="time torch.matmul on the same tensors instead")
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args(argv)
     shapes = sdxl_linear_shapes(args.batch, args.latent, args.half_latent, convs=args.convs)
@@ -185,12 +199,13 @@ def main(argv=None) -> None:
     for casc in args.cascades.split(","):
         lowp, terms = casc.split("x")
         rows = time_shapes(shapes, lowp, int(terms), prepared=args.prepared, static_scales=args.static_scales,
-                           geglu=args.geglu)
+                           geglu=args.geglu, dtype=args.dtype, torch_matmul=args.torch_matmul)
         total_us = sum(r["us_per_step"] for r in rows)
         summary["cascades"][casc] = {"linear_ms_per_step": round(total_us * 1e-3, 3),
                                      "tflops_fp32_equiv": round(flops / total_us * 1e-6, 1), "shapes": rows}
         if not args.json:
-            print(f"== {casc}{' (prepared weights)' if args.prepared else ''}: {total_us * 1e-3:.3f} ms of Linear work per "
+            label = f"torch.matmul {args.dtype}" if args.torch_matmul else f"{casc} on {args.dtype} tensors"
+            print(f"== {label}{' (prepared weights)' if args.prepared else ''}: {total_us * 1e-3:.3f} ms of Linear work per "
                   f"UNet step, {flops / total_us * 1e-6:.1f} TFLOP/s fp32-equivalent")
             for r in rows:
                 print(f"  {r['name']:50s} x{r['count']:3d}  [{r['M']:6d} x {r['K']:5d}] x [{r['K']:5d} x {r['N']:5d}]"

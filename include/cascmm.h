@@ -100,7 +100,9 @@ int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,
  * several weights).  The kernels are persistent, so the launch gap and the cold first loads of
  * every GEMM after the first disappear.  Counterpart in the reference: the fused to_k/to_v
  * Linear of basedxl/modules/attn.py:23-39, which gets the same effect by concatenating the
- * weights; here the weights stay separate tensors. */
+ * weights; here the weights stay separate tensors.  fp16 / bf16 tensors as one term of their
+ * own format take their fast path when the workspace holds count * cascmm_workspace_bytes(...)
+ * (every distinct B[i] is re-laid there). */
 int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, void* const* C,
                         const void* const* bias,
                         int64_t M, int64_t N, int64_t K,

@@ -694,3 +694,21 @@ def test_wrapper_shapes_like_the_reference(gpu_device):
     assert torch.equal(r5.reshape(30, 48), r4.reshape(30, 48))
     at = _gpu(torch.randn(64, 40, generator=g)).t()          # [40, 64] with a column stride: made contiguous like :158
     torch.testing.assert_close(cascaded_lowp_matmul(at, b), (at.double() @ b.double()).float(), rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_grouped_sixteen_bit_launch_takes_the_fast_path(gpu_device, dtype):
+    """q/k/v of 16-bit tensors in one launch: every right operand is re-laid in the workspace and
+    the copy-only kernels run; results equal the single launches (same kernels, same order of
+    accumulation per tile when the same tile is chosen, else one 16-bit ulp)."""
+    g = torch.Generator().manual_seed(61)
+    a = _gpu(torch.randn(512, 640, generator=g)).to(dtype)
+    ws = [_gpu(torch.randn(640, 640, generator=g) * 0.05).to(dtype) for _ in range(3)]
+    outs = cascaded_lowp_matmul_grouped([a, a, a], [ws[0], ws[1], ws[0]])
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for o, w in zip(outs, [ws[0], ws[1], ws[0]]):
+        single = cascaded_lowp_matmul(a, w)
+        want = oc.fp64_matmul(a.cpu().float(), w.cpu().float())
+        assert bool(((o.float() - single.float()).abs() <= ulp * single.float().abs() + 1e-3).all())
+        assert bool(((o.cpu().double() - want).abs() <= ulp * want.abs() + 1e-3).all())
+    assert torch.equal(outs[0], outs[2])
