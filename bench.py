@@ -1,18 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the cascaded low-precision matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload ffn|attn]
 
-One "step" is one pass of the hot path over the SDXL 64x64-stage self-attention
-projections on one GPU's patch share: X fp32 [M = 2 x 2048 tokens, K = 640] through four
-independent Linear weights W fp32 [640, 640] (to_q, to_k, to_v from X, to_out from a second
-activation tensor of the same shape), each as a 2-term bf16 cascade with the three products
-hi.hi + hi.lo + lo.hi, fp32 accumulation.  Inputs are synthetic (seeded normal) and resident
-in HBM before the timed region.  Both operands are split inside the timed kernels.
+One "step" is one pass of the hot path over one batch of synthetic input:
 
-Prints ONE JSON line: the whole-job fp32-equivalent throughput (2*M*N*K per GEMM, whatever
-the term count), the roofline of the GEMM kernel measured live with events on the stream the
-kernels run on, and the CPU oracle timed on this host's cores on a bounded sample.
+* ``--workload ffn`` (default; the shape the headline metric is quoted on): the GEGLU feed-forward
+  block of the SDXL 32x32 stage, full image: X fp32 [M = 2 x 1024 tokens, K = 1280] x W1 fp32
+  [1280, 10240], then G fp32 [2048, 5120] x W2 fp32 [5120, 1280] -- two GEMMs per step;
+* ``--workload attn``: the self-attention projections of the 64x64 stage on one GPU's patch share:
+  X fp32 [M = 2 x 2048 tokens, K = 640] through four Linear weights W fp32 [640, 640] (to_q, to_k,
+  to_v from X in one grouped launch, to_out from a second activation tensor).
+
+Every GEMM is a 2-term bf16 cascade with the three products hi.hi + hi.lo + lo.hi and fp32
+accumulation.  Inputs are synthetic (seeded normal; weights x 0.02) and resident in HBM before the
+timed region.  Both operands are split inside the timed kernels.
+
+Prints ONE JSON line: the whole-job fp32-equivalent throughput (2*M*N*K per GEMM, whatever the term
+count), the roofline of the GEMM kernel that takes most of the step, measured live with events on
+the stream the kernels run on, and the CPU oracle timed on this host's cores on a bounded sample.
 """
 from __future__ import annotations
 
@@ -26,40 +32,79 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-M, K, N = 4096, 640, 640
-N_PROJ = 4
 TERMS, PRODUCTS_PER_ELEMENT = 2, 3  # bf16 hi/lo, tri product set
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
-# HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
-# summary under profiles/ gives the commands and the calibration); keyed by (--group, GEMMs).
-TRAFFIC_BYTES_PER_LAUNCH = {("qkv+o", 3): 2 * 21945.3 * 1024 + 30720.0 * 1024}
 SEED = 1
+METRIC = {"ffn": "fp32-equiv TFLOP/s + % of MFMA roofline at SDXL FFN shape; rel-Frobenius err",
+          "attn": "fp32-equiv TFLOP/s + % of MFMA roofline at SDXL self-attention projection shape; rel-Frobenius err"}
+# HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
+# summaries under profiles/ give the commands and the calibration); keyed by (workload, launch label).
+TRAFFIC_BYTES_PER_LAUNCH = {
+    ("ffn", "ff.net.0.proj (W1)"): 2 * 94514.0 * 1024 + 90624.0 * 1024,
+    ("attn", "to_q/to_k/to_v grouped"): 2 * 21930.0 * 1024 + 30720.0 * 1024,
+}
 
 
-def make_inputs(device):
+class Launch:
+    """One kernel launch of a step: `gemms` problems of one shape (a_list[i] x w_list[i] -> outs[i])."""
+
+    def __init__(self, label, M, K, N, a_idx, w_idx):
+        self.label, self.M, self.K, self.N = label, M, K, N
+        self.a_idx, self.w_idx = a_idx, w_idx     # indices into a buffer set's activations / weights
+        self.gemms = len(w_idx)
+
+    @property
+    def flops(self):            # fp32-equivalent
+        return 2.0 * self.M * self.N * self.K * self.gemms
+
+    @property
+    def algorithmic_bytes(self):   # every distinct operand once, every result once
+        return 4 * (len(set(self.a_idx)) * self.M * self.K + self.gemms * (self.K * self.N + self.M * self.N))
+
+
+def workload(name, group):
+    """(description, activation shapes, weight shapes, launches) of one step."""
+    if name == "ffn":
+        acts = [(2048, 1280), (2048, 5120)]
+        wts = [(1280, 10240), (5120, 1280)]
+        launches = [Launch("ff.net.0.proj (W1)", 2048, 1280, 10240, [0], [0]), Launch("ff.net.2 (W2)", 2048, 5120, 1280, [1], [1])]
+        desc = ("cfg3: SDXL 32x32-stage GEGLU FFN, full image: X fp32 [2048,1280] ~N(0,1) x W1 fp32 [1280,10240] ~N(0,0.02), "
+                "then G fp32 [2048,5120] ~N(0,1) x W2 fp32 [5120,1280] ~N(0,0.02) (a synthetic second input, not the gated "
+                "output of the first GEMM); hi=bf16(x), lo=bf16(x-hi), products hi.hi+hi.lo+lo.hi, fp32 accumulate, fp32 out")
+        return desc, acts, wts, launches
+    acts = [(4096, 640), (4096, 640)]
+    wts = [(640, 640)] * 4
+    if group == "qkv+o":
+        launches = [Launch("to_q/to_k/to_v grouped", 4096, 640, 640, [0, 0, 0], [0, 1, 2]), Launch("to_out", 4096, 640, 640, [1], [3])]
+    elif group == "all":
+        launches = [Launch("q/k/v/out grouped", 4096, 640, 640, [0, 0, 0, 1], [0, 1, 2, 3])]
+    else:
+        launches = [Launch(n, 4096, 640, 640, [a], [w]) for n, a, w in (("to_q", 0, 0), ("to_k", 0, 1), ("to_v", 0, 2), ("to_out", 1, 3))]
+    desc = ("cfg2: SDXL 64x64-stage self-attention projections on one GPU's patch share: X fp32 [4096,640] ~N(0,1) x W fp32 "
+            "[640,640] ~N(0,0.02), q/k/v/out = 4 GEMMs per step; hi=bf16(x), lo=bf16(x-hi), products hi.hi+hi.lo+lo.hi, "
+            "fp32 accumulate, fp32 out")
+    return desc, acts, wts, launches
+
+
+def make_inputs(acts, wts, device):
     import torch
 
     g = torch.Generator().manual_seed(SEED)
-    x = torch.randn(M, K, generator=g, dtype=torch.float32)
-    y = torch.randn(M, K, generator=g, dtype=torch.float32)
-    ws = [torch.randn(K, N, generator=g, dtype=torch.float32) * 0.02 for _ in range(N_PROJ)]
-    cpu = (x, y, ws)
-    dev = (x.to(device), y.to(device), [w.to(device) for w in ws])
-    return cpu, dev
+    a_cpu = [torch.randn(m, k, generator=g, dtype=torch.float32) for m, k in acts]
+    w_cpu = [torch.randn(k, n, generator=g, dtype=torch.float32) * 0.02 for k, n in wts]
+    return (a_cpu, w_cpu), ([a.to(device) for a in a_cpu], [w.to(device) for w in w_cpu])
 
 
-def cpu_baseline(cpu_inputs, repeats=5):
+def cpu_baseline(cpu_inputs, launches, repeats=5):
     """The oracle's CPU emulation of the same step, timed on this host (rank 0, N = 1)."""
     import torch
     from oracle import cascade as oc
 
-    x, y, ws = cpu_inputs
+    a_cpu, w_cpu = cpu_inputs
     torch.set_num_threads(min(os.cpu_count() or 1, 16))
 
     def step():
-        outs = [oc.cascade_matmul_ref(x, ws[i], "bf16", 2, "tri") for i in range(3)]
-        outs.append(oc.cascade_matmul_ref(y, ws[3], "bf16", 2, "tri"))
-        return outs
+        return [oc.cascade_matmul_ref(a_cpu[a], w_cpu[w], "bf16", 2, "tri") for ln in launches for a, w in zip(ln.a_idx, ln.w_idx)]
 
     step()
     times = []
@@ -70,12 +115,12 @@ def cpu_baseline(cpu_inputs, repeats=5):
     times.sort()
     med = times[len(times) // 2]
     return {
-        "value": round(N_PROJ * 2.0 * M * N * K / med * 1e-12, 4),
+        "value": round(sum(ln.flops for ln in launches) / med * 1e-12, 4),
         "unit": "TFLOP/s fp32-equiv",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{repeats} timed repeats (median) of the full 4-projection step, torch CPU emulation: "
-                  f"split + 3 fp32 matmuls per projection; {med * 1e3:.1f} ms per step",
+        "sample": f"{repeats} timed repeats (median) of the full step ({sum(ln.gemms for ln in launches)} GEMMs), torch CPU "
+                  f"emulation: split + 3 fp32 matmuls per GEMM; {med * 1e3:.1f} ms per step",
     }
 
 
@@ -84,16 +129,20 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=["ffn", "attn"], default="ffn",
+                    help="ffn: the two GEMMs of the 32x32-stage GEGLU feed-forward block (the shape the metric is quoted on); "
+                         "attn: the four 64x64-stage self-attention projections of one GPU's patch share")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--group", choices=["qkv+o", "all", "none"], default="qkv+o",
-                    help="how the four GEMMs of a step are launched: to_q/to_k/to_v (same input) as one grouped launch "
-                         "plus to_out on its own (default), all four in one grouped launch, or four separate launches")
+                    help="attn only: how the four GEMMs of a step are launched: to_q/to_k/to_v (same input) as one grouped "
+                         "launch plus to_out on its own (default), all four in one grouped launch, or four separate launches")
     ap.add_argument("--streams", type=int, default=1,
-                    help="number of HIP streams the four independent GEMMs of a step are spread over")
+                    help="number of HIP streams the launches of a step are spread over (attn --group none: the four "
+                         "GEMMs are independent)")
     ap.add_argument("--rotate", type=int, default=1,
-                    help="number of distinct input/weight/output buffer sets the steps cycle through (1 = the same "
-                         "70 MB every step, resident in the Infinity Cache; 8 = 560 MB, every step reads HBM-cold data)")
+                    help="number of distinct input/weight/output buffer sets the steps cycle through (1 = the same buffers "
+                         "every step, resident in the Infinity Cache; 8 = every step reads HBM-cold data)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -109,47 +158,57 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
-    cpu_in, (x, y, ws) = make_inputs(dev)
-    outs = [torch.empty(M, N, device=dev, dtype=torch.float32) for _ in range(N_PROJ)]
+    desc, acts, wts, launches = workload(args.workload, args.group)
+    cpu_in, (a_dev, w_dev) = make_inputs(acts, wts, dev)
 
-    ins = [x, x, x, y]
+    def out_buffers():
+        return [[torch.empty(ln.M, ln.N, device=dev, dtype=torch.float32) for _ in range(ln.gemms)] for ln in launches]
+
     # --rotate R: R - 1 further copies of every buffer; step i uses set i % R
-    sets = [(ins, ws, outs)]
+    sets = [(a_dev, w_dev, out_buffers())]
     for _ in range(max(1, args.rotate) - 1):
-        x2, y2 = x.clone(), y.clone()
-        sets.append(([x2, x2, x2, y2], [w.clone() for w in ws], [torch.empty_like(o) for o in outs]))
+        sets.append(([a.clone() for a in a_dev], [w.clone() for w in w_dev], out_buffers()))
+    set_bytes = sum(t.numel() * 4 for t in a_dev + w_dev) + sum(o.numel() * 4 for lo in sets[0][2] for o in lo)
     step_no = [0]
-    extra = [torch.cuda.Stream() for _ in range(max(0, min(args.streams, N_PROJ) - 1))]
+    extra = [torch.cuda.Stream() for _ in range(max(0, min(args.streams, len(launches)) - 1))]
+
+    def run_launch(i, bufs):
+        a, w, o = bufs
+        ln = launches[i]
+        if ln.gemms == 1:
+            cascaded_lowp_matmul(a[ln.a_idx[0]], w[ln.w_idx[0]], out=o[i][0])
+        else:
+            cascaded_lowp_matmul_grouped([a[j] for j in ln.a_idx], [w[j] for j in ln.w_idx], outs=o[i])
 
     def step():
-        # the four projections are independent GEMMs; with --streams > 1 they are enqueued on
-        # several streams (forked from and joined back into the current one) so that the tail
-        # of one kernel overlaps the start of the next
-        ins, ws, outs = sets[step_no[0] % len(sets)]
+        # with --streams > 1 the launches are enqueued on several streams (forked from and joined
+        # back into the current one) so that the tail of one kernel overlaps the start of the next
+        bufs = sets[step_no[0] % len(sets)]
         step_no[0] += 1
-        if args.group == "qkv+o":
-            cascaded_lowp_matmul_grouped(ins[:3], ws[:3], outs=outs[:3])
-            cascaded_lowp_matmul(ins[3], ws[3], out=outs[3])
-            return
-        if args.group == "all":
-            cascaded_lowp_matmul_grouped(ins, ws, outs=outs)
+        if not extra:
+            for i in range(len(launches)):
+                run_launch(i, bufs)
             return
         cur = torch.cuda.current_stream()
         lanes = [cur] + extra
         for s_ in extra:
             s_.wait_stream(cur)
-        for i in range(N_PROJ):
+        for i in range(len(launches)):
             with torch.cuda.stream(lanes[i % len(lanes)]):
-                cascaded_lowp_matmul(ins[i], ws[i], out=outs[i])
+                run_launch(i, bufs)
         for s_ in extra:
             cur.wait_stream(s_)
 
-    # correctness of what is being timed: error vs fp64 next to the oracle cascade's error
+    # correctness of what is being timed: error vs fp64 next to the oracle cascade's error, on
+    # the last GEMM of the step (the smaller one of the ffn workload: the CPU side takes seconds)
     step()
     torch.cuda.synchronize()
-    exp = oc.fp64_matmul(cpu_in[1], cpu_in[2][3])
-    err_k = oc.error_metrics(outs[3].cpu(), exp)
-    err_o = oc.error_metrics(oc.cascade_matmul_ref(cpu_in[1], cpu_in[2][3], "bf16", 2, "tri"), exp)
+    chk = launches[-1]
+    a_chk, w_chk = cpu_in[0][chk.a_idx[-1]], cpu_in[1][chk.w_idx[-1]]
+    exp = oc.fp64_matmul(a_chk, w_chk)
+    err_k = oc.error_metrics(sets[0][2][-1][-1].cpu(), exp)
+    err_o = oc.error_metrics(oc.cascade_matmul_ref(a_chk, w_chk, "bf16", 2, "tri"), exp)
+    del exp
     if not (err_k["rel_fro"] <= 1.25 * err_o["rel_fro"] and err_k["max_abs"] <= 1.25 * err_o["max_abs"]):
         sys.exit(f"bench.py: kernel error {err_k} exceeds 1.25x the oracle cascade's {err_o}")
 
@@ -186,7 +245,7 @@ def main():
     # above leave it idle for seconds): untimed replays for about 0.3 s, then the W warm-up steps
     t_spin = time.perf_counter()
     while time.perf_counter() - t_spin < 0.3:
-        for _ in range(20):
+        for _ in range(5):
             run()
         torch.cuda.synchronize()
     for _ in range(max(1, args.warmup // per_graph)):
@@ -203,7 +262,7 @@ def main():
     ev_ms = e0.elapsed_time(e1)
 
     ms_per_step = wall * 1e3 / args.steps
-    flops_step = N_PROJ * 2.0 * M * N * K
+    flops_step = sum(ln.flops for ln in launches)
     value = flops_step / (wall / args.steps) * 1e-12
 
     # The kernels of a step, each timed on its own: a graph that holds that launch REPS times
@@ -212,16 +271,17 @@ def main():
     # object describes the one that takes most of the step.
     REPS = 10
     l = _lib.lib()
-    kinds = {"qkv+o": [("to_q/to_k/to_v grouped", 3, lambda: cascaded_lowp_matmul_grouped(ins[:3], ws[:3], outs=outs[:3])),
-                       ("to_out", 1, lambda: cascaded_lowp_matmul(ins[3], ws[3], out=outs[3]))],
-             "all": [("q/k/v/out grouped", 4, lambda: cascaded_lowp_matmul_grouped(ins, ws, outs=outs))],
-             "none": [("one projection", 1, lambda: cascaded_lowp_matmul(ins[3], ws[3], out=outs[3]))]}[args.group]
     per_kernel = []
-    for label, gemms, fn in kinds:
+    seen = {}
+    for i, ln in enumerate(launches):
+        key = (ln.M, ln.K, ln.N, ln.gemms)
+        if key in seen:      # same shape and group size: the same kernel (attn --group none)
+            seen[key]["launches_per_step"] += 1
+            continue
         g1 = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g1):
             for _ in range(REPS):
-                fn()
+                run_launch(i, sets[0])
         nrep = max(1, args.steps // REPS)
         for _ in range(max(1, args.warmup // REPS)):
             g1.replay()
@@ -233,21 +293,24 @@ def main():
         k1.record()
         torch.cuda.synchronize()
         us = k0.elapsed_time(k1) * 1e3 / (nrep * REPS)
-        vidx = l.cascmm_select_variant_grouped(gemms, M, N, K, K, N, N, 0, 0, 2, 0)
-        per_kernel.append({
-            "launch": label, "gemms": gemms, "kernel": l.cascmm_variant_name(vidx).decode(), "launch_us": round(us, 3),
-            "launches_per_step": (N_PROJ if args.group == "none" else 1),
-            "flops_per_launch": PRODUCTS_PER_ELEMENT * 2.0 * M * N * K * gemms,
-            "algorithmic_bytes_per_launch": 4 * (M * K + gemms * (K * N + M * N)),
-            "mfma_tflops": round(PRODUCTS_PER_ELEMENT * 2.0 * M * N * K * gemms / (us * 1e-6) * 1e-12, 2),
-            "fp32_equiv_tflops": round(2.0 * M * N * K * gemms / (us * 1e-6) * 1e-12, 2),
-        })
+        vidx = l.cascmm_select_variant_grouped(ln.gemms, ln.M, ln.N, ln.K, ln.K, ln.N, ln.N, 0, 0, 2, 0)
+        rec = {
+            "launch": ln.label, "gemms": ln.gemms, "M": ln.M, "K": ln.K, "N": ln.N,
+            "kernel": l.cascmm_variant_name(vidx).decode(), "launch_us": round(us, 3), "launches_per_step": 1,
+            "flops_per_launch": PRODUCTS_PER_ELEMENT * ln.flops,
+            "algorithmic_bytes_per_launch": ln.algorithmic_bytes,
+            "mfma_tflops": round(PRODUCTS_PER_ELEMENT * ln.flops / (us * 1e-6) * 1e-12, 2),
+            "fp32_equiv_tflops": round(ln.flops / (us * 1e-6) * 1e-12, 2),
+        }
+        seen[key] = rec
+        per_kernel.append(rec)
     dom = max(per_kernel, key=lambda r: r["launch_us"] * r["launches_per_step"])
-    launches_per_step = {"qkv+o": 2, "all": 1, "none": N_PROJ}[args.group]
-    vname = dom["kernel"]
+    cache = (f"same buffers every step ({set_bytes / 1e6:.0f} MB working set, resident in the 256 MB Infinity Cache)"
+             if len(sets) == 1 else
+             f"{len(sets)} buffer sets in rotation ({set_bytes * len(sets) / 1e6:.0f} MB: inputs and weights come from HBM)")
 
     result = {
-        "metric": "fp32-equiv TFLOP/s, 2-term bf16 cascade, SDXL 64x64-stage self-attn projections (one GPU's patch share)",
+        "metric": METRIC[args.workload],
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -260,27 +323,23 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": "cfg2: X fp32 [4096,640] ~N(0,1) x W fp32 [640,640] ~N(0,0.02), q/k/v/out = 4 GEMMs per step, "
-                        "hi=bf16(x), lo=bf16(x-hi), products hi.hi+hi.lo+lo.hi, fp32 accumulate, fp32 out",
-            "M": M, "N": N, "K": K, "gemms_per_step": N_PROJ, "terms": TERMS, "products": "tri",
+            "workload": desc,
+            "gemms": [{"M": ln.M, "K": ln.K, "N": ln.N, "count": ln.gemms} for ln in launches],
+            "gemms_per_step": sum(ln.gemms for ln in launches), "terms": TERMS, "products": "tri",
             "launch": (f"hip graph replay ({per_graph} steps per graph)" if graph is not None else "python ctypes")
-                      + f", {len(extra) + 1} stream(s), "
-                      + {"qkv+o": "2 launches per step: to_q/to_k/to_v grouped (3 GEMMs, one activation tensor) + to_out",
-                         "all": "1 grouped launch per step (4 GEMMs)", "none": "4 launches per step"}[args.group],
-            "launches_per_step": launches_per_step,
-            "kernel": vname, "seed": SEED,
-            "cache_regime": ("same buffers every step (70 MB working set, resident in the 256 MB Infinity Cache)"
-                             if len(sets) == 1 else
-                             f"{len(sets)} buffer sets in rotation ({70 * len(sets)} MB: inputs and weights come from HBM)"),
+                      + f", {len(extra) + 1} stream(s), {len(launches)} launches per step: " + " + ".join(ln.label for ln in launches),
+            "launches_per_step": len(launches),
+            "kernel": dom["kernel"], "seed": SEED,
+            "cache_regime": cache,
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": dom["kernel"] + " (" + dom["launch"] + ", " + str(dom["gemms"]) + " GEMMs per launch)",
+            "kernel": dom["kernel"] + " (" + dom["launch"] + ", " + str(dom["gemms"]) + " GEMM(s) per launch)",
             "achieved": dom["mfma_tflops"],
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(dom["mfma_tflops"] / PEAK_BF16_TFLOPS, 4),
-            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.group, dom["gemms"])),
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dom["launch"])),
             "traffic_is": "HBM-side bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE "
                           "(x1.0), factors from a 256 MiB copy in the same runs; see profiles/",
             "launch_us": dom["launch_us"],
@@ -293,11 +352,11 @@ def main():
             "step_time_us_from_events": round(ev_ms * 1e3 / args.steps, 3),
             "kernels_of_a_step": per_kernel,
         },
-        "error": {"kernel_rel_fro": err_k["rel_fro"], "oracle_rel_fro": err_o["rel_fro"],
+        "error": {"checked_gemm": chk.label, "kernel_rel_fro": err_k["rel_fro"], "oracle_rel_fro": err_o["rel_fro"],
                   "kernel_max_abs": err_k["max_abs"], "oracle_max_abs": err_o["max_abs"]},
     }
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cpu_in)
+        result["cpu_baseline"] = cpu_baseline(cpu_in, launches)
     print(json.dumps(result))
 
 
