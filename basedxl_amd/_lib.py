@@ -34,7 +34,7 @@ SIGNATURES = {
     "cascmm_prepare_weight": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p,
                                       c_size_t, c_void_p]),
     "cascmm_gemm_prepared": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 5 + [c_int] * 4
-                             + [c_void_p, c_void_p, c_int]),
+                             + [c_void_p, c_void_p, c_size_t, c_void_p, c_int]),
     "cascmm_prepare_weight_glu": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p,
                                           c_size_t, c_void_p]),
     "cascmm_gemm_prepared_glu": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 5 + [c_int] * 4

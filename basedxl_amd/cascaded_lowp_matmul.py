@@ -171,9 +171,18 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
             _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _DTYPES[adt], exps.data_ptr() + 8 * i,
                                                     stream), "cascmm_tensor_exp(A)")
             exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
-    gemm = _lib.lib().cascmm_gemm_prepared_glu if w0.glu else _lib.lib().cascmm_gemm_prepared
-    st = gemm(n, pa, pb, pc, pbias, M, N, K, lda, max(NO, 1), _DTYPES[adt], w0.fmt, w0.terms,
-              _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None, stream, variant)
+    common = (n, pa, pb, pc, pbias, M, N, K, lda, max(NO, 1), _DTYPES[adt], w0.fmt, w0.terms,
+              _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None)
+    if w0.glu:
+        st = _lib.lib().cascmm_gemm_prepared_glu(*common, stream, variant)
+    else:
+        # room for the partial results of a K split (single fp32 problems with few tiles)
+        ws = None
+        if n == 1 and adt == torch.float32:
+            need = _lib.lib().cascmm_workspace_bytes(M, N, K, _DTYPES[adt], w0.fmt, w0.terms, _lib.PROD_BY_NAME[products])
+            ws = _workspace(dev, stream, need)
+        st = _lib.lib().cascmm_gemm_prepared(*common, ws.data_ptr() if ws is not None else None,
+                                             ws.numel() if ws is not None else 0, stream, variant)
     _lib.check(st, "cascmm_gemm_prepared")
     return [o.reshape(*a.shape[:-1], NO) for o, a in zip(outs, a_list)]
 

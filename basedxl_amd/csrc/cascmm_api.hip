@@ -100,13 +100,14 @@ static const TunedCost kTuned[] = {
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.224, 6.84, 0.80, 0.70},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri", 2.907, 13.81, 0.70, 0.50},
     // right operand prepared (sweep over M in 1024..8192 of the UNet's (K, N) pairs)
-    {"t64x160x64_w2x1x2_d2_bf16x2_tri_bpre", 0.817, 5.30, 1.00, 0.80},
-    {"t64x160x64_w2x1x2_d3_bf16x2_tri_bpre", 0.811, 5.90, 1.00, 0.90},
-    {"t128x128x64_w2x2x1_d2_bf16x2_tri_bpre", 1.105, 6.41, 0.90, 0.70},
-    {"t128x160x32_w2x1x2_d3_bf16x2_tri_bpre", 1.332, 8.84, 0.80, 0.50},
-    {"t256x128x32_w4x1x1_d2_bf16x2_tri_bpre", 1.926, 8.80, 0.80, 0.90},
-    {"t64x64x64_w2x2x1_d3_bf16x2_tri_bpre", 0.484, 1.88, 1.00, 1.00},
-    {"t64x256x32_w1x4x1_d3_bf16x2_tri_bpre", 1.128, 5.55, 0.90, 0.60},
+    {"t64x160x64_w2x1x2_d2_bf16x2_tri_bpre", 0.925, 5.57, 0.80, 0.60},
+    {"t64x160x64_w2x1x2_d3_bf16x2_tri_bpre", 0.891, 6.26, 0.90, 0.80},
+    {"t128x128x64_w2x2x1_d2_bf16x2_tri_bpre", 1.193, 6.27, 0.90, 0.80},
+    {"t128x160x32_w2x1x2_d3_bf16x2_tri_bpre", 1.501, 9.45, 0.70, 0.50},
+    {"t256x128x32_w4x1x1_d2_bf16x2_tri_bpre", 2.192, 9.64, 0.70, 0.70},
+    {"t64x64x64_w2x2x1_d3_bf16x2_tri_bpre", 0.515, 2.08, 1.00, 1.00},
+    {"t64x256x32_w1x4x1_d3_bf16x2_tri_bpre", 1.250, 5.89, 0.80, 0.50},
+    {"t256x160x32_w4x1x1_d2_bf16x2_tri_bpre", 2.837, 12.00, 0.60, 0.50},
 };
 
 constexpr int kMaxTileSplits = 4;
@@ -523,11 +524,12 @@ int cascmm_gemm_prepared_glu(int count, const void* const* A, const void* const*
 
 int cascmm_gemm_prepared(int count, const void* const* A, const void* const* Bprep, void* const* C,
                          const void* const* bias, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int dtype,
-                         int fmt, int terms, int products, const int32_t* tensor_exps, void* stream, int variant) {
+                         int fmt, int terms, int products, const int32_t* tensor_exps, void* workspace,
+                         size_t workspace_bytes, void* stream, int variant) {
   if (!A || !Bprep || !C) return CASCMM_ERR_NULL_POINTER;
   Problem q{M, N, K, lda, N, ldc, dtype, fmt, terms, products};
   q.bpre = true;
-  return gemm_impl(count, A, Bprep, C, bias, q, tensor_exps, nullptr, 0, (hipStream_t)stream, variant);
+  return gemm_impl(count, A, Bprep, C, bias, q, tensor_exps, workspace, workspace_bytes, (hipStream_t)stream, variant);
 }
 
 int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc, int dtype, int fmt,
@@ -537,7 +539,7 @@ int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, i
   q.bpre = true;
   const int st = check_problem(q);
   if (st != CASCMM_OK) return st;
-  return select_variant(q, fast_ok(q, nullptr, nullptr), count, 0);   // cascmm_gemm_prepared brings no workspace: no K split
+  return select_variant(q, fast_ok(q, nullptr, nullptr), count);
 }
 
 size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fmt, int terms, int products) {

@@ -121,8 +121,9 @@ int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, v
  * (device int32, NULL = 0) is the scale exponent applied before the split; pass the same value
  * as e_B in tensor_exps of the GEMM.
  * cascmm_gemm_prepared runs `count` (1..8) GEMMs C[i] = A[i] . B[i] (+ bias[i]) of one shape whose
- * right operands are prepared buffers; arguments as cascmm_gemm_grouped, without ldb and
- * workspace.  Only the fast kernels exist for it: A must be fp32 with 16-byte aligned rows
+ * right operands are prepared buffers; arguments as cascmm_gemm_grouped, without ldb (the
+ * workspace, which may be NULL, is used for the K split of under-filled single launches and
+ * holds cascmm_workspace_bytes(...)).  Only the fast kernels exist for it: A must be fp32 with 16-byte aligned rows
  * (CASCMM_ERR_ALIGNMENT otherwise), K a multiple of 32 or 64 depending on the kernel
  * (CASCMM_ERR_BAD_FORMAT when no kernel fits), the prepared buffer below 2 GiB
  * (CASCMM_ERR_TOO_LARGE).  The results equal cascmm_gemm's bit for bit when the same kernel
@@ -135,7 +136,8 @@ int cascmm_gemm_prepared(int count, const void* const* A, const void* const* Bpr
                          const void* const* bias,
                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
                          int dtype, int fmt, int terms, int products,
-                         const int32_t* tensor_exps, void* stream, int variant);
+                         const int32_t* tensor_exps,
+                         void* workspace, size_t workspace_bytes, void* stream, int variant);
 int cascmm_select_variant_prepared(int count, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
                                    int dtype, int fmt, int terms, int products);
 
