@@ -214,7 +214,9 @@ struct TileGemm {
     // other threads, so that every wave stages the same number of elements per K step.
     static constexpr int NQT = (HAS_A && HAS_Q && Q_UNITS < NTR) ? Q_UNITS : 0;   // threads with a B block
     static constexpr int A_LO_NUM = A_UNITS - 4 * (NTR - NQT);
-    static constexpr bool WEIGHTED = NQT > 0 && A_LO_NUM >= 0 && A_LO_NUM % NTR == 0 && NQT % kWave == 0;
+    // (not with twelve waves per workgroup: at three waves per SIMD a wave has 168 registers, and the
+    // A_HI-deep ring of the weighted deal makes the producer loop spill)
+    static constexpr bool WEIGHTED = NQT > 0 && A_LO_NUM >= 0 && A_LO_NUM % NTR == 0 && NQT % kWave == 0 && TL::NT <= 512;
     static constexpr int A_LO = WEIGHTED ? A_LO_NUM / NTR : 0, A_HI = A_LO + 4;
     static constexpr int A_IT = !HAS_A ? 0 : WEIGHTED ? A_HI : (A_UNITS + NTR - 1) / NTR;
     static constexpr bool A_ALL = !WEIGHTED && A_UNITS % NTR == 0;   // every thread has A_IT valid units
