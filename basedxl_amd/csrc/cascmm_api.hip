@@ -161,7 +161,24 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count, si
   // the plain B-direct kernels were slower than the LDS-tiled ones on every shape measured:
   // they stay selectable by index only
   if (name[0] == 'b' && name[1] == 'd') return 1e6 + rounds * step * ksteps;
-  return rounds * (step * ksteps + 5.0) + (v.fast ? 0.0 : 1e3);
+  double best = rounds * (step * ksteps + 5.0) + (v.fast ? 0.0 : 1e3);
+  // the same K split as above for the kernels without measured constants (three-term and fp8
+  // cascades on the shapes that leave CUs idle)
+  if (v.fast && count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0 && !q.glu && !q.bpre) {
+    const int64_t bk_steps = (q.K + v.BK - 1) / v.BK;
+    for (int sp = 2; sp <= kMaxTileSplits; ++sp) {
+      if (bk_steps % sp != 0 || bk_steps / sp < 4 || tiles * sp > kNumCUs) continue;
+      if (ws_bytes < (size_t)sp * q.M * q.N * sizeof(float)) continue;
+      const double r = 0.55 + 0.45 * tiles * sp / kNumCUs;
+      const double reduce_us = 2.0 + (double)(sp + 1) * q.M * q.N * 4.0 / 4.0e6;
+      const double c = r * (step * ksteps / sp + 5.0) + reduce_us;
+      if (c < best) {
+        best = c;
+        if (splits_out) *splits_out = sp;
+      }
+    }
+  }
+  return best;
 }
 
 // ws_bytes: workspace the caller brought (split-K variants that need more are skipped)
