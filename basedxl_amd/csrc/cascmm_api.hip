@@ -80,7 +80,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   return true;
 }
 
-// Cost model.  The two-term bf16 kernels, which carry the SDXL workload, are costed from
+// Cost model.  The two-term bf16 and three-term fp8 kernels, which carry the SDXL workload, are costed from
 // constants measured on MI355X (sweep over the UNet's Linear shapes, HIP-graph replay): a launch
 // takes  rounds x (K/64 x step64 + fixed)  microseconds, where a partly filled last round counts
 // as  tail + (1 - tail) x fill  of a full one, with one `tail` for a launch that has no full
@@ -99,6 +99,11 @@ static const TunedCost kTuned[] = {
     {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.064, 4.69, 0.90, 0.80},
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.224, 6.84, 0.80, 0.70},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri", 2.907, 13.81, 0.70, 0.50},
+    // three fp8 terms (static tensor scales)
+    {"t128x128x32_w4x2x1_d2_fp8x3_tri", 2.547, 6.33, 1.00, 0.90},
+    {"t64x64x64_w2x2x1_d2_fp8x3_tri", 1.016, 2.50, 1.00, 1.00},
+    {"t128x128x32_w2x2x1_d2_fp8x3_tri", 2.211, 6.93, 0.90, 0.80},
+    {"t64x128x64_w2x2x2_d2_fp8x3_tri", 1.409, 4.91, 1.00, 0.90},
     // right operand prepared (sweep over M in 1024..8192 of the UNet's (K, N) pairs)
     {"t64x160x64_w2x1x2_d2_bf16x2_tri_bpre", 0.925, 5.57, 0.80, 0.60},
     {"t64x160x64_w2x1x2_d3_bf16x2_tri_bpre", 0.891, 6.26, 0.90, 0.80},

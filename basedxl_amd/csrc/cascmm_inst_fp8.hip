@@ -10,6 +10,8 @@ static const VariantDesc kTable[] = {
     // three terms (12 significand bits), six products.  name, BM, BN, BK, WM, WN, WK, DEPTH
     CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp8x3_tri", 128, 128, 32, 4, 2, 1, 2, F32, F8, 3, false, true),
     CASCMM_TILE_VARIANT("t64x64x64_w2x2x1_d2_fp8x3_tri", 64, 64, 64, 2, 2, 1, 2, F32, F8, 3, false, true),
+    CASCMM_TILE_VARIANT("t128x128x32_w2x2x1_d2_fp8x3_tri", 128, 128, 32, 2, 2, 1, 2, F32, F8, 3, false, true),
+    CASCMM_TILE_VARIANT("t64x128x64_w2x2x2_d2_fp8x3_tri", 64, 128, 64, 2, 2, 2, 2, F32, F8, 3, false, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x3_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 3, false, false),
     CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp8x2_tri", 128, 128, 32, 4, 2, 1, 2, F32, F8, 2, false, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp8x2_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, F8, 2, false, false),
