@@ -30,7 +30,7 @@ struct TileBD {
   static constexpr int KSUB = BK / 16;
   static_assert(BM % 32 == 0, "BM");
   static_assert(BK == 32 || BK == 64, "BK");
-  static_assert(KSUB * 8 <= 60, "B loads of one K step must fit the vmcnt counter");
+  static_assert(KSUB * 8 <= 32, "the B loads of two K steps in flight must fit the vmcnt counter");
 };
 
 template <class TL, int TERMS>
@@ -164,25 +164,31 @@ struct BDirectGemm {
     }
     constexpr int kChunkSteps = (AC::kChunkK / TL::BK) > 0 ? (AC::kChunkK / TL::BK) : 1;
 
-    // raw B of one K step: KSUB slices x 8 k rows (this lane's k-group) of this lane's column
-    float raw[TL::KSUB][8];
-    auto load_b = [&](int kt) {
+    // raw B of a K step: KSUB slices x 8 k rows (this lane's k-group) of this lane's column; two
+    // steps are kept in flight (the loads of step kt + 2 are issued as soon as step kt is split)
+    float raw[2][TL::KSUB][8];
+    auto load_b = [&](int kt, float (&r)[TL::KSUB][8]) {
 #pragma unroll
       for (int sub = 0; sub < TL::KSUB; ++sub)
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          raw[sub][e] = llvm_raw_buffer_load_f32(rb, voff_b, (kt * TL::BK + sub * 16 + e) * ldb_bytes, 0);
+          r[sub][e] = llvm_raw_buffer_load_f32(rb, voff_b, (kt * TL::BK + sub * 16 + e) * ldb_bytes, 0);
     };
-    if (ktiles > 0) load_b(0);
+    if (ktiles > 0) load_b(0, raw[0]);
+    if (ktiles > 1) load_b(1, raw[1]);
 
     __syncthreads();
-    for (int kt = 0; kt < ktiles; ++kt) {
+    for (int kt2 = 0; kt2 < ktiles; kt2 += 2)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int kt = kt2 + half;
+      if (kt >= ktiles) break;
       const u32x4* sa = lds + (kt & 1) * LL::kStage;
-      // split this step's B (frees the raw registers), then refill them for the next step
+      // split this step's B (frees its raw registers), then refill them for the step after next
       u32x4 bt[TL::KSUB][TERMS];
 #pragma unroll
-      for (int sub = 0; sub < TL::KSUB; ++sub) split8<FMT, TERMS>(raw[sub], bt[sub]);
-      if (kt + 1 < ktiles) load_b(kt + 1);
+      for (int sub = 0; sub < TL::KSUB; ++sub) split8<FMT, TERMS>(raw[half][sub], bt[sub]);
+      if (kt + 2 < ktiles) load_b(kt + 2, raw[half]);
 #pragma unroll
       for (int sub = 0; sub < TL::KSUB; ++sub) {
         const int kg = sub * 2 + g;
