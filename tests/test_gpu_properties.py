@@ -102,3 +102,49 @@ def test_prepared_weight_has_the_same_properties(gpu_device, M, K, N):
     c = cascaded_lowp_matmul(a, pw)
     assert torch.equal(cascaded_lowp_matmul(a[pr].contiguous(), pw), c[pr])
     assert torch.equal(cascaded_lowp_matmul(a * 4.0, pw), c * 4.0)
+
+
+def test_random_shapes_strides_and_cascades_integer_exact(gpu_device):
+    """Seeded sweep over what a caller can vary at once -- M, N, K (odd sizes included), row
+    strides of A and of the result, leading batch dims, bias, dtype, cascade and product set -- with
+    the kernel left to the library's own selection.  Operands are small integers, so every cascade
+    that keeps enough products equals the integer matmul exactly (for 16-bit outputs: after one
+    rounding), whatever kernel, tile edge or K tail the case lands on."""
+    import numpy as np
+
+    from basedxl_amd import cascaded_lowp_matmul_grouped
+
+    rng = np.random.default_rng(20240607)
+    cascades = [("bf16", 1, "tri"), ("bf16", 2, "tri"), ("bf16", 2, "full"), ("bf16", 3, "tri"), ("fp16", 1, "tri"),
+                ("fp16", 2, "tri"), ("fp16", 3, "tri"), ("fp8", 3, "full"), ("fp8", 3, "tri"), ("fp8", 2, "full")]
+    sizes = [1, 2, 3, 7, 16, 31, 32, 33, 64, 77, 96, 128, 154, 160, 200, 256, 320]
+    for case in range(120):
+        M, N, K = (int(rng.choice(sizes)) for _ in range(3))
+        lowp, terms, products = cascades[case % len(cascades)]
+        dtype = [torch.float32, torch.float32, torch.float16, torch.bfloat16][case % 4]
+        if dtype != torch.float32:
+            lowp, terms, products = ("fp16" if dtype == torch.float16 else "bf16"), 1, "tri"
+        # fp8 keeps 4 significand bits per term: 'tri' with three terms is exact only on one-term operands
+        hi = 7 if (lowp == "fp8" and products == "tri") or dtype != torch.float32 else 15
+        pad_a, pad_c = int(rng.integers(0, 3)) * 4, int(rng.integers(0, 3)) * 4
+        a = torch.tensor(rng.integers(-hi, hi + 1, (M, K)), dtype=torch.float32)
+        b = torch.tensor(rng.integers(-hi, hi + 1, (K, N)), dtype=torch.float32)
+        bias = torch.tensor(rng.integers(-hi, hi + 1, (N,)), dtype=torch.float32) if case % 3 == 0 else None
+        want = a.long() @ b.long() + (bias.long() if bias is not None else 0)
+        print("fuzz", case, M, N, K, lowp, terms, products, dtype, pad_a, pad_c, bias is not None, flush=True)
+        a_full = torch.full((M, K + pad_a), 99.0, device="cuda:0", dtype=dtype)      # rows padded with junk
+        a_full[:, :K] = a.to("cuda:0").to(dtype)
+        ad, bd = a_full[:, :K], b.to("cuda:0").to(dtype)
+        bias_d = None if bias is None else bias.to("cuda:0").to(dtype)
+        out_full = torch.full((M, N + pad_c), -77.0, device="cuda:0", dtype=dtype)   # result rows padded too
+        kw = dict(lowp=lowp, terms=terms, products=products)
+        if case % 5 == 0 and M % 2 == 0 and pad_a == 0:
+            got = cascaded_lowp_matmul(ad.reshape(2, M // 2, K), bd, bias=bias_d, **kw).reshape(M, N)
+        elif case % 7 == 0:
+            got = cascaded_lowp_matmul_grouped([ad, ad], [bd, bd], biases=None if bias is None else [bias_d] * 2, **kw)[1]
+        else:
+            got = cascaded_lowp_matmul(ad, bd, bias=bias_d, out=out_full[:, :N], **kw)
+            assert got.data_ptr() == out_full.data_ptr()
+            assert bool((out_full[:, N:] == -77.0).all())                            # nothing written past a row's N columns
+        want_t = want.to(torch.float32).to(dtype)      # 16-bit results: the exact integer rounded once
+        assert torch.equal(got.cpu(), want_t), (case, M, N, K, lowp, terms, products, dtype)
