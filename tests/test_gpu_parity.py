@@ -311,6 +311,21 @@ def test_error_vs_fp64_within_bound_of_oracle(gpu_device, case, fmt, terms, prod
     assert got["max_abs"] <= tol * ref["max_abs"], (got["max_abs"], ref["max_abs"])
 
 
+@pytest.mark.parametrize("fmt,terms", [("bf16", 2), ("fp16", 3)])
+def test_ffn_shape_at_full_size_meets_the_bound(gpu_device, fmt, terms):
+    """The GEGLU projection of the 32x32 stage at its full size (2048 x 1280 x 10240, the benchmark's
+    dominant GEMM), both cascades the configuration names; the down projection at full size is in
+    ACC_CASES."""
+    _say("accuracy, full FFN up projection", fmt, terms)
+    a, b = oc.make_operands(2048, 1280, 10240, seed=12, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, fmt, terms, "tri"), exp)
+    got = oc.error_metrics(cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp=fmt, terms=terms).cpu(), exp)
+    _say(f"   rel_fro kernel {got['rel_fro']:.3e} oracle {ref['rel_fro']:.3e}  max_abs kernel {got['max_abs']:.3e} "
+         f"oracle {ref['max_abs']:.3e}")
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+
+
 def test_every_headline_variant_meets_the_bound(gpu_device):
     a, b = oc.make_operands(1024, 640, 640, seed=9, w_std=0.02)
     exp = oc.fp64_matmul(a, b)
