@@ -166,7 +166,7 @@ def test_gated_kernels_integer_exact_value_and_gate_pairing(gpu_device):
     h = (a.long() @ w.long() + bias.long()).double()
     want = h[:, :inner] * torch.nn.functional.gelu(h[:, inner:])
     ran = 0
-    for lowp, terms in (("bf16", 2), ("bf16", 3), ("fp16", 3)):
+    for lowp, terms in (("bf16", 2), ("bf16", 3), ("fp16", 3), ("fp8", 3)):
         pw = PreparedWeight(w.to("cuda:0"), lowp=lowp, terms=terms, glu=True)
         for v in _glu_variants():
             name = _lib.lib().cascmm_variant_name(v).decode()
@@ -181,7 +181,7 @@ def test_gated_kernels_integer_exact_value_and_gate_pairing(gpu_device):
             # fp32 gate: 1 + erf(g / sqrt 2) cancels for g << 0, an absolute error of about |value * g| * 2^-24
             torch.testing.assert_close(y.cpu().double(), want, rtol=1e-5, atol=2e-5, msg=lambda m: f"{name}: {m}")
             ran += 1
-    assert ran >= 5
+    assert ran >= 6
 
 
 @pytest.mark.gpu
