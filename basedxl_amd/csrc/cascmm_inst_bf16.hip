@@ -32,6 +32,7 @@ static const VariantDesc kTable[] = {
     CASCMM_TILE_VARIANT("t128x128x32_w4x1x1_d3_bf16x2_full", 128, 128, 32, 4, 1, 1, 3, F32, BF, 2, true, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x2_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 2, true, false),
     CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_bf16x3_tri", 128, 128, 32, 4, 2, 1, 2, F32, BF, 3, false, true),
+    CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d3_bf16x3_tri", 64, 64, 32, 2, 2, 1, 3, F32, BF, 3, false, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x3_tri_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 3, false, false),
     CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_bf16x3_full", 128, 128, 32, 4, 2, 1, 2, F32, BF, 3, true, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_bf16x3_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, BF, 3, true, false),
