@@ -51,7 +51,8 @@
 
 namespace cascmm {
 
-template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2, int NP_ = 4, bool QUADS_ = true>
+template <int BM_, int BN_, int BK_, int WM_, int WN_, int WK_ = 1, int DEPTH_ = 2, int NP_ = 4, bool QUADS_ = true,
+          bool PAIRS_ = false>
 struct Tile {
   static constexpr int BM = BM_, BN = BN_, BK = BK_, WM = WM_, WN = WN_, WK = WK_, DEPTH = DEPTH_, NP = NP_;
   static constexpr int NCW = WM * WN * WK;   // consumer waves
@@ -66,6 +67,10 @@ struct Tile {
   // (QUADS_ = false: every column one at a time, which gives units small enough to spread
   // evenly over eight producer waves.)
   static constexpr int BNQ = QUADS_ ? (BN / 128) * 128 : 0, BNS = BN - BNQ;
+  // PAIRS_: the permuted columns are staged two at a time (8-byte loads, 8 k x 2 n per unit)
+  // instead of four: twice as many, half as large units, so that every producer thread gets
+  // the same mix of units and needs a smaller register ring
+  static constexpr int QN = PAIRS_ ? 2 : 4;
   // a consumer wave must own whole runs of permuted blocks: all four of a group, or two
   static_assert(BNQ == 0 || WTN % 128 == 0 || WTN == 64 || (WN == 1), "wave tile vs permuted B columns");
   static_assert(BNQ == 0 || WN == 1 || BNS == 0, "mixed B column layouts need one consumer wave column");
@@ -118,6 +123,8 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 __device__ float llvm_raw_buffer_load_f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.f32");
 __device__ f32x4 llvm_raw_buffer_load_v4f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
+typedef float f32x2_ld __attribute__((ext_vector_type(2)));
+__device__ f32x2_ld llvm_raw_buffer_load_v2f32(i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v2f32");
 __device__ void llvm_raw_buffer_store_f32(float v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.f32");
 __device__ void llvm_raw_buffer_store_v4f32(f32x4 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v4f32");
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -150,7 +157,7 @@ struct TileGemm {
   static constexpr int ES = sizeof(IoT);
   static constexpr int NCLS = AC::kCount;
   static constexpr int A_UNITS = TL::KG * TL::BM;
-  static constexpr int Q_UNITS = TL::KG * (TL::BNQ / 4);   // 8(k) x 4(n) blocks of B
+  static constexpr int Q_UNITS = TL::KG * (TL::BNQ / TL::QN);   // 8(k) x 4(n) (or 8 x 2) blocks of B
   static constexpr int B_UNITS = TL::KG * TL::BNS;         // 8(k) x 1(n) columns of B
   static constexpr int D = TL::DEPTH;
   static_assert(!BPRE || TL::BNQ == 0, "prepared B is staged column by column");
@@ -185,7 +192,8 @@ struct TileGemm {
     const float t = ax > 4.0f ? 0.f : __builtin_amdgcn_exp2f(p);   // beyond: erfc < 1.6e-8, taken as 0
     return v * (0.5f * g * (g < 0.f ? t : 2.f - t));
   }
-  static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // quads per row of the permuted part
+  static constexpr int QN = TL::QN;
+  static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / QN : 1;   // blocks per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
 
   // ---- producer waves: global -> split -> LDS, one stage per barrier interval -----------------
@@ -232,9 +240,22 @@ struct TileGemm {
     static constexpr int B_IT = HAS_S ? (B_UNITS + NTR - 1) / NTR : 0;
     static_assert((A_IT * 2 + Q_IT * 8 + B_IT * (BPRE ? PL : 8)) * D <= 60, "too many loads in flight for the vmcnt counter");
 
+    // one k row of a block of QN consecutive columns: a 16-byte or an 8-byte load
+    static __device__ __forceinline__ void load_block(i32x4 rsrc, int voff, int soff, float (&dst)[QN]) {
+      if constexpr (QN == 4) {
+        const f32x4 v = llvm_raw_buffer_load_v4f32(rsrc, voff, soff, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[i] = v[i];
+      } else {
+        const f32x2_ld v = llvm_raw_buffer_load_v2f32(rsrc, voff, soff, 0);
+        dst[0] = v[0];
+        dst[1] = v[1];
+      }
+    }
+
     struct Regs {
       float a[A_IT > 0 ? A_IT : 1][8];
-      float q[Q_IT > 0 ? Q_IT : 1][8][4];
+      float q[Q_IT > 0 ? Q_IT : 1][8][QN];
       float b[B_IT > 0 ? B_IT : 1][BREGS];
     };
 
@@ -262,8 +283,11 @@ struct TileGemm {
 #pragma unroll
       for (int it = 0; it < Q_IT; ++it) {
         const int u = rtid + it * NTR;
-        const int quad = u % QW, kg = u / QW;
-        c.lds_q[it] = u < Q_UNITS ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) : -1;
+        // column 4 * quad + QN * sub is the block's first; consecutive threads take consecutive
+        // quads (consecutive LDS slots), the second halves of the quads follow the first halves
+        const int blk = u % QW, kg = u / QW;
+        const int quad = blk % (TL::BNQ / 4), sub = blk / (TL::BNQ / 4);
+        c.lds_q[it] = u < Q_UNITS ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) + QN * sub * 32 : -1;
       }
 #pragma unroll
       for (int it = 0; it < B_IT; ++it) {
@@ -312,10 +336,11 @@ struct TileGemm {
       for (int it = 0; it < Q_IT; ++it) {
         int u = rtid + it * NTR;
         u = u < Q_UNITS ? u : Q_UNITS - 1;
-        const int quad = u % QW, kg = u / QW;
+        const int blk = u % QW, kg = u / QW;
+        const int quad = blk % (TL::BNQ / 4), sub = blk / (TL::BNQ / 4);
         const int last_quad = last_col >> 2;  // fast path: N % 4 == 0, a quad is wholly in or out
         const int qc = quad < last_quad ? quad : last_quad;
-        c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc) * ES);
+        c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc + QN * sub) * ES);
       }
 #pragma unroll
       for (int it = 0; it < B_IT; ++it) {
@@ -351,9 +376,7 @@ struct TileGemm {
         const int soff_b = (k0 + e) * c.ldb_bytes;
 #pragma unroll
         for (int it = 0; it < Q_IT; ++it) {
-          const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], soff_b, 0);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
+          load_block(c.rb, c.voff_q[it], soff_b, r.q[it][e]);
         }
 #pragma unroll
         for (int it = 0; it < B_IT; ++it) r.b[it][e] = llvm_raw_buffer_load_f32(c.rb, c.voff_b[it], soff_b, 0);
@@ -395,11 +418,12 @@ struct TileGemm {
       for (int it = 0; it < Q_IT; ++it) {
         int u = rtid + it * NTR;
         u = u < Q_UNITS ? u : Q_UNITS - 1;
-        const int quad = u % QW, kg = u / QW;
+        const int blk = u % QW, kg = u / QW;
         const int k = k0 + kg * 8;
+        const int quad = blk % (TL::BNQ / 4), sub = blk / (TL::BNQ / 4);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          int col = n0 + 4 * quad + i;
+        for (int i = 0; i < QN; ++i) {
+          int col = n0 + 4 * quad + QN * sub + i;
           col = col < p.N ? col : p.N - 1;
           const IoT* src = B + (int64_t)k * p.ldb + col;
 #pragma unroll
@@ -457,7 +481,7 @@ struct TileGemm {
       for (int it = 0; it < Q_IT; ++it) {
         if (Q_UNITS % NTR == 0 || c.lds_q[it] >= 0) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
+          for (int i = 0; i < QN; ++i) {
             float x[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = r.q[it][e][i];
@@ -470,9 +494,7 @@ struct TileGemm {
         if (ISSUE) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            const f32x4 v = llvm_raw_buffer_load_v4f32(c.rb, c.voff_q[it], (k_next + e) * c.ldb_bytes, 0);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) r.q[it][e][i] = v[i];
+            load_block(c.rb, c.voff_q[it], (k_next + e) * c.ldb_bytes, r.q[it][e]);
           }
         }
       }

@@ -78,6 +78,12 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
    LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, Lowp<FMT>::planes(TERMS)>::kBytes, FAST, true,   \
    &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP>, IODT, FMT, TERMS, FULL, FAST>}
 
+// permuted B columns staged in 8 x 2 blocks (Tile's PAIRS flag)
+#define CASCMM_TILE_VARIANT_PAIRS(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)             \
+  {NAME, KIND_TILE, IODT, FMT, TERMS, FULL, BM, BN, BK, Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, true, true>::NT,    \
+   LdsLayout<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, true, true>, Lowp<FMT>::planes(TERMS)>::kBytes, FAST, true,    \
+   &launch_tile<Tile<BM, BN, BK, WM, WN, WK, DEPTH, NP, true, true>, IODT, FMT, TERMS, FULL, FAST>}
+
 // K splits of the skinny path: enough workgroups to occupy every CU, each with at least one
 // K step of `bk`; the same function sizes the workspace
 inline int skinny_splits(int64_t M, int64_t N, int64_t K, int bm, int bn, int bk) {
