@@ -15,7 +15,7 @@ class BasedXLLowPLinear(nn.Module):
     into its store (the reference adds it in a second kernel, lowp_linear.py:17-19)."""
 
     def __init__(self, submodule: nn.Linear, *, lowp: Optional[str] = None, terms: Optional[int] = None,
-                 products: str = "tri", prepared: bool = False):
+                 products: str = "tri", prepared: Optional[bool] = None):
         super().__init__()
         self.in_features = submodule.in_features
         self.out_features = submodule.out_features
@@ -25,7 +25,12 @@ class BasedXLLowPLinear(nn.Module):
         self.lowp, self.terms, self.products = d_lowp if lowp is None else lowp, d_terms if terms is None else terms, products
         self._weight_exp = None   # fp8: tensor-scale exponent of the weight, found on first use
         # prepared=True: the weight is also kept split (once, on first use on the GPU); inputs
-        # the prepared kernels do not take (not fp32, K not a multiple of 64) use the raw weight
+        # the prepared kernels do not take (K not a multiple of 64, ...) use the raw weight.
+        # Default: on for fp16 / bf16 weights multiplied as one term of their own format (there
+        # "prepared" is only a re-layout of the weight, which the raw path would redo in every
+        # call), off for fp32 weights (both operands are then split inside every GEMM)
+        if prepared is None:
+            prepared = self.weight.dtype != torch.float32 and (self.lowp, self.terms) == (d_lowp, d_terms)
         self.prepared = prepared
         self._prepared_weight = None
 

@@ -268,3 +268,24 @@ def test_geglu_module_sixteen_bit_tensors(gpu_device, dtype, fmt, ulp):
                                    proj.bias.detach().cpu().float(), fmt, 1)
     err = (y.cpu().float() - want).abs()
     assert bool((err <= ulp * want.abs() + 1e-6).all()), float((err / want.abs().clamp_min(1e-6)).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,fmt,ulp", [(torch.float16, "fp16", 2.0 ** -10), (torch.bfloat16, "bf16", 2.0 ** -7)])
+def test_linear_wrapper_keeps_sixteen_bit_weights_prepared_by_default(gpu_device, dtype, fmt, ulp):
+    """fp16 / bf16 modules (the dtype the reference runs in): the wrapper re-lays its weight once
+    instead of in every call; fp32 modules split both operands in every call unless asked."""
+    torch.manual_seed(45)
+    lin = torch.nn.Linear(640, 320).to("cuda:0").to(dtype)
+    mod = BasedXLLowPLinear(lin)
+    assert mod.prepared and not BasedXLLowPLinear(torch.nn.Linear(64, 64)).prepared
+    assert not BasedXLLowPLinear(lin, lowp="bf16", terms=2).prepared      # other cascades: raw weight
+    x = torch.randn(2, 100, 640, device="cuda:0").to(dtype)
+    y = mod(x)
+    assert mod._prepared_weight is not None and y.dtype == dtype and y.shape == (2, 100, 320)
+    want = oc.cascade_matmul_ref(x.cpu().float().reshape(-1, 640), lin.weight.detach().cpu().float().T.contiguous(), fmt, 1) \
+        + lin.bias.detach().cpu().float()
+    err = (y.cpu().float().reshape(-1, 320) - want).abs()
+    assert bool((err <= ulp * want.abs() + 1e-3).all())
+    assert torch.equal(BasedXLLowPLinear(lin, prepared=False)(x), y) or \
+        bool(((BasedXLLowPLinear(lin, prepared=False)(x).float() - y.float()).abs() <= ulp * y.float().abs() + 1e-3).all())
