@@ -50,7 +50,9 @@ def sdxl_linear_shapes(batch: int = 2, latent: int = 128, half_latent: bool = Fa
             LinearShape(f"attn1.to_q/k/v d={d}", blocks, tok, d, d, group=3),
             LinearShape(f"attn1.to_out d={d}", blocks, tok, d, d),
             LinearShape(f"attn2.to_q d={d}", blocks, tok, d, d),
-            LinearShape(f"attn2.to_k/v d={d}", blocks, txt, 2048, d, group=2),
+            # key and value of the text tokens as ONE [2048, 2 d] projection, the way the reference's
+            # attention wrapper fuses them (basedxl/modules/attn.py:23-39) and BasedXLFusedKV does here
+            LinearShape(f"attn2.to_kv d={d}", blocks, txt, 2048, 2 * d),
             LinearShape(f"attn2.to_out d={d}", blocks, tok, d, d),
             LinearShape(f"ff.geglu_proj d={d}", blocks, tok, d, 8 * d, gated=True),
             LinearShape(f"ff.out d={d}", blocks, tok, 4 * d, d),
