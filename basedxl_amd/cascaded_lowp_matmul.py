@@ -108,6 +108,20 @@ class PreparedWeight:
                            _DTYPES[w.dtype], self.fmt, self.terms, self.exp.data_ptr() if self.exp is not None else None,
                            self.slots.data_ptr(), self.slots.numel(), stream), "cascmm_prepare_weight")
 
+    @classmethod
+    def from_slots(cls, slots: torch.Tensor, K: int, N: int, dtype: torch.dtype, lowp: str, terms: int, glu: bool = False,
+                   exp: Optional[torch.Tensor] = None) -> "PreparedWeight":
+        """The object around operand slots that already exist (``prepared.slots`` of an earlier
+        preparation with the same K, N, dtype and cascade); nothing is computed."""
+        self = cls.__new__(cls)
+        self.K, self.N, self.shape = int(K), int(N), (int(K), int(N))
+        self.lowp, self.terms, self.fmt = lowp, int(terms), _lib.FMT_BY_NAME[lowp]
+        self.dtype, self.device = dtype, slots.device
+        self.glu = bool(glu)
+        self.out_features = self.N // 2 if self.glu else self.N
+        self.exp, self.slots = exp, slots
+        return self
+
     def usable_with(self, a2: torch.Tensor) -> bool:
         """Whether the prepared kernels take this left operand: fp32 (or fp16 / bf16 tensors with a
         weight of the same dtype kept as one term of that format), K a multiple of 64, rows 16-byte

@@ -43,7 +43,22 @@ class BasedXLLowPGEGLU(nn.Module):
         # 16-bit tensors have prepared kernels only for one term of their own format
         return x.dtype == torch.float32 or (self.lowp, self.terms) == default_cascade(x.dtype)
 
+    def prepare(self) -> None:
+        """Prepare the gated weight now (needs the weight on the GPU); otherwise on the first eager call."""
+        if self.weight.is_cuda and self.in_features % 64 == 0 and self.inner % 32 == 0 and (
+                self._prepared is None or self._prepared.device != self.weight.device):
+            self._prepared = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms, glu=True)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if torch.compiler.is_compiling() and self._prepared is not None and x.dtype == self.weight.dtype:
+            from ..compiled import cascade_linear
+            return cascade_linear(x, self.weight, self._prepared.slots, self.bias, self.lowp, self.terms, self.products,
+                                  True, self._prepared.exp)
+        if torch.compiler.is_compiling():
+            from ..compiled import cascade_linear
+            h = cascade_linear(x, self.weight, None, self.bias, self.lowp, self.terms, self.products, False, None)
+            value, gate = h.chunk(2, dim=-1)
+            return value * F.gelu(gate)
         if self._fusable(x):
             if self._prepared is None or self._prepared.device != self.weight.device:
                 self._prepared = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms, glu=True)

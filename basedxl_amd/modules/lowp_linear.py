@@ -34,7 +34,22 @@ class BasedXLLowPLinear(nn.Module):
         self.prepared = prepared
         self._prepared_weight = None
 
+    def prepare(self) -> None:
+        """Split / re-lay the weight now (needs the weight on the GPU); otherwise it happens on the
+        first eager call.  A model that is compiled before it ever ran eagerly should call this."""
+        if self.prepared and self.weight.is_cuda and (self._prepared_weight is None
+                                                      or self._prepared_weight.device != self.weight.device):
+            self._prepared_weight = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms)
+        if self.lowp == "fp8" and self.weight.is_cuda and (self._weight_exp is None or self._weight_exp.device != self.weight.device):
+            self._weight_exp = tensor_scale_exp(self.weight)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if torch.compiler.is_compiling():
+            # traced by torch.compile: one opaque op (whatever was prepared before tracing is used)
+            from ..compiled import cascade_linear
+            pw = self._prepared_weight
+            return cascade_linear(x, self.weight, None if pw is None else pw.slots, self.bias, self.lowp, self.terms,
+                                  self.products, False, self._weight_exp if pw is None else pw.exp)
         if self.prepared and x.is_cuda:
             if self._prepared_weight is None or self._prepared_weight.device != self.weight.device:
                 self._prepared_weight = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms)

@@ -52,6 +52,18 @@ class BasedXLLowPConv1x1(nn.Module):
         if x.dim() != 4 or x.shape[1] != self.in_channels:
             raise ValueError(f"expected [B, {self.in_channels}, H, W], got {tuple(x.shape)}")
         B, _, H, W = x.shape
+        if torch.compiler.is_compiling():
+            # traced by torch.compile: the GEMMs as opaque ops (one per image for NCHW input)
+            from ..compiled import cascade_linear
+            if x.is_contiguous(memory_format=torch.channels_last) and not x.is_contiguous():
+                y = cascade_linear(x.permute(0, 2, 3, 1), self.weight_t, None, self.bias, self.lowp, self.terms,
+                                   self.products, False, None)
+                return y.permute(0, 3, 1, 2)
+            xc = x.contiguous()
+            ys = [cascade_linear(self.weight, xc[b].reshape(self.in_channels, H * W), None, None, self.lowp, self.terms,
+                                 self.products, False, None) for b in range(B)]
+            out = torch.stack(ys).reshape(B, self.out_channels, H, W)
+            return out if self.bias is None else out + self.bias.view(1, -1, 1, 1)
         rows = x.permute(0, 2, 3, 1)
         if rows.is_contiguous() and not x.is_contiguous():
             if self.lowp == "fp8" and (self._weight_exp is None or self._weight_exp.device != x.device):

@@ -289,3 +289,73 @@ def test_linear_wrapper_keeps_sixteen_bit_weights_prepared_by_default(gpu_device
     assert bool((err <= ulp * want.abs() + 1e-3).all())
     assert torch.equal(BasedXLLowPLinear(lin, prepared=False)(x), y) or \
         bool(((BasedXLLowPLinear(lin, prepared=False)(x).float() - y.float()).abs() <= ulp * y.float().abs() + 1e-3).all())
+
+
+# ---------------------------------------------------------------------------------- torch.compile
+
+
+def test_custom_op_shapes_without_a_gpu():
+    """The op's shape-only implementation, which is all a tracer runs (fake tensors: no data, no GPU)."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from basedxl_amd import compiled  # noqa: F401  (registers the op)
+
+    with FakeTensorMode():
+        x = torch.empty(2, 77, 640, device="cuda")
+        w = torch.empty(640, 1280, device="cuda")
+        assert torch.ops.basedxl_amd.cascade_linear(x, w, None, None, "bf16", 2, "tri", False, None).shape == (2, 77, 1280)
+        assert torch.ops.basedxl_amd.cascade_linear(x, w, None, None, "bf16", 2, "tri", True, None).shape == (2, 77, 640)
+
+
+class _FeedForward(torch.nn.Module):
+    """The shape of a transformer block's feed-forward part: GEGLU projection, then the output Linear."""
+
+    def __init__(self, d, dtype):
+        super().__init__()
+        self.proj = torch.nn.Linear(d, 8 * d, dtype=dtype)
+        self.out = torch.nn.Linear(4 * d, d, dtype=dtype)
+
+    def forward(self, x):
+        return self.out(self.proj(x))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_patched_model_traces_under_torch_compile(gpu_device, dtype):
+    """The reference compiles its UNet with fullgraph=True (unet.py:76-78): a model whose Linear
+    layers were swapped must trace without a graph break and give the eager result.  (Backend
+    "aot_eager": traces and functionalises like the default backend but generates no code.)"""
+    from basedxl_amd import BasedXLLowPGEGLU, BasedXLLowPLinear
+
+    torch.manual_seed(46)
+    m = _FeedForward(128, dtype).to("cuda:0")
+    m.proj = BasedXLLowPGEGLU(m.proj)
+    m.out = BasedXLLowPLinear(m.out, prepared=True)
+    x = torch.randn(2, 96, 128, device="cuda:0", dtype=dtype)
+    with torch.no_grad():
+        eager = m(x)                       # first eager call prepares the weights
+        assert m.proj._prepared is not None and m.out._prepared_weight is not None
+        compiled = torch.compile(m, backend="aot_eager", fullgraph=True)
+        traced = compiled(x)
+        assert torch.equal(traced, eager)
+        assert torch.equal(compiled(x * 2), m(x * 2))
+        # never run eagerly: prepare() does what the first eager call would have done
+        m2 = _FeedForward(128, dtype).to("cuda:0")
+        m2.proj, m2.out = BasedXLLowPGEGLU(m2.proj), BasedXLLowPLinear(m2.out, prepared=True)
+        m2.proj.prepare()
+        m2.out.prepare()
+        assert torch.equal(torch.compile(m2, backend="aot_eager", fullgraph=True)(x), m2(x))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_pointwise_conv_traces_under_torch_compile(gpu_device, channels_last):
+    torch.manual_seed(47)
+    mod = BasedXLLowPConv1x1(torch.nn.Conv2d(64, 128, 1).to("cuda:0")).to("cuda:0")
+    x = torch.randn(2, 64, 16, 8, device="cuda:0")
+    if channels_last:
+        x = x.contiguous(memory_format=torch.channels_last)
+    with torch.no_grad():
+        eager = mod(x)
+        traced = torch.compile(mod, backend="aot_eager", fullgraph=True)(x)
+    torch.testing.assert_close(traced, eager, rtol=0, atol=2e-5)   # per-image launches may pick another tile than the grouped one
