@@ -679,7 +679,7 @@ def test_unet_shape_harness_and_error_script_run(gpu_device, capsys):
     from basedxl_amd import measure_error, unet_shapes
 
     shapes = [s for s in unet_shapes.sdxl_linear_shapes(batch=1, latent=32, half_latent=True)
-              if s.name.startswith(("attn1.to_q/k/v d=640", "attn2.to_k/v d=640", "time_embedding.linear_1"))]
+              if s.name.startswith(("attn1.to_q/k/v d=640", "attn2.to_kv d=640", "time_embedding.linear_1"))]
     for prepared in (False, True):
         rows = unet_shapes.time_shapes(shapes, "bf16", 2, prepared=prepared, iters=2)
         assert len(rows) == 3 and all(r["launch_us"] > 0 for r in rows)
