@@ -273,7 +273,19 @@ def test_sixteen_bit_integers_full_product_set_is_exact(gpu_device):
     full = cascaded_lowp_matmul(_gpu(at), _gpu(bt), products="full").cpu().numpy().astype(np.int64)
     tri = cascaded_lowp_matmul(_gpu(at), _gpu(bt), products="tri").cpu()
     assert np.array_equal(full[keep], want[keep])
-    assert torch.equal(tri, oc.cascade_matmul_ref(at, bt, "bf16", 2, "tri"))
+    # the tri set, in exact integer arithmetic: hi.hi + hi.lo + lo.hi (the splits of integers are integers)
+    (ah, al), (bh, bl) = (tuple(t.numpy().astype(np.int64) for t in oc.split_terms(x, "bf16", 2)[0]) for x in (at, bt))
+    assert np.array_equal(ah + al, a) and np.array_equal(bh + bl, b)
+    tri_exact = ah @ bh + ah @ bl + al @ bh
+    # wherever no partial sum, in any order, can leave the 24-bit range the kernel must return exactly that
+    # integer; elsewhere the summation order decides single roundings of the fp32 accumulator
+    safe = (np.abs(ah) + np.abs(al)) @ (np.abs(bh) + np.abs(bl)) < 2 ** 24
+    assert safe.sum() > safe.size // 4
+    got = tri.numpy().astype(np.int64)
+    assert np.array_equal(got[safe], tri_exact[safe])
+    assert np.all(np.abs(got - tri_exact) <= 8)           # three roundings below 2^26 (ulp 4, half an ulp each), with margin
+    ref = oc.cascade_matmul_ref(at, bt, "bf16", 2, "tri").numpy().astype(np.int64)
+    assert np.array_equal(ref[safe], tri_exact[safe])
 
 
 # ---------------------------------------------------------------------------------------
