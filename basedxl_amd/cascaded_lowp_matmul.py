@@ -73,7 +73,10 @@ class PreparedWeight:
     """A constant right operand ``w`` ([K, N]: the ``[in, out]`` weight of
     basedxl/modules/lowp_linear.py:12) split once on the GPU into the terms of a cascade and
     kept as MFMA operand slots; ``cascaded_lowp_matmul(a, prepared)`` then splits only ``a``.
-    The arithmetic is the same as with the raw weight (same split, same products).
+    The arithmetic is the same as with the raw weight (same split, same products).  Kernels for
+    prepared weights exist for bf16 x 2, bf16 x 3, fp16 x 3 and fp8 x 3 with the 'tri' product set and
+    for fp16 / bf16 tensors as one term of their own format, K a multiple of 64 and N of 4; the
+    product with any other combination fails with CascmmError (use the raw weight there).
 
     ``glu=True``: ``w`` is the ``[in, 2 * inner]`` weight of a gated projection (diffusers' GEGLU:
     ``h = x @ w + b; y = h[:, :inner] * gelu(h[:, inner:])``); its columns are stored so that a
@@ -155,7 +158,13 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
             raise ValueError("grouped problems must share one shape, cascade and activation dtype")
         if a.dtype not in _DTYPES:
             raise TypeError(f"unsupported dtype {a.dtype}")
-        a2s.append(_rows(a.reshape(-1, w.K)))
+        a2 = _rows(a.reshape(-1, w.K))
+        # the prepared kernels load 16 bytes of a row at a time: rows that do not start on such a
+        # boundary are copied, as basedxl/triton/cascaded_lowp_matmul.py:158 copies every `a`
+        per16 = 16 // a2.element_size()
+        if a2.data_ptr() % 16 != 0 or (a2.shape[0] > 1 and a2.stride(0) % per16 != 0):
+            a2 = a2.contiguous()
+        a2s.append(a2)
     M, K, N = a2s[0].shape[0], w0.K, w0.N
     NO = w0.out_features                       # columns of the result (N / 2 for a gated weight)
     lda = a2s[0].stride(0) if M > 1 else max(K, 1)

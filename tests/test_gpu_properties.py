@@ -104,6 +104,23 @@ def test_prepared_weight_has_the_same_properties(gpu_device, M, K, N):
     assert torch.equal(cascaded_lowp_matmul(a * 4.0, pw), c * 4.0)
 
 
+def test_prepared_weight_takes_rows_that_are_not_16_byte_aligned(gpu_device):
+    """A view whose rows start at odd element offsets (row stride K + 3, first element shifted by
+    one) gives the same bits as its contiguous copy: the wrapper copies what the prepared kernels
+    cannot load, as the reference copies every ``a`` (basedxl/triton/cascaded_lowp_matmul.py:158)."""
+    g = torch.Generator(device="cuda:0").manual_seed(11)
+    K, N, M = 512, 320, 130
+    store = torch.randn(M, K + 3, device="cuda:0", generator=g)
+    b = torch.randn(K, N, device="cuda:0", generator=g) * 0.02
+    pw = PreparedWeight(b)
+    a = store[:, 1:K + 1]
+    assert a.data_ptr() % 16 != 0 and a.stride(0) % 4 != 0
+    want = cascaded_lowp_matmul(a.contiguous(), pw)
+    assert torch.equal(cascaded_lowp_matmul(a, pw), want)
+    # the raw weight gives the same sum of the same products, in the summation order of its own kernel
+    torch.testing.assert_close(want, cascaded_lowp_matmul(a, b), rtol=1e-5, atol=1e-5)
+
+
 def test_random_shapes_strides_and_cascades_integer_exact(gpu_device):
     """Seeded sweep over what a caller can vary at once -- M, N, K (odd sizes included), row
     strides of A and of the result, leading batch dims, bias, dtype, cascade and product set -- with
