@@ -288,6 +288,32 @@ def test_sixteen_bit_integers_full_product_set_is_exact(gpu_device):
     assert np.array_equal(ref[safe], tri_exact[safe])
 
 
+@pytest.mark.parametrize("lowp,terms", [("bf16", 2), ("fp16", 3), ("bf16", 1)])
+def test_non_finite_operands_poison_their_row_or_column_only(gpu_device, lowp, terms):
+    """A NaN or an infinity in A spoils exactly its row of the result, one in B exactly its column,
+    as in the oracle (the residual of an infinite term is inf - inf); every other element keeps
+    the bits it has without them."""
+    _say("non-finite", lowp, terms)
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn(96, 128, generator=g)
+    b = torch.randn(128, 80, generator=g) * 0.02
+    clean = cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp=lowp, terms=terms).cpu()
+    a2, b2 = a.clone(), b.clone()
+    a2[5, 17] = float("nan")
+    a2[40, 3] = float("inf")
+    b2[100, 9] = -float("inf")
+    got = cascaded_lowp_matmul(_gpu(a2), _gpu(b2), lowp=lowp, terms=terms).cpu()
+    want = oc.cascade_matmul_ref(a2, b2, lowp, terms, "tri")
+    bad = torch.zeros(96, 80, dtype=torch.bool)
+    bad[5, :] = bad[40, :] = True
+    bad[:, 9] = True
+    # one term has no residual: an infinite operand gives +-inf (or NaN against a zero), never a finite value
+    assert not torch.isfinite(got[bad]).any() and not torch.isfinite(want[bad]).any()
+    if terms > 1:
+        assert torch.isnan(got[bad]).all() and torch.isnan(want[bad]).all()
+    assert torch.equal(got[~bad], clean[~bad])
+
+
 # ---------------------------------------------------------------------------------------
 # accuracy bound against the oracle on the baseline configurations
 # ---------------------------------------------------------------------------------------
