@@ -165,3 +165,58 @@ def test_random_shapes_strides_and_cascades_integer_exact(gpu_device):
             assert bool((out_full[:, N:] == -77.0).all())                            # nothing written past a row's N columns
         want_t = want.to(torch.float32).to(dtype)      # 16-bit results: the exact integer rounded once
         assert torch.equal(got.cpu(), want_t), (case, M, N, K, lowp, terms, products, dtype)
+
+
+def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
+    """The reference compiles its UNet (unet.py:76-78), and compiled models are commonly replayed
+    from device graphs: every launch path of the library -- LDS-tiled kernel, K split with its
+    reduction pass, skinny split-K kernel, grouped launch, 16-bit tensors (weights re-laid into the
+    workspace), prepared and gated weights, fp8 with the scale found on the device -- is captured
+    once and replayed with fresh operand values; each replay must return the bits of the eager call
+    on the same values (nothing host-side, no memset, no allocation inside the captured region
+    after the warm-up)."""
+    from basedxl_amd import cascaded_lowp_matmul_grouped
+
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(5)
+    rn = lambda *s, dtype=torch.float32: torch.randn(*s, device=dev, generator=g).to(dtype)
+    w = {
+        "tile": rn(640, 640) * 0.02, "ksplit": rn(5120, 1280) * 0.02, "skinny": rn(2048, 640) * 0.02,
+        "h": (rn(640, 640) * 0.02).half(), "glu": rn(640, 1280) * 0.02, "fp8": rn(320, 640) * 0.02,
+    }
+    x = {"tile": rn(2048, 640), "ksplit": rn(1024, 5120), "skinny": rn(154, 2048), "h": rn(1024, 640).half(),
+         "glu": rn(512, 640), "fp8": rn(512, 320)}
+    pw, pg = PreparedWeight(w["tile"]), PreparedWeight(w["glu"], glu=True)
+
+    def run():
+        return [
+            cascaded_lowp_matmul(x["tile"], w["tile"]),
+            cascaded_lowp_matmul(x["ksplit"], w["ksplit"]),
+            cascaded_lowp_matmul(x["skinny"], w["skinny"]),
+            cascaded_lowp_matmul_grouped([x["tile"]] * 3, [w["tile"]] * 3)[2],
+            cascaded_lowp_matmul_grouped([x["h"]] * 2, [w["h"]] * 2)[1],
+            cascaded_lowp_matmul(x["tile"], pw),
+            cascaded_lowp_matmul(x["glu"], pg),
+            cascaded_lowp_matmul(x["fp8"], w["fp8"], lowp="fp8", terms=3),
+        ]
+
+    run()                                            # warm-up: workspaces exist before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()                                        # and on a side stream, as torch's capture recipe asks
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run()
+    for rep in range(3):
+        for k in x:                                  # new values in the captured buffers
+            x[k].copy_(rn(*x[k].shape, dtype=x[k].dtype) * (1.0 + rep))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = run()                                 # eager work between the replays
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), (rep, i)
