@@ -209,8 +209,7 @@ struct GemmParams {
   int tiles_m, tiles_n;
   int k_splits;          // split-K path only
   int k_per_split;       // split-K path only (multiple of the kernel's BK)
-  float* partials;       // split-K workspace: [k_splits][M][N] fp32 after the counters
-  unsigned* counters;    // split-K arrival counters, one per output tile
+  float* partials;       // split-K workspace: [k_splits][M][N] fp32
   const int32_t* tensor_exps;
 };
 

@@ -195,6 +195,7 @@ struct TileGemm {
   static constexpr int QN = TL::QN;
   static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / QN : 1;   // blocks per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part
+  static constexpr int QUADS = TL::BNQ > 0 ? TL::BNQ / 4 : 1;   // groups of four permuted columns
 
   // ---- producer waves: global -> split -> LDS, one stage per barrier interval -----------------
   // Barrier protocol over the global step sequence g of a workgroup (every wave executes the
@@ -286,7 +287,7 @@ struct TileGemm {
         // column 4 * quad + QN * sub is the block's first; consecutive threads take consecutive
         // quads (consecutive LDS slots), the second halves of the quads follow the first halves
         const int blk = u % QW, kg = u / QW;
-        const int quad = blk % (TL::BNQ / 4), sub = blk / (TL::BNQ / 4);
+        const int quad = blk % QUADS, sub = blk / QUADS;
         c.lds_q[it] = u < Q_UNITS ? kg * LL::kBPlane + (quad >> 5) * 128 + (quad & 31) + QN * sub * 32 : -1;
       }
 #pragma unroll
@@ -337,7 +338,7 @@ struct TileGemm {
         int u = rtid + it * NTR;
         u = u < Q_UNITS ? u : Q_UNITS - 1;
         const int blk = u % QW, kg = u / QW;
-        const int quad = blk % (TL::BNQ / 4), sub = blk / (TL::BNQ / 4);
+        const int quad = blk % QUADS, sub = blk / QUADS;
         const int last_quad = last_col >> 2;  // fast path: N % 4 == 0, a quad is wholly in or out
         const int qc = quad < last_quad ? quad : last_quad;
         c.voff_q[it] = (int)((kg * 8 * p.ldb + 4 * qc + QN * sub) * ES);
@@ -420,7 +421,7 @@ struct TileGemm {
         u = u < Q_UNITS ? u : Q_UNITS - 1;
         const int blk = u % QW, kg = u / QW;
         const int k = k0 + kg * 8;
-        const int quad = blk % (TL::BNQ / 4), sub = blk / (TL::BNQ / 4);
+        const int quad = blk % QUADS, sub = blk / QUADS;
 #pragma unroll
         for (int i = 0; i < QN; ++i) {
           int col = n0 + 4 * quad + QN * sub + i;
