@@ -190,9 +190,14 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
     exps = None
     if w0.fmt == _lib.FMT_FP8:
         exps = torch.empty(2 * n, dtype=torch.int32, device=dev)
+        first = {}                                   # one pass per distinct left operand (q / k / v share theirs)
         for i in range(n):
-            _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _DTYPES[adt], exps.data_ptr() + 8 * i,
-                                                    stream), "cascmm_tensor_exp(A)")
+            j = first.setdefault(a2s[i].data_ptr(), i)
+            if j == i:
+                _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _DTYPES[adt], exps.data_ptr() + 8 * i,
+                                                        stream), "cascmm_tensor_exp(A)")
+            else:
+                exps[2 * i:2 * i + 1].copy_(exps[2 * j:2 * j + 1])
             exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
     common = (n, pa, pb, pc, pbias, M, N, K, lda, max(NO, 1), _DTYPES[adt], w0.fmt, w0.terms,
               _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None)
@@ -305,9 +310,14 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
         # tensor scale exponents {e_A, e_B} of every problem, computed on the device
         exps = torch.empty(2 * n, dtype=torch.int32, device=dev)
         dt = _DTYPES[a_list[0].dtype]
+        first = {}                                   # one pass per distinct left operand (q / k / v share theirs)
         for i in range(n):
-            _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, dt, exps.data_ptr() + 8 * i, stream),
-                       "cascmm_tensor_exp(A)")
+            j = first.setdefault(a2s[i].data_ptr(), i)
+            if j == i:
+                _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, dt, exps.data_ptr() + 8 * i, stream),
+                           "cascmm_tensor_exp(A)")
+            else:
+                exps[2 * i:2 * i + 1].copy_(exps[2 * j:2 * j + 1])
             _lib.check(_lib.lib().cascmm_tensor_exp(b_list[i].data_ptr(), K, N, max(N, 1), dt,
                                                     exps.data_ptr() + 8 * i + 4, stream), "cascmm_tensor_exp(B)")
     # 16-bit tensors as one term of their own format: room for every right operand re-laid as operand slots
