@@ -38,6 +38,22 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> Optional[torch
     return ws
 
 
+_exp_scratch: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _activation_exps(a2: torch.Tensor, lda: int, second: Optional[torch.Tensor], out_ptr: int, stream: int) -> None:
+    """{e_A, e_B} at ``out_ptr`` (device int32[2]) in one launch: the fp8 scale exponent of ``a2`` found
+    on the device, next to the kept exponent ``second`` of the other operand (skipped when None)."""
+    dev = a2.device
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream)
+    scratch = _exp_scratch.get(key)
+    if scratch is None:
+        scratch = _exp_scratch[key] = torch.zeros(2, dtype=torch.int32, device=dev)   # the kernel leaves it zeroed
+    _lib.check(_lib.lib().cascmm_tensor_exps(a2.data_ptr(), a2.shape[0], a2.shape[1], lda, _DTYPES[a2.dtype],
+                                             second.data_ptr() if second is not None else None, out_ptr,
+                                             scratch.data_ptr(), stream), "cascmm_tensor_exps")
+
+
 def _check_device_tensor(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(
@@ -194,11 +210,10 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
         for i in range(n):
             j = first.setdefault(a2s[i].data_ptr(), i)
             if j == i:
-                _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, _DTYPES[adt], exps.data_ptr() + 8 * i,
-                                                        stream), "cascmm_tensor_exp(A)")
+                _activation_exps(a2s[i], lda, w_list[i].exp, exps.data_ptr() + 8 * i, stream)
             else:
                 exps[2 * i:2 * i + 1].copy_(exps[2 * j:2 * j + 1])
-            exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
+                exps[2 * i + 1:2 * i + 2].copy_(w_list[i].exp.reshape(1))
     common = (n, pa, pb, pc, pbias, M, N, K, lda, max(NO, 1), _DTYPES[adt], w0.fmt, w0.terms,
               _lib.PROD_BY_NAME[products], exps.data_ptr() if exps is not None else None)
     if w0.glu:
@@ -233,13 +248,9 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
         exps = tensor_exps.contiguous()
     elif fmt == _lib.FMT_FP8:
         exps = torch.empty(2, dtype=torch.int32, device=a2.device)
-        _lib.check(l.cascmm_tensor_exp(a2.data_ptr(), M, K, a2.stride(0), dt, exps.data_ptr(), stream),
-                   "cascmm_tensor_exp(A)")
-        if b_exp is not None:
-            exps[1:2].copy_(b_exp.reshape(1))
-        else:
-            _lib.check(l.cascmm_tensor_exp(b2.data_ptr(), K, N, b2.stride(0), dt, exps.data_ptr() + 4, stream),
-                       "cascmm_tensor_exp(B)")
+        _activation_exps(a2, a2.stride(0) if M > 1 else max(K, 1), b_exp, exps.data_ptr(), stream)
+        if b_exp is None:
+            _activation_exps(b2, b2.stride(0) if K > 1 else max(N, 1), None, exps.data_ptr() + 4, stream)
     st = l.cascmm_gemm_variant(
         a2.data_ptr(), b2.data_ptr(), out2.data_ptr(), bias.data_ptr() if bias is not None else None,
         M, N, K, a2.stride(0) if M > 1 else max(K, 1), b2.stride(0) if K > 1 else max(N, 1),
@@ -253,14 +264,16 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
 
 def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp: Optional[str] = None,
                                  terms: Optional[int] = None,
-                                 products: str = "tri", variant: int = -1):
+                                 products: str = "tri", variant: int = -1, b_exps=None):
     """Several independent cascade GEMMs of one shape in ONE kernel launch.
 
     ``a_list[i]`` ([..., K], the same tensor may appear several times) times ``b_list[i]``
     ([K, N], contiguous) -> ``outs[i]``.  This is what the reference gets for to_k / to_v by
     concatenating the two weights into one Linear (basedxl/modules/attn.py:23-39); here the
     weights stay separate and up to 8 problems share one persistent launch, which removes
-    the launch gap and the cold start of every GEMM after the first.
+    the launch gap and the cold start of every GEMM after the first.  ``b_exps`` (fp8): the tensor
+    scale exponents of the right operands (``tensor_scale_exp(b)``, device int32[1] each) when the
+    caller keeps them, as a layer does for its constant weight; otherwise they are found in every call.
     """
     import ctypes
 
@@ -313,13 +326,15 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
         first = {}                                   # one pass per distinct left operand (q / k / v share theirs)
         for i in range(n):
             j = first.setdefault(a2s[i].data_ptr(), i)
+            kept = b_exps[i] if b_exps is not None else None
             if j == i:
-                _lib.check(_lib.lib().cascmm_tensor_exp(a2s[i].data_ptr(), M, K, lda, dt, exps.data_ptr() + 8 * i, stream),
-                           "cascmm_tensor_exp(A)")
+                _activation_exps(a2s[i], lda, kept, exps.data_ptr() + 8 * i, stream)
             else:
                 exps[2 * i:2 * i + 1].copy_(exps[2 * j:2 * j + 1])
-            _lib.check(_lib.lib().cascmm_tensor_exp(b_list[i].data_ptr(), K, N, max(N, 1), dt,
-                                                    exps.data_ptr() + 8 * i + 4, stream), "cascmm_tensor_exp(B)")
+                if kept is not None:
+                    exps[2 * i + 1:2 * i + 2].copy_(kept.reshape(1))
+            if kept is None:
+                _activation_exps(b_list[i], max(N, 1), None, exps.data_ptr() + 8 * i + 4, stream)
     # 16-bit tensors as one term of their own format: room for every right operand re-laid as operand slots
     ws = None
     if a_list[0].dtype != torch.float32:

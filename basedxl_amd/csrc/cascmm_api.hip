@@ -232,8 +232,9 @@ __global__ void fill_bias_kernel(void* C, const void* bias, int M, int N, int64_
 // exponent e with max|x| * 2^e in (224, 448]
 __global__ void amax_begin_kernel(int32_t* exp_out) { *exp_out = 0; }
 
+// bit pattern of max|x| over the elements this thread visits, reduced over its wave
 template <int IODT>
-__global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld, int32_t* exp_out) {
+__device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64_t cols, int64_t ld) {
   typedef typename IoType<IODT>::T T;
   const T* src = (const T*)x;
   unsigned best = 0;
@@ -264,18 +265,52 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t rows, 
     const unsigned other = (unsigned)__shfl_xor((int)best, off, 64);
     best = other > best ? other : best;
   }
-  if ((threadIdx.x & 63) == 0 && best != 0) atomicMax((unsigned*)exp_out, best);
+  return best;
 }
 
-__global__ void amax_end_kernel(int32_t* exp_out) {
-  const unsigned bits = (unsigned)*exp_out;
+// the exponent e with max|x| * 2^e in (224, 448], from the bit pattern of max|x|
+__device__ __forceinline__ int exp_of_amax(unsigned bits) {
   int e = 0;
   if (bits != 0 && bits < 0x7F800000u) {   // finite and non-zero
     int ex;
     const float m = frexpf(__builtin_bit_cast(float, bits), &ex);   // m in [0.5, 1)
     e = m <= 0.875f ? 9 - ex : 8 - ex;                              // 448 = 0.875 * 2^9
   }
-  *exp_out = e;
+  return e;
+}
+
+template <int IODT>
+__global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld, int32_t* exp_out) {
+  const unsigned best = amax_scan<IODT>(x, rows, cols, ld);
+  if ((threadIdx.x & 63) == 0 && best != 0) atomicMax((unsigned*)exp_out, best);
+}
+
+__global__ void amax_end_kernel(int32_t* exp_out) { *exp_out = exp_of_amax((unsigned)*exp_out); }
+
+// The same search in ONE launch.  scratch = {running max, arrival count}, both zero on entry: every
+// workgroup folds its maximum in, fences, and takes a ticket; the one that draws the last ticket sees
+// every other workgroup's contribution, writes {e_x, *second} and leaves the scratch zeroed for the
+// next call.  No workgroup waits for another.
+template <int IODT>
+__global__ __launch_bounds__(256) void amax_single_launch_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld,
+                                                                 const int32_t* second, int32_t* exps_out, unsigned* scratch) {
+  __shared__ unsigned wave_best[4];
+  const unsigned best = amax_scan<IODT>(x, rows, cols, ld);
+  if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  unsigned b = wave_best[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) b = wave_best[w] > b ? wave_best[w] : b;
+  if (b != 0) atomicMax(&scratch[0], b);
+  __threadfence();
+  const unsigned ticket = atomicAdd(&scratch[1], 1u);
+  if (ticket != gridDim.x - 1) return;
+  __threadfence();
+  const unsigned bits = atomicExch(&scratch[0], 0u);
+  atomicExch(&scratch[1], 0u);
+  exps_out[0] = exp_of_amax(bits);
+  if (second) exps_out[1] = *second;
 }
 
 template <int IODT, int FMT, int TERMS>
@@ -644,6 +679,28 @@ int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int
       hipLaunchKernelGGL((amax_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
   }
   hipLaunchKernelGGL(amax_end_kernel, dim3(1), dim3(1), 0, s, exp_out);
+  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+}
+
+int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const int32_t* second_exp,
+                       int32_t* exps_out, int32_t* scratch, void* stream) {
+  if (dtype != CASCMM_DT_F32 && dtype != CASCMM_DT_F16 && dtype != CASCMM_DT_BF16) return CASCMM_ERR_BAD_DTYPE;
+  if (rows < 0 || cols < 0 || ld < cols) return CASCMM_ERR_BAD_SHAPE;
+  if (!exps_out || !scratch || (rows * cols > 0 && !x)) return CASCMM_ERR_NULL_POINTER;
+  if (rows > INT32_MAX || cols > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t total = rows * cols;
+  // (an empty tensor: one workgroup that scans nothing and writes e = 0)
+  const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((total + 4095) / 4096, 1024));
+  if (dtype == CASCMM_DT_F32)
+    hipLaunchKernelGGL((amax_single_launch_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+                       exps_out, (unsigned*)scratch);
+  else if (dtype == CASCMM_DT_F16)
+    hipLaunchKernelGGL((amax_single_launch_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+                       exps_out, (unsigned*)scratch);
+  else
+    hipLaunchKernelGGL((amax_single_launch_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+                       exps_out, (unsigned*)scratch);
   return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 

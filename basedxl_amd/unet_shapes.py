@@ -138,11 +138,19 @@ def time_shapes(shapes: List[LinearShape], lowp: str, terms: int, prepared: bool
             def run():
                 cascaded_lowp_matmul_prepared([a] * s.group, pw, outs=outs)
         elif s.group > 1:
+            # fp8: a layer keeps the scale of its constant weight (modules/lowp_linear.py); the scale of
+            # the activations is found in every call
+            from . import tensor_scale_exp
+            wexp = [tensor_scale_exp(w) for w in ws] if lowp == "fp8" else None
+
             def run():
-                cascaded_lowp_matmul_grouped([a] * s.group, ws, outs=outs, lowp=lowp, terms=terms)
+                cascaded_lowp_matmul_grouped([a] * s.group, ws, outs=outs, lowp=lowp, terms=terms, b_exps=wexp)
         else:
+            from . import tensor_scale_exp
+            wexp = tensor_scale_exp(ws[0]) if lowp == "fp8" else None
+
             def run():
-                cascaded_lowp_matmul(a, ws[0], out=outs[0], lowp=lowp, terms=terms)
+                cascaded_lowp_matmul(a, ws[0], out=outs[0], lowp=lowp, terms=terms, b_exp=wexp)
         if gate == "unfused":
             gemm, gated_out = run, torch.empty(s.M, s.N // 2, device=dev, dtype=tdt)
 
@@ -186,7 +194,7 @@ def main(argv=None) -> None:
     ap.add_argument("--convs", action="store_true", help="include the 1x1 shortcut convolutions as GEMMs")
     ap.add_argument("--cascades", default="bf16x2,fp8x3")
     ap.add_argument("--prepared", action="store_true", help="split the weights once (PreparedWeight)")
-    ap.add_argument("--static-scales", action="store_true", help="fp8: tensor scales found once, not in every call")
+    ap.add_argument("--static-scales", action="store_true", help="fp8: the activation scale too is found once, not in every call (the weight scale always is)")
     ap.add_argument("--geglu", choices=["off", "unfused", "fused"], default="off",
                     help="gated projections: time the GEMM alone, with torch's gate after it, or the fused kernel")
     ap.add_argument("--dtype", choices=["fp32", "fp16", "bf16"], default="fp32",

@@ -188,6 +188,15 @@ const char* cascmm_variant_name(int variant);
 int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype,
                       int32_t* exp_out, void* stream);
 
+/* The same search in one kernel launch, for the per-call scale of the activations in front of a
+ * layer whose weight scale is kept (the counterpart of a layer's one-time weight preparation,
+ * basedxl/modules/lowp_linear.py:12): writes exps_out[0] = e of x and, when second_exp is non-NULL,
+ * exps_out[1] = *second_exp, i.e. the {e_A, e_B} pair cascmm_gemm takes.  scratch: two device int32
+ * that are zero before the first call; every call leaves them zero again.  Calls that share a
+ * scratch must be ordered (one stream). */
+int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype,
+                       const int32_t* second_exp, int32_t* exps_out, int32_t* scratch, void* stream);
+
 /* The operand split alone (a test hook for parity of the split with the CPU oracle):
  * out is fp32 [terms][n]; term i holds lowp(r_i * 2^(tensor_exp + shift*i)) upcast to fp32
  * with r_0 = x, r_{i+1} = r_i - t_i / 2^(tensor_exp + shift*i); shift = 0 / 11 / 4 for

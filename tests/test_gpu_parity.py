@@ -107,6 +107,41 @@ def test_tensor_exp_edges(gpu_device, values):
     assert int(ed.cpu()[0]) == oc.tensor_scale_exp(x, "fp8"), values
 
 
+def test_single_launch_scale_search_equals_the_oracle_call_after_call(gpu_device):
+    """cascmm_tensor_exps: one launch, many workgroups, a scratch pair that every call must leave
+    zeroed.  Tensors of every layout the scan distinguishes (contiguous fp32, padded rows, 16-bit),
+    sizes from one element to thousands of workgroups' worth, the maximum placed in the first, the
+    last and a middle element; the kept exponent of the other operand is passed through."""
+    _say("single-launch scale search")
+    l, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
+    scratch = torch.zeros(2, dtype=torch.int32, device="cuda:0")
+    kept = torch.tensor([-7], dtype=torch.int32, device="cuda:0")
+    out = torch.full((2,), 99, dtype=torch.int32, device="cuda:0")
+    g = torch.Generator().manual_seed(17)
+    case = 0
+    for rows, cols, pad in [(1, 1, 0), (3, 2, 3), (7, 333, 0), (64, 64, 0), (154, 2048, 0), (4096, 640, 0), (1000, 1003, 5),
+                            (8192, 1280, 0), (0, 16, 0)]:
+        for dtype, code in [(torch.float32, _lib.DT_F32), (torch.float16, _lib.DT_F16), (torch.bfloat16, _lib.DT_BF16)]:
+            for where in ("first", "last", "middle"):
+                case += 1
+                x = (torch.randn(rows, cols, generator=g) * 10.0 ** float(torch.randint(-3, 3, (1,), generator=g))).to(dtype)
+                if x.numel():
+                    flat = x.view(-1)
+                    flat[{"first": 0, "last": -1, "middle": x.numel() // 2}[where]] = flat.abs().max() * 3
+                store = torch.full((rows, cols + pad), 6e4, dtype=dtype)              # junk beyond each row's cols
+                store[:, :cols] = x
+                xd = store.to("cuda:0")
+                second = kept if case % 2 else None
+                out.fill_(99)
+                st = l.cascmm_tensor_exps(xd.data_ptr(), rows, cols, cols + pad, code, second.data_ptr() if second is not None else None,
+                                          out.data_ptr(), scratch.data_ptr(), stream)
+                assert st == 0, l.cascmm_strerror(st)
+                got = out.cpu().tolist()
+                assert got[0] == oc.tensor_scale_exp(x.float(), "fp8"), (rows, cols, pad, dtype, where)
+                assert got[1] == (-7 if second is not None else 99)
+    assert scratch.cpu().tolist() == [0, 0]
+
+
 # ---------------------------------------------------------------------------------------
 # exact integer known-answer tests, every kernel variant, ragged shapes
 # ---------------------------------------------------------------------------------------
