@@ -98,7 +98,7 @@ static const TunedCost kTuned[] = {
     {"t64x64x64_w2x2x1_d3_bf16x2_tri", 0.671, 2.34, 1.00, 1.00},
     {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.064, 4.69, 0.90, 0.80},
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.224, 6.84, 0.80, 0.70},
-    {"t256x160x32_w4x1x1_d2_bf16x2_tri", 2.907, 13.81, 0.70, 0.50},
+    {"t256x160x32_w4x1x1_d2_bf16x2_tri", 3.250, 5.00, 0.70, 0.50},
     // three fp16 / bf16 terms
     {"t128x128x32_w4x2x1_d2_fp16x3_tri", 3.107, 7.22, 0.90, 0.80},
     {"t64x64x32_w2x2x1_d3_fp16x3_tri", 1.088, 2.27, 1.00, 1.00},
