@@ -82,6 +82,31 @@ def test_select_variant_prefers_sensible_tiles():
     assert l.cascmm_select_variant(4, 4, 4, 4, 4, 4, 0, 5, 2, 0) == -4
 
 
+def test_baseline_shapes_get_the_kernels_the_measurements_name():
+    """The kernels behind the committed profiles and the bench's traffic figures: if the cost model
+    drifts to another tile for these shapes, those figures describe the wrong kernel."""
+    l = _lib.lib()
+    names = _lib.variant_names()
+    pick = lambda M, K, N: names[l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0) & 0xFFFF]
+    assert pick(2048, 1280, 10240) == "t256x160x32_w4x1x1_d2_bf16x2_tri"          # cfg3, first GEMM
+    assert pick(154, 2048, 1280).startswith("skinny") and pick(154, 2048, 640).startswith("skinny")   # cfg4
+    grouped = names[l.cascmm_select_variant_grouped(3, 4096, 640, 640, 640, 640, 640, 0, 0, 2, 0) & 0xFFFF]
+    assert grouped == "t256x128x32_w4x1x1_d2_bf16x2_tri"                           # cfg2, to_q / to_k / to_v
+    assert pick(4096, 640, 640) == "t64x160x64_w2x1x2_d2_p8_bf16x2_tri"            # cfg2, to_out
+
+
+def test_scale_search_argument_validation():
+    l = _lib.lib()
+    ok = 16   # any non-NULL value: these calls return before touching the device
+    assert l.cascmm_tensor_exps(ok, 4, 4, 4, 7, None, ok, ok, None) == -3          # dtype
+    assert l.cascmm_tensor_exps(ok, 4, 4, 3, 0, None, ok, ok, None) == -2          # ld < cols
+    assert l.cascmm_tensor_exps(ok, -1, 4, 4, 0, None, ok, ok, None) == -2
+    assert l.cascmm_tensor_exps(None, 4, 4, 4, 0, None, ok, ok, None) == -1
+    assert l.cascmm_tensor_exps(ok, 4, 4, 4, 0, None, None, ok, None) == -1
+    assert l.cascmm_tensor_exps(ok, 4, 4, 4, 0, None, ok, None, None) == -1         # the scratch is not optional
+    assert l.cascmm_tensor_exps(ok, 2 ** 31, 4, 4, 0, None, ok, ok, None) == -9
+
+
 def test_cpu_tensors_are_rejected_without_fallback():
     import torch
     from basedxl_amd import cascaded_lowp_matmul
@@ -103,7 +128,8 @@ def test_unet_shape_table_matches_the_architecture():
     assert sum(s.count for s in full if s.name.startswith("attn1.to_out")) == 70
     assert 8.0e12 < total_flops(full) < 9.5e12
     half = sdxl_linear_shapes(half_latent=True)
-    kv = [s for s in half if s.name.startswith("attn2.to_k/v")]
+    kv = [s for s in half if s.name.startswith("attn2.to_kv")]
+    assert len(kv) == 2
     assert all(s.M == 154 and s.K == 2048 for s in kv)
     assert [s.M for s in half if s.name.startswith("attn1.to_out")] == [4096, 1024]
     assert 0.5 * total_flops(full) < total_flops(half) < 0.52 * total_flops(full) + total_flops(kv)
