@@ -220,3 +220,41 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), (rep, i)
+
+
+def test_operands_beyond_two_gib_are_addressed_correctly(gpu_device):
+    """The fast kernels address rows through 32-bit offsets from a per-tile buffer descriptor, the
+    bounds-checked ones through 64-bit pointers: a left operand and a result of 2.3 GB each (row offsets
+    cross 2^31 bytes inside the matrix) and a right operand of 2.4 GB must give the exact integer
+    products in the rows on both sides of every boundary.  Operands are made on the device; only the
+    sampled rows are recomputed (in float64, exact for these integers)."""
+    from basedxl_amd import cascaded_lowp_matmul_grouped
+
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(3)
+    ints = lambda *shape, hi=7: torch.randint(-hi, hi + 1, shape, device=dev, generator=g).to(torch.float32)
+    M, K, N = 900_000, 640, 640
+    a, b, bias = ints(M, K), ints(K, N), ints(N)
+    edge = (2 ** 31) // (K * 4)                    # first row that starts beyond 2^31 bytes
+    rows = torch.tensor([0, 1, 255, 256, edge - 1, edge, edge + 1, edge + 300, M - 257, M - 2, M - 1], device=dev)
+    want = a[rows].double() @ b.double() + bias.double()
+    for kw in (dict(), dict(lowp="fp16", terms=3), dict(lowp="fp8", terms=3, products="full")):
+        c = cascaded_lowp_matmul(a, b, bias=bias, **kw)
+        assert torch.equal(c[rows].double(), want), kw
+        del c
+    c = cascaded_lowp_matmul(a, PreparedWeight(b), bias=bias)
+    assert torch.equal(c[rows].double(), want)
+    del c
+    second = cascaded_lowp_matmul_grouped([a, a], [b, b.clone()])[1]
+    assert torch.equal(second[rows].double(), want - bias.double())
+    del second, a
+    torch.cuda.empty_cache()
+    # a right operand beyond 2 GiB takes the kernels with 64-bit addressing
+    M, K, N = 96, 16384, 36864
+    a, b = ints(M, K, hi=3), ints(K, N, hi=3)
+    assert b.numel() * 4 > 2 ** 31
+    assert torch.equal(cascaded_lowp_matmul(a, b).double(), a.double() @ b.double())
+    b2 = b[:, :32000].contiguous()                 # just under 2 GiB: the fast split-K kernels for few rows
+    assert torch.equal(cascaded_lowp_matmul(a, b2).double(), a.double() @ b2.double())
+    del a, b, b2
+    torch.cuda.empty_cache()
