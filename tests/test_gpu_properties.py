@@ -258,3 +258,35 @@ def test_operands_beyond_two_gib_are_addressed_correctly(gpu_device):
     assert torch.equal(cascaded_lowp_matmul(a, b2).double(), a.double() @ b2.double())
     del a, b, b2
     torch.cuda.empty_cache()
+
+
+def test_two_streams_do_not_share_scratch(gpu_device):
+    """The library keeps no state; the Python operator keeps one workspace (K-split partials, re-laid
+    16-bit weights) and one scale-search scratch PER STREAM.  Launches that need them, issued
+    alternately on two streams with different operands, must give what each gives alone."""
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    jobs = []
+    for i in range(2):
+        jobs.append(dict(x=rn(1024, 5120), w=rn(5120, 1280) * 0.02,                       # K split: partials in the workspace
+                         xh=rn(1024, 640).half(), wh=(rn(640, 640) * 0.02).half(),        # 16-bit: weight re-laid into it
+                         x8=rn(512, 320) * (1 + 10 * i), w8=rn(320, 640) * 0.02))         # fp8: scale found on the device
+
+    def run(j):
+        return [cascaded_lowp_matmul(j["x"], j["w"]), cascaded_lowp_matmul(j["xh"], j["wh"]),
+                cascaded_lowp_matmul(j["x8"], j["w8"], lowp="fp8", terms=3)]
+
+    alone = [run(j) for j in jobs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [[], []]
+    for rep in range(8):
+        for i, s in enumerate(streams):
+            with torch.cuda.stream(s):
+                got[i].append(run(jobs[i]))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for outs in got[i]:
+            for a, b in zip(outs, alone[i]):
+                assert torch.equal(a, b)
