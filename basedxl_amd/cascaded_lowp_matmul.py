@@ -23,19 +23,70 @@ from . import _lib
 
 _DTYPES = {torch.float32: _lib.DT_F32, torch.float16: _lib.DT_F16, torch.bfloat16: _lib.DT_BF16}
 
-#: persistent zero-initialised split-K workspaces, one per (device index, stream handle)
-_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+#: persistent split-K / re-lay workspaces (contents need no initialisation), one per (device index,
+#: stream handle) for eager launches and one per device (key "capture") for launches recorded into a
+#: device graph
+_workspaces: Dict[Tuple[int, object], torch.Tensor] = {}
+_MIN_WORKSPACE = 1 << 20
+
+
+def reserve_workspace(nbytes: int, device=None) -> None:
+    """Make sure the workspace that launches recorded into a device graph use holds ``nbytes``, so
+    that a capture allocates nothing.  Every eager launch does this for its own need, so a capture
+    that follows the usual eager warm-up of the same calls finds its workspace already there."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), "capture")
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _workspaces[key] = torch.empty(max(nbytes, _MIN_WORKSPACE), dtype=torch.uint8, device=dev)
 
 
 def _workspace(device: torch.device, stream: int, nbytes: int) -> Optional[torch.Tensor]:
+    """Launches on one stream are ordered, so they can share one buffer; launches replayed from
+    graphs share the per-device capture buffer (graphs that use it must not replay concurrently)."""
     if nbytes == 0:
         return None
-    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if torch.cuda.is_current_stream_capturing():
+        ws = _workspaces.get((index, "capture"))
+        if ws is None or ws.numel() < nbytes:
+            # no eager warm-up came first: the buffer comes from the graph's own pool (an
+            # allocation inside the capture, but no fill: nothing is recorded for it)
+            ws = _workspaces[(index, "capture")] = torch.empty(max(nbytes, _MIN_WORKSPACE), dtype=torch.uint8, device=device)
+        return ws
+    reserve_workspace(nbytes, device)
+    key = (index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        ws = torch.empty(max(nbytes, _MIN_WORKSPACE), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+_ws_need: Dict[tuple, int] = {}
+
+
+def _workspace_bytes(M: int, N: int, K: int, dt: int, fmt: int, terms: int, products: int) -> int:
+    """cascmm_workspace_bytes, remembered per problem (it walks the whole variant table)."""
+    key = (M, N, K, dt, fmt, terms, products)
+    need = _ws_need.get(key)
+    if need is None:
+        need = _ws_need[key] = _lib.lib().cascmm_workspace_bytes(M, N, K, dt, fmt, terms, products)
+    return need
+
+
+def _check_bias(bias: Optional[torch.Tensor], like: torch.Tensor, n: int) -> Optional[torch.Tensor]:
+    """A bias the kernels can read: on the device of ``like``, its dtype, 1-D, ``n`` long, contiguous.
+    Checked before any launch: the C side sees only a pointer."""
+    if bias is None:
+        return None
+    _check_device_tensor(bias, "bias")
+    if bias.device != like.device:
+        raise ValueError(f"bias is on {bias.device} but the operands are on {like.device}")
+    if bias.dtype != like.dtype or bias.dim() != 1 or bias.shape[0] != n:
+        raise ValueError(f"bias must be a 1-D tensor of length N = {n} with the dtype of a ({like.dtype}), "
+                         f"got shape {tuple(bias.shape)} {bias.dtype}")
+    return bias.contiguous()
 
 
 _exp_scratch: Dict[Tuple[int, int], torch.Tensor] = {}
@@ -45,7 +96,11 @@ def _activation_exps(a2: torch.Tensor, lda: int, second: Optional[torch.Tensor],
     """{e_A, e_B} at ``out_ptr`` (device int32[2]) in one launch: the fp8 scale exponent of ``a2`` found
     on the device, next to the kept exponent ``second`` of the other operand (skipped when None)."""
     dev = a2.device
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    capturing = torch.cuda.is_current_stream_capturing()
+    key = (index, "capture" if capturing else stream)
+    if not capturing and (index, "capture") not in _exp_scratch:
+        _exp_scratch[(index, "capture")] = torch.zeros(2, dtype=torch.int32, device=dev)
     scratch = _exp_scratch.get(key)
     if scratch is None:
         scratch = _exp_scratch[key] = torch.zeros(2, dtype=torch.int32, device=dev)   # the kernel leaves it zeroed
@@ -132,6 +187,11 @@ class PreparedWeight:
                    exp: Optional[torch.Tensor] = None) -> "PreparedWeight":
         """The object around operand slots that already exist (``prepared.slots`` of an earlier
         preparation with the same K, N, dtype and cascade); nothing is computed."""
+        if lowp not in _lib.FMT_BY_NAME:
+            raise ValueError(f"lowp must be one of {sorted(_lib.FMT_BY_NAME)}, got {lowp!r}")
+        if lowp == "fp8" and (exp is None or exp.dtype != torch.int32 or exp.numel() != 1 or exp.device != slots.device):
+            raise ValueError("fp8 operand slots need the tensor-scale exponent they were prepared with "
+                             "(exp: int32[1] on the device of the slots)")
         self = cls.__new__(cls)
         self.K, self.N, self.shape = int(K), int(N), (int(K), int(N))
         self.lowp, self.terms, self.fmt = lowp, int(terms), _lib.FMT_BY_NAME[lowp]
@@ -141,16 +201,33 @@ class PreparedWeight:
         self.exp, self.slots = exp, slots
         return self
 
-    def usable_with(self, a2: torch.Tensor) -> bool:
+    def usable_with(self, a2: torch.Tensor, products: str = "tri") -> bool:
         """Whether the prepared kernels take this left operand: fp32 (or fp16 / bf16 tensors with a
         weight of the same dtype kept as one term of that format), K a multiple of 64, rows 16-byte
         aligned (anything else goes through the raw weight)."""
         if self.K % 64 != 0 or self.N % 4 != 0 or a2.data_ptr() % 16 != 0:
             return False
+        if not self.has_kernel(a2.dtype, products):
+            return False
         if a2.dtype == torch.float32:
             return a2.shape[0] <= 1 or a2.stride(0) % 4 == 0
         return (a2.dtype == self.dtype and self.terms == 1 and default_cascade(a2.dtype)[0] == self.lowp
                 and (a2.shape[0] <= 1 or a2.stride(0) % 8 == 0))
+
+    def has_kernel(self, dtype: torch.dtype, products: str = "tri") -> bool:
+        """Whether the library has a prepared-operand kernel for this weight's cascade with left
+        operands of ``dtype`` (a host-side table lookup, remembered)."""
+        key = (dtype, products)
+        hit = self._kernel_known.get(key) if hasattr(self, "_kernel_known") else None
+        if hit is None:
+            if not hasattr(self, "_kernel_known"):
+                self._kernel_known = {}
+            st = -1
+            if dtype in _DTYPES and products in _lib.PROD_BY_NAME:
+                st = _lib.lib().cascmm_select_variant_prepared(1, 256, self.N, self.K, self.K, self.out_features, _DTYPES[dtype],
+                                                               self.fmt, self.terms, _lib.PROD_BY_NAME[products])
+            hit = self._kernel_known[key] = st >= 0
+        return hit
 
 
 def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, products: str = "tri", variant: int = -1):
@@ -196,7 +273,11 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
         if o.numel() != M * NO or not o.is_contiguous() or o.dtype != adt:
             raise ValueError("every out must be a contiguous [M, N] tensor of the dtype of a")
     if biases is not None:
-        biases = [None if bb is None else bb.contiguous() for bb in biases]
+        if len(biases) != n:
+            raise ValueError("one bias (or None) per problem")
+        biases = [_check_bias(bb, a2s[0], N) for bb in biases]   # (a gated weight takes all N = 2 * inner entries)
+    if w0.fmt == _lib.FMT_FP8 and any(w.exp is None for w in w_list):
+        raise ValueError("an fp8 PreparedWeight needs its tensor-scale exponent (exp)")
     arr = ctypes.c_void_p * n
     pa = arr(*[t.data_ptr() for t in a2s])
     pb = arr(*[w.slots.data_ptr() for w in w_list])
@@ -222,7 +303,7 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
         # room for the partial results of a K split (single fp32 problems with few tiles)
         ws = None
         if n == 1 and adt == torch.float32:
-            need = _lib.lib().cascmm_workspace_bytes(M, N, K, _DTYPES[adt], w0.fmt, w0.terms, _lib.PROD_BY_NAME[products])
+            need = _workspace_bytes(M, N, K, _DTYPES[adt], w0.fmt, w0.terms, _lib.PROD_BY_NAME[products])
             ws = _workspace(dev, stream, need)
         st = _lib.lib().cascmm_gemm_prepared(*common, ws.data_ptr() if ws is not None else None,
                                              ws.numel() if ws is not None else 0, stream, variant)
@@ -238,7 +319,7 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
     dt = _DTYPES[a2.dtype]
     l = _lib.lib()
     stream = torch.cuda.current_stream(a2.device).cuda_stream
-    ws_bytes = l.cascmm_workspace_bytes(M, N, K, dt, fmt, terms, products)
+    ws_bytes = _workspace_bytes(M, N, K, dt, fmt, terms, products)
     ws = _workspace(a2.device, stream, ws_bytes)
     exps = None
     if fmt == _lib.FMT_FP8 and tensor_exps is not None:
@@ -311,7 +392,9 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
         if o.numel() != M * N or not o.is_contiguous() or o.dtype != a_list[0].dtype:
             raise ValueError("every out must be a contiguous [M, N] tensor of the dtype of a")
     if biases is not None:
-        biases = [None if bb is None else bb.contiguous() for bb in biases]
+        if len(biases) != n:
+            raise ValueError("one bias (or None) per problem")
+        biases = [_check_bias(bb, a2s[0], N) for bb in biases]
     arr = ctypes.c_void_p * n
     pa = arr(*[t.data_ptr() for t in a2s])
     pb = arr(*[t.data_ptr() for t in b_list])
@@ -338,7 +421,7 @@ def cascaded_lowp_matmul_grouped(a_list, b_list, *, outs=None, biases=None, lowp
     # 16-bit tensors as one term of their own format: room for every right operand re-laid as operand slots
     ws = None
     if a_list[0].dtype != torch.float32:
-        need = _lib.lib().cascmm_workspace_bytes(M, N, K, _DTYPES[a_list[0].dtype], fmt, terms, prod)
+        need = _workspace_bytes(M, N, K, _DTYPES[a_list[0].dtype], fmt, terms, prod)
         ws = _workspace(dev, stream, n * need) if need else None
     st = _lib.lib().cascmm_gemm_grouped(n, pa, pb, pc, pbias, M, N, K, lda, max(N, 1), max(N, 1),
                                         _DTYPES[a_list[0].dtype], fmt, terms, prod,
@@ -395,11 +478,7 @@ def cascaded_lowp_matmul(
     if products not in _lib.PROD_BY_NAME:
         raise ValueError(f"products must be 'tri' or 'full', got {products!r}")
     fmt, prod = _lib.FMT_BY_NAME[lowp], _lib.PROD_BY_NAME[products]
-    if bias is not None:
-        _check_device_tensor(bias, "bias")
-        if bias.dtype != a.dtype or bias.dim() != 1 or bias.shape[0] != b.shape[-1]:
-            raise ValueError("bias must be a 1-D tensor of length N with the dtype of a")
-        bias = bias.contiguous()
+    bias = _check_bias(bias, a, b.shape[-1])
 
     K, N = b.shape[-2], b.shape[-1]
 

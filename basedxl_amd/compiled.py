@@ -25,7 +25,7 @@ def cascade_linear(x: torch.Tensor, weight: torch.Tensor, slots: Optional[torch.
         pw = PreparedWeight.from_slots(slots, K, N, weight.dtype, lowp, terms, glu, b_exp)
         x2 = x.reshape(-1, K)
         few_rows = x2.shape[0] < 32 and x2.dtype == torch.float32 and not glu
-        if glu or (not few_rows and pw.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous())):
+        if glu or (not few_rows and pw.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous(), products)):
             return cascaded_lowp_matmul(x, pw, bias=bias, products=products)
     return cascaded_lowp_matmul(x, weight, bias=bias, lowp=lowp, terms=terms, products=products, b_exp=b_exp)
 

@@ -2,6 +2,8 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <unordered_map>
 #include <vector>
 
 #include "cascmm_variants.h"
@@ -29,6 +31,12 @@ static const std::vector<VariantDesc>& table() {
   }();
   return t;
 }
+
+struct TunedCost;
+// per variant, resolved once when the table is built: its measured cost constants (or none) and what
+// kind of kernel its name says it is
+struct VariantInfo { const TunedCost* tuned; bool p8; bool bdirect; };
+static const std::vector<VariantInfo>& variant_info();
 
 static bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 static size_t dtype_size(int dt) { return dt == CASCMM_DT_F32 ? 4 : 2; }
@@ -122,11 +130,27 @@ static const TunedCost kTuned[] = {
 
 constexpr int kMaxTileSplits = 4;
 
+static const std::vector<VariantInfo>& variant_info() {
+  static const std::vector<VariantInfo> info = [] {
+    std::vector<VariantInfo> v;
+    for (const VariantDesc& d : table()) {
+      VariantInfo i{nullptr, strstr(d.name, "_p8_") != nullptr, d.name[0] == 'b' && d.name[1] == 'd'};
+      for (const TunedCost& t : kTuned)
+        if (strcmp(t.name, d.name) == 0) i.tuned = &t;
+      v.push_back(i);
+    }
+    return v;
+  }();
+  return info;
+}
+
 // ws_bytes: workspace the caller brought; *splits_out: K split the cost was computed for (the
 // LDS-tiled two-term bf16 kernels may split K over up to kMaxTileSplits work items per tile when a
 // single problem has too few tiles to occupy the chip and the workspace holds the partials)
-static double variant_cost(const VariantDesc& v, const Problem& q, int count, size_t ws_bytes = 0,
+static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes = 0,
                            int* splits_out = nullptr) {
+  const VariantDesc& v = table()[vi];
+  const VariantInfo& info = variant_info()[vi];
   if (splits_out) *splits_out = 1;
   const double tiles = (double)count * (double)((q.M + v.BM - 1) / v.BM) * (double)((q.N + v.BN - 1) / v.BN);
   const double full = (double)(int64_t)(tiles / kNumCUs);
@@ -138,8 +162,8 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count, si
     if ((double)((q.M + 63) / 64) * (double)((q.N + 127) / 128) >= kNumCUs / 2) return 1e9;
     return 1e-6 * (double)(((q.M + v.BM - 1) / v.BM) * v.BM) + 1e-8 * v.BM;
   }
-  for (const TunedCost& t : kTuned) {
-    if (strcmp(t.name, v.name) != 0) continue;
+  if (info.tuned) {
+    const TunedCost& t = *info.tuned;
     const double tail = full == 0 ? t.tail_first : t.tail_later;
     const double rounds = full + (rem > 0 ? tail + (1.0 - tail) * rem / kNumCUs : 0.0);
     // tiles that hang over the edge of C take the bounds-checked epilogue and load clamped
@@ -165,12 +189,11 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count, si
   }
   const double rounds = full + (rem > 0 ? 0.55 + 0.45 * rem / kNumCUs : 0.0);
   double step = ((double)v.BM * v.BN + 64.0 * (v.BM + v.BN)) / 20000.0;
-  const char* name = v.name;
-  if (strstr(name, "_p8_")) step *= 0.94;
+  if (info.p8) step *= 0.94;
   const double ksteps = (double)((q.K + 63) / 64);
   // the plain B-direct kernels were slower than the LDS-tiled ones on every shape measured:
   // they stay selectable by index only
-  if (name[0] == 'b' && name[1] == 'd') return 1e6 + rounds * step * ksteps;
+  if (info.bdirect) return 1e6 + rounds * step * ksteps;
   double best = rounds * (step * ksteps + 5.0) + (v.fast ? 0.0 : 1e3);
   // the same K split as above for the kernels without measured constants (three-term and fp8
   // cascades on the shapes that leave CUs idle)
@@ -192,8 +215,57 @@ static double variant_cost(const VariantDesc& v, const Problem& q, int count, si
 }
 
 // ws_bytes: workspace the caller brought (split-K variants that need more are skipped)
+// The selection walks the whole table and costs every candidate; a model calls the same few dozen
+// problems over and over (eagerly, ~750 Linear calls per UNet step), so the answers are remembered.
+struct SelectKey {
+  int64_t M, N, K;
+  size_t ws_bytes;
+  int dtype, fmt, terms, products, count, flags;   // flags: fast | bpre << 1 | glu << 2
+  bool operator==(const SelectKey& o) const {
+    return M == o.M && N == o.N && K == o.K && ws_bytes == o.ws_bytes && dtype == o.dtype && fmt == o.fmt &&
+           terms == o.terms && products == o.products && count == o.count && flags == o.flags;
+  }
+};
+struct SelectKeyHash {
+  size_t operator()(const SelectKey& k) const {
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&](uint64_t v) { h = (h ^ v) * 1099511628211ull; };
+    mix((uint64_t)k.M); mix((uint64_t)k.N); mix((uint64_t)k.K); mix((uint64_t)k.ws_bytes);
+    mix(((uint64_t)k.dtype << 40) ^ ((uint64_t)k.fmt << 32) ^ ((uint64_t)k.terms << 24) ^ ((uint64_t)k.products << 16) ^
+        ((uint64_t)k.count << 8) ^ (uint64_t)k.flags);
+    return (size_t)h;
+  }
+};
+struct SelectHit { int variant, splits; };
+
+static int select_variant_uncached(const Problem& q, bool fast, int count, size_t ws_bytes, int* splits_out);
+
 static int select_variant(const Problem& q, bool fast, int count, size_t ws_bytes = (size_t)-1,
                           int* splits_out = nullptr) {
+  static std::mutex mu;
+  static std::unordered_map<SelectKey, SelectHit, SelectKeyHash> memo;
+  const SelectKey key{q.M, q.N, q.K, ws_bytes, q.dtype, q.fmt, q.terms, q.products, count,
+                      (fast ? 1 : 0) | (q.bpre ? 2 : 0) | (q.glu ? 4 : 0)};
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = memo.find(key);
+    if (it != memo.end()) {
+      if (splits_out) *splits_out = it->second.splits;
+      return it->second.variant;
+    }
+  }
+  int splits = 1;
+  const int v = select_variant_uncached(q, fast, count, ws_bytes, &splits);
+  {
+    std::lock_guard<std::mutex> lock(mu);
+    if (memo.size() >= 4096) memo.clear();
+    memo[key] = SelectHit{v, splits};
+  }
+  if (splits_out) *splits_out = splits;
+  return v;
+}
+
+static int select_variant_uncached(const Problem& q, bool fast, int count, size_t ws_bytes, int* splits_out) {
   const auto& t = table();
   int best = -1;
   double best_cost = 0;
@@ -205,7 +277,7 @@ static int select_variant(const Problem& q, bool fast, int count, size_t ws_byte
         skinny_workspace_bytes(q.M, q.N, q.K, t[i].BM, t[i].BN, t[i].BK) > ws_bytes)
       continue;
     int sp = 1;
-    const double c = variant_cost(t[i], q, count, ws_bytes, &sp);
+    const double c = variant_cost(i, q, count, ws_bytes, &sp);
     if (best < 0 || c < best_cost) {
       best = i;
       best_cost = c;
@@ -333,13 +405,14 @@ __global__ void split_terms_kernel(const void* x, float* out, int64_t n, int ten
 template <int IODT, int FMT>
 static int launch_split(const void* x, float* out, int64_t n, int terms, int tensor_exp, hipStream_t s) {
   const unsigned grid = (unsigned)((n + 255) / 256);
+  hipError_t err = hipSuccess;
   switch (terms) {
-    case 1: hipLaunchKernelGGL((split_terms_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
-    case 2: hipLaunchKernelGGL((split_terms_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
-    case 3: hipLaunchKernelGGL((split_terms_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
+    case 1: CASCMM_LAUNCH(err, (split_terms_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
+    case 2: CASCMM_LAUNCH(err, (split_terms_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
+    case 3: CASCMM_LAUNCH(err, (split_terms_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, x, out, n, tensor_exp); break;
     default: return CASCMM_ERR_BAD_FORMAT;
   }
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
 // Splits a weight once: thread (kg, n) reads the 8 values B[8 kg .. 8 kg + 7][n] (zero beyond K),
@@ -378,13 +451,14 @@ static int launch_prepare(const void* B, int K, int N, int64_t ldb, int terms, c
                           int glu) {
   const int64_t total = (int64_t)((K + 7) / 8) * N;
   const unsigned grid = (unsigned)((total + 255) / 256);
+  hipError_t err = hipSuccess;
   switch (terms) {
-    case 1: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
-    case 2: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
-    case 3: hipLaunchKernelGGL((prepare_weight_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
+    case 1: CASCMM_LAUNCH(err, (prepare_weight_kernel<IODT, FMT, 1>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
+    case 2: CASCMM_LAUNCH(err, (prepare_weight_kernel<IODT, FMT, 2>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
+    case 3: CASCMM_LAUNCH(err, (prepare_weight_kernel<IODT, FMT, 3>), dim3(grid), dim3(256), 0, s, B, K, N, ldb, e, out, glu); break;
     default: return CASCMM_ERR_BAD_FORMAT;
   }
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
 template <int IODT>
@@ -428,16 +502,17 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   if (q.K == 0) {
     const int64_t total = q.M * q.N;
     const unsigned grid = (unsigned)((total + 255) / 256);
+    hipError_t err = hipSuccess;
     for (int i = 0; i < count; ++i) {
       const void* b = bias ? bias[i] : nullptr;
       if (q.dtype == CASCMM_DT_F32)
-        hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
+        CASCMM_LAUNCH(err, (fill_bias_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
       else if (q.dtype == CASCMM_DT_F16)
-        hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
+        CASCMM_LAUNCH(err, (fill_bias_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
       else
-        hipLaunchKernelGGL((fill_bias_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
+        CASCMM_LAUNCH(err, (fill_bias_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, stream, C[i], b, (int)q.M, (int)q.N, q.ldc);
     }
-    return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+    return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
   }
   if (onthefly_prepare_ok(q, count, A, B, workspace, workspace_bytes)) {
     // fp16 x fp16 (bf16 x bf16) tensors as one term: re-lay B as operand slots in the workspace
@@ -624,10 +699,11 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
   // K split of the LDS-tiled kernels: up to kMaxTileSplits partial results when some kernel
   // would run the problem with at most half the CUs busy
   if (dtype == CASCMM_DT_F32 && N % 4 == 0) {
-    for (const auto& v : table()) {
+    for (int vi = 0; vi < (int)table().size(); ++vi) {
+      const VariantDesc& v = table()[vi];
       if (v.kind != KIND_TILE || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
       int sp = 1;
-      variant_cost(v, q, 1, (size_t)-1, &sp);
+      variant_cost(vi, q, 1, (size_t)-1, &sp);
       const size_t n = sp > 1 ? (size_t)kMaxTileSplits * M * N * sizeof(float) : 0;
       need = n > need ? n : need;
     }
@@ -667,19 +743,20 @@ int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int
   if (rows > INT32_MAX || cols > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
   hipStream_t s = (hipStream_t)stream;
   // *exp_out holds the bit pattern of the running max|x| until the last kernel replaces it
-  hipLaunchKernelGGL(amax_begin_kernel, dim3(1), dim3(1), 0, s, exp_out);
+  hipError_t err = hipSuccess;
+  CASCMM_LAUNCH(err, amax_begin_kernel, dim3(1), dim3(1), 0, s, exp_out);
   const int64_t total = rows * cols;
   if (total > 0) {
     const unsigned grid = (unsigned)std::min<int64_t>((total + 4095) / 4096, 1024);
     if (dtype == CASCMM_DT_F32)
-      hipLaunchKernelGGL((amax_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
+      CASCMM_LAUNCH(err, (amax_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
     else if (dtype == CASCMM_DT_F16)
-      hipLaunchKernelGGL((amax_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
+      CASCMM_LAUNCH(err, (amax_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
     else
-      hipLaunchKernelGGL((amax_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
+      CASCMM_LAUNCH(err, (amax_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, exp_out);
   }
-  hipLaunchKernelGGL(amax_end_kernel, dim3(1), dim3(1), 0, s, exp_out);
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  CASCMM_LAUNCH(err, amax_end_kernel, dim3(1), dim3(1), 0, s, exp_out);
+  return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
 int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, const int32_t* second_exp,
@@ -691,17 +768,18 @@ int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, in
   hipStream_t s = (hipStream_t)stream;
   const int64_t total = rows * cols;
   // (an empty tensor: one workgroup that scans nothing and writes e = 0)
+  hipError_t err = hipSuccess;
   const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((total + 4095) / 4096, 1024));
   if (dtype == CASCMM_DT_F32)
-    hipLaunchKernelGGL((amax_single_launch_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
   else if (dtype == CASCMM_DT_F16)
-    hipLaunchKernelGGL((amax_single_launch_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
   else
-    hipLaunchKernelGGL((amax_single_launch_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
-  return hipGetLastError() == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }
 
 int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms, int tensor_exp,

@@ -3,6 +3,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 #include "../../include/cascmm.h"
 
 namespace cascmm {
@@ -15,6 +18,28 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kWave = 64;
+
+// Kernel launch whose status is the return value of the launch call itself: polling the runtime's
+// "last error" afterwards would also return (and clear) an error some unrelated earlier call of the
+// process left behind.
+template <typename... KArgs, typename... Args>
+inline hipError_t launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                                Args&&... args) {
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "argument count does not match the kernel's signature");
+  std::tuple<KArgs...> vals{static_cast<KArgs>(args)...};
+  return std::apply(
+      [&](auto&... v) {
+        void* ptrs[] = {(void*)&v...};
+        return hipLaunchKernel((const void*)kernel, grid, block, ptrs, lds_bytes, stream);
+      },
+      vals);
+}
+// keeps the first failure of a sequence of launches in ERR
+#define CASCMM_LAUNCH(ERR, ...)                                \
+  do {                                                         \
+    const hipError_t cascmm_e_ = launch_kernel(__VA_ARGS__);   \
+    if ((ERR) == hipSuccess) (ERR) = cascmm_e_;                \
+  } while (0)
 
 // ---------------------------------------------------------------------------------------
 // memory element types (what A, B, C, bias are stored as)

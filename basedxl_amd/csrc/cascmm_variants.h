@@ -8,7 +8,30 @@
 namespace cascmm {
 
 enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1 };
-constexpr int kNumCUs = 256;  // MI355X
+constexpr int kNumCUs = 256;  // MI355X: what the cost model's constants were measured on
+constexpr int kMaxDevices = 64;
+
+// compute units of the current device (asked once per device; kNumCUs when no device answers, as in
+// a build container, where only the host-side selection logic runs)
+inline int device_index() {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess || d < 0 || d >= kMaxDevices) {
+    (void)hipGetLastError();   // a failure of this query is handled here and not left behind
+    return -1;
+  }
+  return d;
+}
+inline int device_cus() {
+  static int cus[kMaxDevices] = {0};
+  const int d = device_index();
+  if (d < 0) return kNumCUs;
+  if (cus[d] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess || n <= 0) n = kNumCUs;
+    cus[d] = n;   // (a benign race: every thread stores the same value)
+  }
+  return cus[d];
+}
 
 struct VariantDesc {
   const char* name;
@@ -29,20 +52,26 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
   constexpr int lds = LdsLayout<TL, Lowp<FMT>::planes(TERMS)>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] {
-      attr_err = hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    });
-    if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
+    // more than 64 KB of LDS must be asked for once per device (the attribute is per device)
+    static bool lds_set[kMaxDevices] = {false};
+    const int d = device_index();
+    if (d < 0) return CASCMM_ERR_LAUNCH;
+    if (!lds_set[d]) {
+      if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return CASCMM_ERR_LAUNCH;
+      lds_set[d] = true;
+    }
   }
-  // persistent grid: at most as many workgroups as can be resident at once
-  static std::once_flag occ_once;
-  static int per_cu = 1;
-  std::call_once(occ_once, [&] {
+  // persistent grid: at most as many workgroups as can be resident at once on this device
+  static int occupancy[kMaxDevices] = {0};
+  const int dev = device_index();
+  if (dev < 0) return CASCMM_ERR_LAUNCH;
+  int per_cu = occupancy[dev];
+  if (per_cu == 0) {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kfn, TL::NT, lds) == hipSuccess && n > 0) per_cu = n;
-  });
+    per_cu = (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kfn, TL::NT, lds) == hipSuccess && n > 0) ? n : 1;
+    occupancy[dev] = per_cu;
+  }
   const int splits = p.k_splits > 1 ? p.k_splits : 1;
   if (splits > 1) {
     // K split: fp32 only, one problem, partial results [split][M][N] in the workspace
@@ -53,16 +82,16 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
     if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
   }
   const int64_t total = (int64_t)splits * p.count * p.tiles_m * p.tiles_n;
-  const int64_t resident = (int64_t)kNumCUs * per_cu;
+  const int64_t resident = (int64_t)device_cus() * per_cu;
   const unsigned grid = (unsigned)(total < resident ? total : resident);
-  hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
-  if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+  if (launch_kernel(kfn, dim3(grid), dim3(TL::NT), lds, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
   if (splits > 1) {
     const int64_t elems = (int64_t)p.M * p.N;
     const int vec_out = p.ldc % 4 == 0 && (uintptr_t)p.C[0] % 16 == 0 && (uintptr_t)p.bias[0] % 16 == 0;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, stream,
-                       (const float*)p.workspace, splits, p.M, p.N, (const float*)p.bias[0], (float*)p.C[0], p.ldc, vec_out);
-    if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+    if (launch_kernel(splitk_reduce_kernel, dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, stream,
+                      (const float*)p.workspace, splits, p.M, p.N, (const float*)p.bias[0], (float*)p.C[0], p.ldc,
+                      vec_out) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
   }
   return CASCMM_OK;
 }
@@ -127,22 +156,24 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   constexpr int lds = LdsLayoutA<TL, TERMS>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] {
-      attr_err = hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    });
-    if (attr_err != hipSuccess) return CASCMM_ERR_LAUNCH;
+    // more than 64 KB of LDS must be asked for once per device (the attribute is per device)
+    static bool lds_set[kMaxDevices] = {false};
+    const int d = device_index();
+    if (d < 0) return CASCMM_ERR_LAUNCH;
+    if (!lds_set[d]) {
+      if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return CASCMM_ERR_LAUNCH;
+      lds_set[d] = true;
+    }
   }
   const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n * (unsigned)p.k_splits;
-  hipLaunchKernelGGL(kfn, dim3(grid), dim3(TL::NT), lds, stream, p);
-  if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+  if (launch_kernel(kfn, dim3(grid), dim3(TL::NT), lds, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
   if (SPLITK && p.k_splits > 1) {
     const int64_t total = (int64_t)gp.M * gp.N;
     const int vec_out = gp.ldc % 4 == 0 && (uintptr_t)p.C % 16 == 0 && (uintptr_t)p.bias % 16 == 0;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, p.partials,
-                       p.k_splits, gp.M, gp.N, (const float*)p.bias, (float*)p.C, gp.ldc, vec_out);
-    if (hipGetLastError() != hipSuccess) return CASCMM_ERR_LAUNCH;
+    if (launch_kernel(splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, p.partials,
+                      p.k_splits, gp.M, gp.N, (const float*)p.bias, (float*)p.C, gp.ldc, vec_out) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
   }
   return CASCMM_OK;
 }

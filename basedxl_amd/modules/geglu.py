@@ -63,7 +63,7 @@ class BasedXLLowPGEGLU(nn.Module):
             if self._prepared is None or self._prepared.device != self.weight.device:
                 self._prepared = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms, glu=True)
             x2 = x.reshape(-1, self.in_features)
-            if self._prepared.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous()):
+            if self._prepared.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous(), self.products):
                 return cascaded_lowp_matmul(x, self._prepared, bias=self.bias, products=self.products)
         h = cascaded_lowp_matmul(x, self.weight, bias=self.bias, lowp=self.lowp, terms=self.terms, products=self.products)
         value, gate = h.chunk(2, dim=-1)

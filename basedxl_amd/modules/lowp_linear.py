@@ -57,7 +57,7 @@ class BasedXLLowPLinear(nn.Module):
             # a handful of rows (time embeddings): the raw fp32 weight has split-K kernels that stream
             # it with every CU, the prepared path has none
             few_rows = x2.shape[0] < 32 and x2.dtype == torch.float32
-            if not few_rows and self._prepared_weight.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous()):
+            if not few_rows and self._prepared_weight.usable_with(x2 if x2.stride(-1) == 1 else x2.contiguous(), self.products):
                 return cascaded_lowp_matmul(x, self._prepared_weight, bias=self.bias, products=self.products)
         if self.lowp == "fp8" and (self._weight_exp is None or self._weight_exp.device != self.weight.device):
             self._weight_exp = tensor_scale_exp(self.weight)

@@ -113,16 +113,20 @@ def split_terms(x: torch.Tensor, fmt: str = "bf16", terms: int = 2,
 
 
 def cascade_matmul_ref(a: torch.Tensor, b: torch.Tensor, fmt: str = "bf16", terms: int = 2,
-                       products: str = "tri") -> torch.Tensor:
+                       products: str = "tri", a_exp: Optional[int] = None,
+                       b_exp: Optional[int] = None) -> torch.Tensor:
     """2-D cascade: fp32 A[M,K] . fp32 B[K,N] through split terms, fp32 accumulation.
 
     One fp32 matmul per kept product on the upcast terms (each elementwise product is
     exact in fp32: 8+8, 11+11 or 4+4 significand bits), products of one scale class
     (i + j) summed first, classes combined from the smallest to the largest magnitude.
+    ``a_exp`` / ``b_exp``: tensor-scale exponents to use instead of the operands' own
+    (fp8; for checking a sample of the rows or columns of a larger product, whose scale
+    comes from the whole tensor).
     """
     assert a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0]
-    ta, sa = split_terms(a, fmt, terms)
-    tb, sb = split_terms(b, fmt, terms)
+    ta, sa = split_terms(a, fmt, terms, a_exp)
+    tb, sb = split_terms(b, fmt, terms, b_exp)
     classes: Dict[int, torch.Tensor] = {}
     inv: Dict[int, float] = {}
     for (i, j) in product_set(terms, products):
