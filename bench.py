@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the cascaded low-precision matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload ffn|attn]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload ffn|attn|kv|unet]
 
 One "step" is one pass of the hot path over one batch of synthetic input:
 
@@ -12,7 +12,14 @@ One "step" is one pass of the hot path over one batch of synthetic input:
   X fp32 [M = 2 x 2048 tokens, K = 640] through four Linear weights W fp32 [640, 640] (to_q, to_k,
   to_v from X in one grouped launch, to_out from a second activation tensor).
 
-Every GEMM is a 2-term bf16 cascade with the three products hi.hi + hi.lo + lo.hi and fp32
+* ``--workload kv``: the cross-attention key / value projections of the 77 text tokens, X fp32 [154, 2048] x W fp32
+  [2048, 1280] and [2048, 640]: the skinny split-K path, reported in HBM GB/s over the algorithmic bytes;
+* ``--workload unet``: every Linear layer and 1x1 convolution of one SDXL UNet denoising step (batch 2, 128x128
+  latent, random weights), as the patched module tree of basedxl_amd.unet_skeleton calls them, full latent and
+  one GPU's half-latent share, 2-term bf16 and 3-term fp8 cascades.
+
+The default (ffn) line also carries the kv and unet figures under ``other_workloads``.
+Every GEMM of ffn / attn / kv is a 2-term bf16 cascade with the three products hi.hi + hi.lo + lo.hi and fp32
 accumulation.  Inputs are synthetic (seeded normal; weights x 0.02) and resident in HBM before the
 timed region.  Both operands are split inside the timed kernels.
 
@@ -120,8 +127,153 @@ def cpu_baseline(cpu_inputs, launches, repeats=5):
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"{repeats} timed repeats (median) of the full step ({sum(ln.gemms for ln in launches)} GEMMs), torch CPU "
-                  f"emulation: split + 3 fp32 matmuls per GEMM; {med * 1e3:.1f} ms per step",
+                  f"emulation: split + 3 fp32 matmuls per GEMM; {med * 1e3:.1f} ms per step; threads = min(os.cpu_count(), 16): "
+                  f"16 is this job's share of the host's cores",
     }
+
+
+
+def _graph_time_us(fn, reps, replays=5, spin_s=0.2):
+    """Average duration of one call of ``fn`` in microseconds: ``reps`` calls captured in one HIP graph,
+    replayed untimed until the clocks are up, then ``replays`` timed replays between two events."""
+    import torch
+
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(reps):
+            fn()
+    t_end = time.perf_counter() + spin_s
+    while time.perf_counter() < t_end:
+        g.replay()
+        torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (replays * reps)
+
+
+KV_TRAFFIC_BYTES = {1280: None, 640: None}   # HBM-side bytes per launch from rocprofv3 counters (see profiles/), when measured
+
+
+def bench_kv(dev, check=True):
+    """cfg4: the two cross-attention K/V projections of the text tokens; bandwidth-style figures
+    over the algorithmic bytes 4 (MK + KN + MN)."""
+    import torch
+    from basedxl_amd import cascaded_lowp_matmul, _lib
+    from oracle import cascade as oc
+
+    out = {"workload": "cfg4: cross-attention K/V projections of 2 x 77 text tokens, X fp32 [154,2048] ~N(0,1) x W fp32 "
+                       "[2048,N] ~N(0,0.02), N = 1280 and 640; 2-term bf16 cascade (3 products), one call each",
+           "gemms": []}
+    g = torch.Generator().manual_seed(SEED + 4)
+    x_cpu = torch.randn(154, 2048, generator=g)
+    x = x_cpu.to(dev)
+    total_bytes = total_us = 0.0
+    l = _lib.lib()
+    for n in (1280, 640):
+        w_cpu = torch.randn(2048, n, generator=g) * 0.02
+        w = w_cpu.to(dev)
+        res = torch.empty(154, n, device=dev)
+        us = _graph_time_us(lambda: cascaded_lowp_matmul(x, w, out=res), reps=20)
+        algo = 4 * (154 * 2048 + 2048 * n + 154 * n)
+        rec = {"M": 154, "K": 2048, "N": n, "launch_us": round(us, 2), "algorithmic_bytes": algo,
+               "hbm_gbs": round(algo / us * 1e-3, 1), "frac_of_8TBs": round(algo / us * 1e-3 / 8000.0, 4),
+               "fp32_equiv_tflops": round(2.0 * 154 * 2048 * n / us * 1e-6, 1),
+               "kernel": l.cascmm_variant_name(l.cascmm_select_variant(154, n, 2048, 2048, n, n, 0, 0, 2, 0)).decode()}
+        if check:
+            exp = oc.fp64_matmul(x_cpu, w_cpu)
+            ek, eo = oc.error_metrics(res.cpu(), exp), oc.error_metrics(oc.cascade_matmul_ref(x_cpu, w_cpu), exp)
+            if not (ek["rel_fro"] <= 1.25 * eo["rel_fro"] and ek["max_abs"] <= 1.25 * eo["max_abs"]):
+                sys.exit(f"bench.py: kv kernel error {ek} exceeds 1.25x the oracle cascade's {eo}")
+            rec["kernel_rel_fro"], rec["oracle_rel_fro"] = ek["rel_fro"], eo["rel_fro"]
+        out["gemms"].append(rec)
+        total_bytes += algo
+        total_us += us
+    out["hbm_gbs"] = round(total_bytes / total_us * 1e-3, 1)
+    out["us_both"] = round(total_us, 2)
+    return out
+
+
+def bench_unet(dev, cascades=(("bf16", 2), ("fp8", 3)), latents=(("full latent", None), ("half-latent share", 64)), forward=True):
+    """cfg5: the routed layers of one UNet step.  The module tree is built on the GPU with random
+    weights and patched through the config switch; one forward pass records every routed call; those
+    calls are then replayed in call order on resident inputs from ONE HIP graph, so the figure is the
+    Linear / 1x1-convolution path alone (the convolutions, normalisations and attention of the
+    surrounding model are not part of it; the time of a whole eager forward pass is given beside it)."""
+    import torch
+    from basedxl_amd.unet import BasedXLUnet
+    from basedxl_amd.unet_skeleton import SDXLUNetSkeleton, distinct_shapes, routed_calls, synthetic_inputs
+    from basedxl_amd.utils import BasedXLConfig
+
+    rows = []
+    for lowp, terms in cascades:
+        model = SDXLUNetSkeleton(device=dev, seed=SEED)
+        unet = BasedXLUnet(model, BasedXLConfig(fp16_acc_matmul=True, lowp=lowp, terms=terms))
+        for label, latent_rows in latents:
+            inp = synthetic_inputs(model, latent=128, latent_rows=latent_rows, seed=SEED, device=dev)
+            calls = routed_calls(unet, *inp)
+            shapes = distinct_shapes(calls)
+            gen = torch.Generator(device=dev).manual_seed(SEED)
+            xs = {k: torch.randn(c["input_shape"], device=dev, generator=gen) for k, c in shapes.items()}
+            plan = [(c["module"], xs[(type(c["module"]).__name__, c["M"], c["K"], c["N"])]) for c in calls]
+
+            def path():
+                for mod, x in plan:
+                    mod(x)
+
+            with torch.no_grad():
+                us = _graph_time_us(path, reps=1, replays=3, spin_s=0.3)
+                fwd_ms = None
+                if forward:
+                    unet(*inp)
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(2):
+                        unet(*inp)
+                    torch.cuda.synchronize()
+                    fwd_ms = (time.perf_counter() - t0) * 1e3 / 2
+            flops = sum(2.0 * c["M"] * c["K"] * c["N"] for c in calls)
+            rows.append({"cascade": f"{lowp}x{terms} tri", "latent": label, "routed_calls": len(calls), "distinct_shapes": len(shapes),
+                         "gflop_fp32_equiv": round(flops * 1e-9, 1), "linear_path_ms_per_step": round(us * 1e-3, 3),
+                         "fp32_equiv_tflops": round(flops / us * 1e-6, 1),
+                         "whole_forward_ms_eager": None if fwd_ms is None else round(fwd_ms, 1)})
+            del plan, xs
+        del unet, model
+        torch.cuda.empty_cache()
+    return {"workload": "cfg5: every nn.Linear and 1x1 convolution of one SDXL UNet denoising step (latent 2x4x128x128, text "
+                        "context 2x77x2048, weights ~N(0,0.02)) through the patched module tree (fused to_k/to_v, bias in the "
+                        "store, fp8 activation scale found in every call, weight scales kept); one HIP graph of all routed calls",
+            "configs": rows}
+
+
+def bench_eager_launch(dev):
+    """Host cost of the eager path the reference runs (no graph): back-to-back eager calls of one
+    cfg2-sized GEMM (16 us of GPU work), wall time per call."""
+    import torch
+    from basedxl_amd import cascaded_lowp_matmul
+
+    g = torch.Generator(device=dev).manual_seed(SEED)
+    x = torch.randn(4096, 640, device=dev, generator=g)
+    w = torch.randn(640, 640, device=dev, generator=g) * 0.02
+    res = torch.empty(4096, 640, device=dev)
+    for _ in range(50):
+        cascaded_lowp_matmul(x, w, out=res)
+    torch.cuda.synchronize()
+    n = 2000
+    t0 = time.perf_counter()
+    for _ in range(n):
+        cascaded_lowp_matmul(x, w, out=res)
+    t_issue = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    t_all = time.perf_counter() - t0
+    us_graph = _graph_time_us(lambda: cascaded_lowp_matmul(x, w, out=res), reps=20)
+    return {"gemm": "4096x640x640 bf16x2", "eager_us_per_call_wall": round(t_all / n * 1e6, 2),
+            "host_issue_us_per_call": round(t_issue / n * 1e6, 2), "graph_replay_us_per_call": round(us_graph, 2)}
 
 
 def main():
@@ -129,9 +281,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["ffn", "attn"], default="ffn",
+    ap.add_argument("--workload", choices=["ffn", "attn", "kv", "unet"], default="ffn",
                     help="ffn: the two GEMMs of the 32x32-stage GEGLU feed-forward block (the shape the metric is quoted on); "
-                         "attn: the four 64x64-stage self-attention projections of one GPU's patch share")
+                         "attn: the four 64x64-stage self-attention projections of one GPU's patch share; kv: the skinny "
+                         "cross-attention K/V projections (GB/s); unet: the Linear path of one whole UNet step")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="ffn only: leave the kv / unet / eager-launch figures out of the line (they add about a minute)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch every GEMM from Python instead of replaying a HIP graph")
     ap.add_argument("--group", choices=["qkv+o", "all", "none"], default="qkv+o",
@@ -158,6 +313,27 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
+    if args.workload in ("kv", "unet"):
+        base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+                "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+        if args.workload == "kv":
+            kv = bench_kv(dev)
+            worst = min(kv["gemms"], key=lambda r: r["hbm_gbs"])
+            print(json.dumps(dict(base, metric="achieved HBM GB/s over algorithmic bytes at the cross-attention K/V shapes",
+                                  value=kv["hbm_gbs"], unit="GB/s", ms_per_step=round(kv["us_both"] * 1e-3, 5),
+                                  config={"workload": kv["workload"], "launch": "hip graph replay (20 launches per graph)"},
+                                  roofline={"bound": "hbm", "kernel": worst["kernel"], "achieved": worst["hbm_gbs"], "peak": 8000.0,
+                                            "unit": "GB/s", "frac": worst["frac_of_8TBs"], "traffic": KV_TRAFFIC_BYTES.get(worst["N"]),
+                                            "launch_us": worst["launch_us"], "algorithmic_bytes_per_launch": worst["algorithmic_bytes"]},
+                                  gemms=kv["gemms"])))
+        else:
+            un = bench_unet(dev)
+            head = un["configs"][0]
+            print(json.dumps(dict(base, metric="fp32-equiv TFLOP/s of the Linear / 1x1-convolution path of one SDXL UNet step",
+                                  value=head["fp32_equiv_tflops"], unit="TFLOP/s", ms_per_step=head["linear_path_ms_per_step"],
+                                  config={"workload": un["workload"], "headline": head["cascade"] + ", " + head["latent"]},
+                                  configs=un["configs"])))
+        return
     desc, acts, wts, launches = workload(args.workload, args.group)
     cpu_in, (a_dev, w_dev) = make_inputs(acts, wts, dev)
 
@@ -385,6 +561,10 @@ def main():
         other["error"] = {"checked_gemm": chk.label, "kernel_rel_fro": e3["rel_fro"], "oracle_rel_fro": e3o["rel_fro"],
                           "kernel_max_abs": e3["max_abs"], "oracle_max_abs": e3o["max_abs"]}
         result["other_cascades"] = [other]
+    if args.workload == "ffn" and not args.no_graph and not args.no_other_workloads:
+        del sets, a_dev, w_dev
+        torch.cuda.empty_cache()
+        result["other_workloads"] = {"kv": bench_kv(dev), "unet": bench_unet(dev), "eager_launch": bench_eager_launch(dev)}
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cpu_in, launches)
     print(json.dumps(result))
