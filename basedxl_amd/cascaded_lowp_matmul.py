@@ -224,7 +224,7 @@ class PreparedWeight:
                 self._kernel_known = {}
             st = -1
             if dtype in _DTYPES and products in _lib.PROD_BY_NAME:
-                st = _lib.lib().cascmm_select_variant_prepared(1, 256, self.N, self.K, self.K, self.out_features, _DTYPES[dtype],
+                st = _lib.lib().cascmm_select_variant_prepared(1, 256, self.N, self.K, self.K, self.N, _DTYPES[dtype],
                                                                self.fmt, self.terms, _lib.PROD_BY_NAME[products])
             hit = self._kernel_known[key] = st >= 0
         return hit
