@@ -588,7 +588,60 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
 
 using namespace cascmm;
 
+// Built-in scratch of cascmm_gemm_noalloc: the K-split partial results that cascmm_gemm keeps in the
+// caller's workspace.  One copy per GPU the library runs on, held until the process ends.  In host
+// code the array's name is only a handle for hipGetSymbolAddress; the device address it returns
+// (per device) is what kernels and copies are given.
+static __device__ __align__(256) unsigned char scratch[CASCMM_NOALLOC_SCRATCH_BYTES];
+
+static int noalloc_scratch(void** out) {
+  static std::mutex mu;
+  static void* ptr_of_device[kMaxDevices] = {nullptr};
+  const int d = device_index();
+  if (d < 0) return CASCMM_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr_of_device[d]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return CASCMM_ERR_LAUNCH;
+    ptr_of_device[d] = p;
+  }
+  *out = ptr_of_device[d];
+  return CASCMM_OK;
+}
+
 extern "C" {
+
+int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt, int terms, int products,
+                        const int32_t* tensor_exps, void* stream) {
+  const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  if (M == 0 || N == 0 || K == 0) return cascmm_gemm(A, B, C, bias, M, N, K, lda, ldb, ldc, dtype, fmt, terms, products,
+                                                     tensor_exps, nullptr, 0, stream);
+  // the scratch that the kernel cascmm_gemm would pick with an unlimited workspace needs for this problem
+  size_t need = 0;
+  const void* const a1[1] = {A};
+  const void* const b1[1] = {B};
+  if (onthefly_prepare_ok(q, 1, a1, b1, (void*)16, (size_t)-1)) {
+    need = (size_t)prepared_bytes(K, N, fmt, 1);            // 16-bit tensors: B re-laid as operand slots
+  } else if (A && B) {
+    int splits = 1;
+    const int v = select_variant(q, fast_ok(q, A, B), 1, (size_t)-1, &splits);
+    if (v < 0) return v;
+    const VariantDesc& d = table()[v];
+    if (d.kind == KIND_SPLITK) need = skinny_workspace_bytes(M, N, K, d.BM, d.BN, d.BK);
+    else if (splits > 1) need = (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
+  }
+  if (need > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) return CASCMM_ERR_SCRATCH_LIMIT;
+  void* ws = nullptr;
+  if (need > 0) {
+    const int ss = noalloc_scratch(&ws);
+    if (ss != CASCMM_OK) return ss;
+  }
+  // (nothing in the scratch has to start at zero: a launch reads back only the partial results it wrote)
+  return gemm_impl(1, &A, &B, &C, bias ? &bias : nullptr, q, tensor_exps, ws, need, (hipStream_t)stream, -1);
+}
 
 int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K,
                         int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt, int terms, int products,
@@ -807,6 +860,7 @@ const char* cascmm_strerror(int status) {
     case CASCMM_ERR_LAUNCH: return "HIP launch failed";
     case CASCMM_ERR_BAD_VARIANT: return "kernel variant unknown or unable to run this problem";
     case CASCMM_ERR_TOO_LARGE: return "dimension too large";
+    case CASCMM_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the library's built-in buffer holds (use cascmm_gemm with a workspace)";
     default: return "unknown status";
   }
 }

@@ -55,7 +55,8 @@ enum cascmm_status {
   CASCMM_ERR_ALIGNMENT = -6,     /* pointer not aligned to its element size */
   CASCMM_ERR_LAUNCH = -7,        /* the HIP runtime refused the launch */
   CASCMM_ERR_BAD_VARIANT = -8,   /* forced kernel variant unknown or unable to run this problem */
-  CASCMM_ERR_TOO_LARGE = -9      /* a dimension exceeds 2^31 - 1 or a product overflows */
+  CASCMM_ERR_TOO_LARGE = -9,     /* a dimension exceeds 2^31 - 1 or a product overflows */
+  CASCMM_ERR_SCRATCH_LIMIT = -10 /* cascmm_gemm_noalloc: the problem needs more than CASCMM_NOALLOC_SCRATCH_BYTES */
 };
 
 /*
@@ -93,6 +94,24 @@ int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,
                         int dtype, int fmt, int terms, int products,
                         const int32_t* tensor_exps,
                         void* workspace, size_t workspace_bytes, void* stream, int variant);
+
+/*
+ * cascmm_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments
+ * and results as cascmm_gemm called with a workspace of cascmm_workspace_bytes(...) bytes, but the
+ * K-split partial results live in a buffer built into the library (CASCMM_NOALLOC_SCRATCH_BYTES of
+ * device memory per GPU, held until the process ends); the call allocates and frees nothing.
+ * A problem for which the kernel cascmm_gemm would pick (given an unlimited workspace) needs more
+ * partial results than that returns CASCMM_ERR_SCRATCH_LIMIT (nothing is launched).  All calls on one GPU share the buffer: calls that may overlap in time on
+ * one GPU (different streams, or graphs replayed concurrently) race on it and must be ordered by the
+ * caller.  Nothing in the buffer needs initialisation between calls.
+ */
+#define CASCMM_NOALLOC_SCRATCH_BYTES (8u << 20)
+int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
+                        int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc,
+                        int dtype, int fmt, int terms, int products,
+                        const int32_t* tensor_exps, void* stream);
 
 /* `count` (1..8) independent GEMMs of one shape, layout and cascade in ONE launch: problem i
  * computes C[i] = A[i] . B[i] (+ bias[i]); A, B, C, bias are HOST arrays of device pointers
