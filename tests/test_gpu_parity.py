@@ -756,10 +756,23 @@ def test_unet_shape_harness_and_error_script_run(gpu_device, capsys):
     for prepared in (False, True):
         rows = unet_shapes.time_shapes(shapes, "bf16", 2, prepared=prepared, iters=2)
         assert len(rows) == 3 and all(r["launch_us"] > 0 for r in rows)
+    # the script's metrics against the oracle's (the pinned ones) on the same tensors, all five fields
     a = torch.randn(96, 128, device="cuda:0")
     b = torch.randn(128, 64, device="cuda:0")
-    m = measure_error.metrics(cascaded_lowp_matmul(a, b), a.double() @ b.double())
-    assert 1e-7 < m["rel_fro"] < 1e-4 and len(m["quantiles"]) == 5
+    out, exact = cascaded_lowp_matmul(a, b), a.double() @ b.double()
+    m = measure_error.metrics(out, exact)
+    o = oc.error_metrics(out.cpu(), exact.cpu())
+    assert m["L1"] == pytest.approx(o["l1"], rel=1e-9) and m["MSE"] == pytest.approx(o["mse"], rel=1e-9)
+    assert m["Max"] == pytest.approx(o["max_abs"], rel=1e-12) and m["rel_fro"] == pytest.approx(o["rel_fro"], rel=1e-9)
+    assert m["quantiles"] == pytest.approx(o["rel_quantiles"], rel=1e-9)          # (6144 elements: no sub-sampling)
+    assert 1e-7 < m["rel_fro"] < 1e-4
+    # and the script itself, on the SDXL shapes with the headline cascade
+    capsys.readouterr()
+    measure_error.main(["--shapes", "sdxl", "--cascades", "bf16x2"])
+    text = capsys.readouterr().out
+    assert text.count("bf16x2 tri") == 2 * 4 and "torch fp32 matmul" in text and "Median rel" in text
+    rows = [ln.split(" | ") for ln in text.splitlines() if ln.startswith(("4096 | ", "2048 | ", "154 | ")) and "bf16x2" in ln]
+    assert len(rows) == 4 and all(3e-6 < float(r[7]) < 6e-6 for r in rows)    # rel. Frobenius of bf16 x 2 on every shape
 
 
 def test_wrapper_shapes_like_the_reference(gpu_device):

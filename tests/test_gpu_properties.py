@@ -173,8 +173,10 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
     reduction pass, skinny split-K kernel, grouped launch, 16-bit tensors (weights re-laid into the
     workspace), prepared and gated weights, fp8 with the scale found on the device -- is captured
     once and replayed with fresh operand values; each replay must return the bits of the eager call
-    on the same values (nothing host-side, no memset, no allocation inside the captured region
-    after the warm-up)."""
+    on the same values.  The library records only kernels; the Python operator allocates its results
+    (and the small fp8 exponent tensors) from the graph's pool during the capture, but no workspace:
+    the eager warm-up has sized the per-device workspace that captured launches use, which the test
+    checks by comparing the memory allocated during the capture with the size of the results."""
     from basedxl_amd import cascaded_lowp_matmul_grouped
 
     dev = "cuda:0"
@@ -207,9 +209,21 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
     with torch.cuda.stream(side):
         run()                                        # and on a side stream, as torch's capture recipe asks
     torch.cuda.current_stream().wait_stream(side)
+    from basedxl_amd.cascaded_lowp_matmul import _workspaces
+    ws_before = {k: v.data_ptr() for k, v in _workspaces.items()}
     graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
     with torch.cuda.graph(graph):
         outs = run()
+    grown = torch.cuda.memory_allocated() - before
+    assert {k: v.data_ptr() for k, v in _workspaces.items()} == ws_before        # no workspace was created or replaced
+    # what the capture allocated: the eight results plus the grouped launches' other results and the
+    # two-int exponent tensor, each rounded up to the allocator's 512-byte granule -- far below the
+    # 21 MB K-split workspace a capture-time allocation would add
+    results = sum(o.numel() * o.element_size() for o in outs)
+    others = 2 * x["tile"].shape[0] * 640 * 4 + x["h"].shape[0] * 640 * 2
+    assert results <= grown <= results + others + 64 * 1024, (grown, results, others)
     for rep in range(3):
         for k in x:                                  # new values in the captured buffers
             x[k].copy_(rn(*x[k].shape, dtype=x[k].dtype) * (1.0 + rep))

@@ -163,7 +163,19 @@ def test_metrics_on_a_known_case():
     assert m["l1"] == pytest.approx(0.375)
     assert m["mse"] == pytest.approx((0.25 + 1.0) / 4)
     assert m["rel_fro"] == pytest.approx(np.sqrt(1.25) / np.sqrt(21.0))
-    assert len(m["rel_quantiles"]) == 5
+    # relative errors |d| / (|e| + 1e-6) of the four elements: 0.5 / 1.000001, 0, 0, 1 / 4.000001;
+    # numpy's linear interpolation on the sorted values [0, 0, 0.25, 0.5] at 1 / 20 / 50 / 80 / 99 %
+    r = sorted([0.5 / 1.000001, 0.0, 0.0, 1.0 / 4.000001])
+    def interp(q):
+        pos = q * 3
+        lo = int(pos)
+        return r[lo] + (r[min(lo + 1, 3)] - r[lo]) * (pos - lo)
+    assert m["rel_quantiles"] == pytest.approx([interp(q) for q in (0.01, 0.2, 0.5, 0.8, 0.99)], rel=1e-12, abs=1e-15)
+    assert m["rel_quantiles"][2] == pytest.approx(0.125, rel=1e-5) and m["rel_quantiles"][0] == 0.0
+    # a larger known case: out = 1.01 x expected everywhere -> every relative error is 0.01 / (1 + 1e-6 / |e|)
+    e = torch.arange(1, 1001, dtype=torch.float64).reshape(10, 100)
+    q = oc.error_metrics((e * 1.01).float(), e)["rel_quantiles"]
+    assert all(abs(v - 0.01) < 1e-6 for v in q) and q == sorted(q)
     assert oc.fp32_equiv_tflops(1024, 1024, 1024, 1e-3) == pytest.approx(2.147483648)
 
 
