@@ -84,6 +84,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full || v.bpre != q.bpre) return false;
   if (v.fast && (!fast || q.K % v.BK != 0)) return false;
   if (v.kind == KIND_SPLITK && (q.M > 5 * v.BM || q.K < 4 * v.BK)) return false;  // skinny: few row tiles, deep K
+  if (v.kind == KIND_W512 && (q.M % v.BM != 0 || q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX)) return false;
   if (q.glu && !v.glu) return false;
   return true;
 }
@@ -107,6 +108,7 @@ static const TunedCost kTuned[] = {
     {"t64x160x64_w2x1x2_d2_p8_bf16x2_tri", 1.064, 4.69, 0.90, 0.80},
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.224, 6.84, 0.80, 0.70},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri", 3.250, 5.00, 0.70, 0.50},
+    {"t256x320x32_w512_bf16x2_tri", 5.65, 16.0, 1.00, 1.00},
     // three fp16 / bf16 terms
     {"t128x128x32_w4x2x1_d2_fp16x3_tri", 3.107, 7.22, 0.90, 0.80},
     {"t64x64x32_w2x2x1_d3_fp16x3_tri", 1.088, 2.27, 1.00, 1.00},

@@ -4,10 +4,12 @@
 #include <mutex>
 
 #include "cascmm_bdirect_kernel.h"
+#include "cascmm_w512_kernel.h"
 
 namespace cascmm {
 
-enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1 };
+// KIND_W512: the large-tile kernel (whole 256 x 320 tiles only, one problem per launch)
+enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2 };
 constexpr int kNumCUs = 256;  // MI355X: what the cost model's constants were measured on
 constexpr int kMaxDevices = 64;
 
@@ -177,6 +179,32 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   }
   return CASCMM_OK;
 }
+
+// the large-tile kernel
+template <int UNUSED>
+int launch_w512(const GroupParams& p, hipStream_t stream) {
+  typedef W512 T;
+  if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
+  if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
+  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
+    return CASCMM_ERR_TOO_LARGE;
+  auto kfn = cascmm_w512_kernel<UNUSED>;
+  static bool lds_set[kMaxDevices] = {false};
+  const int d = device_index();
+  if (d < 0) return CASCMM_ERR_LAUNCH;
+  if (!lds_set[d]) {
+    if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
+    lds_set[d] = true;
+  }
+  const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n);
+  if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
+  return CASCMM_OK;
+}
+
+#define CASCMM_W512_VARIANT(NAME)                                                                                   \
+  {NAME, KIND_W512, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, W512::BM, W512::BN, 32, W512::NT, W512::LDS_BYTES, true, \
+   false, &launch_w512<0>}
 
 // eight producer waves, every B column loaded singly (all producer threads share A and B evenly)
 #define CASCMM_TILE_VARIANT_PS(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)          \

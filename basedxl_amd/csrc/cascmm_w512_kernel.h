@@ -1,0 +1,269 @@
+// Large-tile kernel of the two-term bf16 cascade (gfx950): four waves with 512 registers each.
+//
+// One workgroup = four waves (one per SIMD, 2 x 2) computes a 256 x 320 tile of C; a wave owns
+// 128 x 160 of it, twenty 32 x 32 accumulator blocks: sixteen in the 256 accumulation registers
+// and four in ordinary vector registers.  Against a 64 x 160 wave tile this cuts the LDS bytes read per
+// MFMA by a third and the bytes staged per MFMA by 30 %, and those bytes, not issue slots, are what
+// the chip's power management charges for: with every CU busy the clock settles where the power
+// fits, so fewer bytes moved per MFMA is a higher clock.
+//
+// There are no producer waves (a kernel has one register allocation, so a wave with 512 registers
+// fills its SIMD).  Both operands reach LDS as raw fp32 without passing registers (wave-wide
+// `buffer_load ... lds`, 1 KB each), and every wave splits the values of its own fragments in
+// registers right after reading them:
+//   * A: 256 rows x 16 k per stage; four consecutive lanes fetch the four 16-byte chunks of one row's
+//     64 bytes (whole cache lines), rotated by row / 4 inside the row so that the fragment reads (lane
+//     l: row l%32, chunks 2 (l/32) and 2 (l/32) + 1) spread over all banks;
+//   * B: 16 k rows x 320 columns per stage, 256 consecutive floats per load; lane l of a fragment reads
+//     column l%32 at k = 8 (l/32) .. +7 with eight ds_read_b32 (rows of the odd k-group are rotated by
+//     32 columns, which keeps the two half waves on different banks).
+// Two waves share every row block and every column block, so each value is split twice per
+// workgroup; the split's VALU work issues in the gaps between the wave's own MFMAs, as do the LDS
+// reads and the loads of later stages, and it costs no measurable time there.
+//
+// Stages are 16 k deep (60 MFMAs per wave), four of them in LDS (144 KB).  At the barrier that opens
+// stage s, stage s + 1 has landed as well, so the first fragments of the next stage are read before
+// its barrier and no LDS latency is exposed after it; the loads of stage s + 3 are issued during
+// stage s.  Loads are issued unconditionally (past the last stage the last one is fetched again into
+// a dead buffer): a wave that is alone on its SIMD pays tens of cycles for every branch.
+//
+// The order of everything between two MFMAs is pinned with scheduling fences; the four blocks held
+// in vector registers use the MFMA through inline assembly, because the compiler gives every MFMA it
+// selects an accumulator in the accumulation registers (of which there are sixteen blocks' worth).
+#pragma once
+#include "cascmm_tile_kernel.h"
+
+namespace cascmm {
+
+struct W512 {
+  static constexpr int BM = 256, BN = 320, BK = 16, NS = 4, NT = 256;
+  static constexpr int WTM = 128, WTN = 160, MT = 4, NTL = 5;
+  static constexpr int A_STAGE = BM * BK * 4;       // raw fp32: 64 bytes per row
+  static constexpr int B_STAGE = BK * BN * 4;       // raw fp32
+  static constexpr int STAGE = A_STAGE + B_STAGE;   // 36 KB
+  static constexpr int LDS_BYTES = NS * STAGE;      // 144 KB
+  static constexpr int LOADS = 9;                   // direct loads per wave and stage: 4 of A, 5 of B
+};
+
+typedef __attribute__((address_space(3))) void* w512_lds_ptr;
+
+// MFMA with the accumulator in ordinary vector registers
+__device__ __forceinline__ void w512_mfma_v(u32x4 a, u32x4 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ f32x16 w512_mfma_a(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Host-checked: M % 256 == 0, N % 320 == 0, K % 32 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
+// aligned, M * lda * 4 and K * ldb * 4 below 2 GiB, C rows addressable with 32-bit byte offsets
+// inside a tile.
+// (a template, so that only the translation unit that lists the variant compiles it)
+template <int UNUSED>
+__global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_w512_kernel(const GroupParams p) {
+  typedef W512 T;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char w512_smem[];
+  unsigned char* smem = w512_smem;
+  const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave >> 1) * T::WTM, wn0 = (wave & 1) * T::WTN;
+  int tm, tn;
+  tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * T::BM, n0 = tn * T::BN;
+  const int ksteps = p.K / T::BK;
+  const int ldb_bytes = (int)p.ldb * 4;
+
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.A[0], 0, 0x7FFFFFFF, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.B[0], 0, 0x7FFFFFFF, 0x00020000);
+  // per wave and stage: 4 loads of A (16 rows x 64 bytes each; LDS position 4 row + pos holds chunk
+  // (pos - row / 4) mod 4 of the row) and 5 loads of B (256 consecutive floats of the stage's [16][320]
+  // area)
+  int a_voff[4], a_lds[4], b_voff[5], b_lds[5];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int inst = wave * 4 + j;
+    const int row = inst * 16 + (lane >> 2);
+    const int chunk = ((lane & 3) - (row >> 2)) & 3;
+    a_lds[j] = inst * 1024;
+    a_voff[j] = (int)(((int64_t)(m0 + row) * p.lda + chunk * 4) * 4);
+  }
+#pragma unroll
+  for (int j = 0; j < 5; ++j) {
+    const int inst = wave * 5 + j;
+    const int f = inst * 256 + lane * 4;
+    const int k = f / T::BN, pos = f % T::BN;
+    int n = pos - 32 * ((k >> 3) & 1);
+    n = n < 0 ? n + T::BN : n;
+    b_lds[j] = T::A_STAGE + inst * 1024;
+    b_voff[j] = k * ldb_bytes + (n0 + n) * 4;
+  }
+  auto issue1 = [&](int step_, int j) {
+    const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
+    const int st = step_ % T::NS;
+    if (j < 4)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (w512_lds_ptr)(smem + st * T::STAGE + a_lds[j]), 16, a_voff[j], step * T::BK * 4, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (w512_lds_ptr)(smem + st * T::STAGE + b_lds[j - 4]), 16, b_voff[j - 4],
+                                               step * T::BK * ldb_bytes, 0, 0);
+  };
+
+  // fragment addresses (bytes inside a stage)
+  const int a_row = wm0 + l31;                          // + mi * 32 rows = mi * 2048 bytes (same rotation: 32 / 4 = 8)
+  const int a_frag0 = a_row * 64 + ((2 * g + (a_row >> 2)) & 3) * 16;
+  const int a_frag1 = a_row * 64 + ((2 * g + 1 + (a_row >> 2)) & 3) * 16;
+  int b_frag[T::NTL];
+#pragma unroll
+  for (int ni = 0; ni < T::NTL; ++ni) {
+    int pos = wn0 + ni * 32 + l31 + 32 * g;
+    pos = pos >= T::BN ? pos - T::BN : pos;
+    b_frag[ni] = T::A_STAGE + (8 * g * T::BN + pos) * 4;   // + e * BN * 4
+  }
+
+  f32x16 acc[T::MT][T::NTL];
+#pragma unroll
+  for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
+
+  // ---- software pipeline ---------------------------------------------------------------------
+  // Blocks are numbered t = stage * 5 + ni.  While the 12 MFMAs of block t issue, the raw B values of
+  // block t + 2 are read from LDS and those of block t + 1 (read one block earlier) are split; the A
+  // values of row block ni of the next stage are read and split during block ni (0 .. 3), two loads of
+  // a later stage are issued per block.
+#define W512_FENCE() __builtin_amdgcn_sched_barrier(0)
+  u32x4 Af[2][2][T::MT];   // [buffer][hi / lo][mi]
+  float R[2][8];           // raw B values of two blocks in flight
+  float RA[8];             // raw A values of one row block of the next stage
+  u32x4 H[2], L[2];        // split B of the current / next block
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef float f32x2v __attribute__((ext_vector_type(2)));
+
+  auto read_raw = [&](float (&dst)[8], const unsigned char* stp, int ni, int e0, int e1) {
+#pragma unroll
+    for (int e = e0; e < e1; ++e) dst[e] = *(const float*)(stp + b_frag[ni] + e * T::BN * 4);
+  };
+  // the split of one pair of consecutive k in two halves of three VALU instructions each
+  auto split_1 = [&](float (&x)[8], u32x4& hi, int e) {
+    const f32x2v v = {x[2 * e], x[2 * e + 1]};
+    const unsigned hp = __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+    hi[e] = hp;
+    x[2 * e] = x[2 * e] - __builtin_bit_cast(float, hp << 16);
+  };
+  auto split_2 = [&](float (&x)[8], const u32x4& hi, u32x4& lo, int e) {
+    const f32x2v r = {x[2 * e], x[2 * e + 1] - __builtin_bit_cast(float, hi[e] & 0xFFFF0000u)};
+    lo[e] = __builtin_bit_cast(unsigned, __builtin_convertvector(r, bf16x2));
+  };
+
+#pragma unroll
+  for (int s = 0; s < T::NS - 1; ++s)
+#pragma unroll
+    for (int j = 0; j < T::LOADS; ++j) issue1(s, j);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (18 & 0xF) | ((18 >> 4) << 14));   // vmcnt(18): stage 0 has landed
+  __builtin_amdgcn_s_barrier();
+  {
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi) {
+      const f32x4 x0 = *(const f32x4*)(smem + a_frag0 + mi * 2048), x1 = *(const f32x4*)(smem + a_frag1 + mi * 2048);
+      float x[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        split_1(x, Af[0][0][mi], e);
+        split_2(x, Af[0][0][mi], Af[0][1][mi], e);
+      }
+    }
+    read_raw(R[0], smem, 0, 0, 8);
+    read_raw(R[1], smem, 1, 0, 8);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      split_1(R[0], H[0], e);
+      split_2(R[0], H[0], L[0], e);
+    }
+  }
+
+  for (int s = 0; s < ksteps; s += 2) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      // top of stage s + j: the own loads of stage s + j + 1 have landed, then everybody's
+      __builtin_amdgcn_s_waitcnt(0x0F70 | T::LOADS);                     // vmcnt(9)
+      __builtin_amdgcn_s_barrier();
+      const unsigned char* st0 = smem + ((s + j) % T::NS) * T::STAGE;       // this stage
+      const unsigned char* st1 = smem + ((s + j + 1) % T::NS) * T::STAGE;   // the next one
+#pragma unroll
+      for (int ni = 0; ni < T::NTL; ++ni) {
+        const int t = j * T::NTL + ni;        // block number inside the trip: its parity is static
+        const int cur = t & 1, nxt = cur ^ 1;
+        const int n2 = (ni + 2) % T::NTL;
+        const unsigned char* st2 = (ni + 2 < T::NTL) ? st0 : st1;
+        u32x4(&Ah)[T::MT] = Af[j][0];
+        u32x4(&Al)[T::MT] = Af[j][1];
+        // products lo.hi, hi.lo, hi.hi of the four row blocks: smallest first, consecutive MFMAs on
+        // different accumulators
+        auto mm = [&](int idx) {
+          const int prod = idx >> 2, mi = idx & 3;
+          const u32x4 a = prod == 0 ? Al[mi] : Ah[mi];
+          const u32x4 b = prod == 1 ? L[cur] : H[cur];
+          if (ni < 4) acc[mi][ni] = w512_mfma_a(a, b, acc[mi][ni]);
+          else w512_mfma_v(a, b, acc[mi][ni]);
+        };
+        auto dl = [&](int k) {   // two load slots per block: 10 per stage, 9 used
+          const int slot = ni * 2 + k;
+          if (slot < T::LOADS) issue1(s + j + T::NS - 1, slot);
+        };
+        mm(0); W512_FENCE();
+        read_raw(R[cur], st2, n2, 0, 4); W512_FENCE();
+        mm(1); W512_FENCE();
+        read_raw(R[cur], st2, n2, 4, 8); dl(0); W512_FENCE();
+        mm(2); W512_FENCE();
+        if (ni < 4) {   // row block ni of the next stage
+          const f32x4 x0 = *(const f32x4*)(st1 + a_frag0 + ni * 2048), x1 = *(const f32x4*)(st1 + a_frag1 + ni * 2048);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            RA[e] = x0[e];
+            RA[4 + e] = x1[e];
+          }
+        }
+        W512_FENCE();
+        mm(3); W512_FENCE();
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          split_1(R[nxt], H[nxt], e);
+          if (ni < 4) split_1(RA, Af[j ^ 1][0][ni], e);
+          W512_FENCE();
+          mm(4 + 2 * e); W512_FENCE();
+          split_2(R[nxt], H[nxt], L[nxt], e);
+          if (ni < 4) split_2(RA, Af[j ^ 1][0][ni], Af[j ^ 1][1][ni], e);
+          if (e == 3) dl(1);
+          W512_FENCE();
+          mm(5 + 2 * e); W512_FENCE();
+        }
+      }
+    }
+  }
+#undef W512_FENCE
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // the redundant loads of the last stages land before LDS is given up
+  // the MFMAs written as assembly are invisible to the compiler's hazard handling: their passes
+  // must have drained before the accumulators are read
+  asm volatile("s_nop 7\n s_nop 7\n s_nop 7" ::: "memory");
+
+  // ---- epilogue: of every block a lane holds column l31, rows 8 q + 4 g + e -----------------------
+  float* C = (float*)p.C[0] + (int64_t)(m0 + wm0) * p.ldc + n0 + wn0;
+  const float* bias = (const float*)p.bias[0];
+  const i32x4 rc = make_rsrc(C, 0x7FFFFFFF);
+  const int ldc_bytes = (int)p.ldc * 4;
+#pragma unroll
+  for (int ni = 0; ni < T::NTL; ++ni) {
+    const float bv = bias ? bias[n0 + wn0 + ni * 32 + l31] : 0.f;
+    const int voff = g * 4 * ldc_bytes + (ni * 32 + l31) * 4;
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          llvm_raw_buffer_store_f32(acc[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+  }
+}
+
+}  // namespace cascmm

@@ -88,7 +88,7 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
     l = _lib.lib()
     names = _lib.variant_names()
     pick = lambda M, K, N: names[l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0) & 0xFFFF]
-    assert pick(2048, 1280, 10240) == "t256x160x32_w4x1x1_d2_bf16x2_tri"          # cfg3, first GEMM
+    assert pick(2048, 1280, 10240) == "t256x320x32_w512_bf16x2_tri"               # cfg3, first GEMM
     assert pick(154, 2048, 1280).startswith("skinny") and pick(154, 2048, 640).startswith("skinny")   # cfg4
     grouped = names[l.cascmm_select_variant_grouped(3, 4096, 640, 640, 640, 640, 640, 0, 0, 2, 0) & 0xFFFF]
     assert grouped == "t256x128x32_w4x1x1_d2_bf16x2_tri"                           # cfg2, to_q / to_k / to_v

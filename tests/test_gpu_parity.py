@@ -152,7 +152,7 @@ def _int_case(M, K, N, hi, seed):
     return a, b, a @ b
 
 
-INT_SHAPES = [(16, 32, 16), (17, 33, 19), (154, 64, 48), (1, 7, 1), (130, 40, 81), (256, 192, 160), (300, 128, 200),
+INT_SHAPES = [(256, 64, 320), (512, 96, 640), (16, 32, 16), (17, 33, 19), (154, 64, 48), (1, 7, 1), (130, 40, 81), (256, 192, 160), (300, 128, 200),
               (257, 64, 161), (257, 64, 164), (96, 128, 384), (154, 512, 256), (30, 256, 132), (64, 1024, 128),
               (160, 320, 1284)]
 
@@ -184,6 +184,8 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
             continue  # fast variants need K % BK == 0 and N % 4 == 0 (rejected by the library otherwise)
         if name.startswith("skinny") and (M > 5 * int(name.split("x")[0][6:]) or K < 4 * bk):
             continue  # split-K variants take at most five row tiles and at least four K steps
+        if "_w512_" in name and (M % 256 != 0 or N % 320 != 0 or K % 32 != 0):
+            continue  # the large-tile kernel takes whole 256 x 320 tiles and K in steps of 32
         _say("int-exact", shape, name)
         out = cascaded_lowp_matmul(at7 if small else at, bt7 if small else bt, lowp=fmt, terms=terms, products=products,
                                    variant=vi)
