@@ -300,9 +300,10 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
     if w0.glu:
         st = _lib.lib().cascmm_gemm_prepared_glu(*common, stream, variant)
     else:
-        # room for the partial results of a K split (single fp32 problems with few tiles)
+        # room for the partial results of a K split (single fp32 problems with few tiles) or for the
+        # operand slots of the activations (three fp8 terms)
         ws = None
-        if n == 1 and adt == torch.float32:
+        if adt == torch.float32 and (n == 1 or w0.fmt == _lib.FMT_FP8):
             need = _workspace_bytes(M, N, K, _DTYPES[adt], w0.fmt, w0.terms, _lib.PROD_BY_NAME[products])
             ws = _workspace(dev, stream, need)
         st = _lib.lib().cascmm_gemm_prepared(*common, ws.data_ptr() if ws is not None else None,

@@ -48,8 +48,15 @@ struct Problem {
   bool glu = false;   // gated epilogue: B prepared by cascmm_prepare_weight_glu, C has N / 2 columns
 };
 
+// Three fp8 terms with K a multiple of 64 are prepared for the fp8-rate kernel: [term][K/16][N] slots
+// of 16 k each (the gated layout keeps the older form, whose kernels have the gated store)
+static bool prepared_as_k16_slots(int64_t K, int fmt, int terms, bool glu) {
+  return fmt == CASCMM_FMT_FP8 && terms == 3 && K > 0 && K % F8K64::BK == 0 && !glu;
+}
+
 // bytes of a prepared weight: planes x ceil(K/8) x N operand slots of 16 bytes
-static int64_t prepared_bytes(int64_t K, int64_t N, int fmt, int terms) {
+static int64_t prepared_bytes(int64_t K, int64_t N, int fmt, int terms, bool glu = false) {
+  if (prepared_as_k16_slots(K, fmt, terms, glu)) return f8k64_slot_bytes(N, K);
   const int planes = fmt == CASCMM_FMT_FP8 ? (terms + 1) / 2 : terms;
   return (int64_t)planes * ((K + 7) / 8) * N * 16;
 }
@@ -84,6 +91,10 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   if (v.iodt != q.dtype || v.fmt != q.fmt || v.terms != q.terms || v.full != full || v.bpre != q.bpre) return false;
   if (v.fast && (!fast || q.K % v.BK != 0)) return false;
   if (v.kind == KIND_SPLITK && (q.M > 5 * v.BM || q.K < 4 * v.BK)) return false;  // skinny: few row tiles, deep K
+  if (v.kind == KIND_F8K64 && (q.products != CASCMM_PROD_TRI || q.K % v.BK != 0 || q.K == 0 || q.glu ||
+                               f8k64_slot_bytes(q.M, q.K) > INT32_MAX || f8k64_slot_bytes(q.N, q.K) > INT32_MAX))
+    return false;
+  if (v.bpre && v.kind != KIND_F8K64 && prepared_as_k16_slots(q.K, q.fmt, q.terms, q.glu)) return false;   // other layout
   if (v.kind == KIND_W512 && (q.M % v.BM != 0 || q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX)) return false;
   if (q.glu && !v.glu) return false;
   return true;
@@ -109,6 +120,9 @@ static const TunedCost kTuned[] = {
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.224, 6.84, 0.80, 0.70},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri", 3.250, 5.00, 0.70, 0.50},
     {"t256x320x32_w512_bf16x2_tri", 5.65, 16.0, 1.00, 1.00},
+    // (fixed part: the passes that split the operands)
+    {"t256x160x64_f8k64_fp8x3_tri", 2.6, 22.0, 0.80, 0.60},
+    {"t256x160x64_f8k64_fp8x3_tri_bpre", 2.6, 14.0, 0.80, 0.60},
     // three fp16 / bf16 terms
     {"t128x128x32_w4x2x1_d2_fp16x3_tri", 3.107, 7.22, 0.90, 0.80},
     {"t64x64x32_w2x2x1_d3_fp16x3_tri", 1.088, 2.27, 1.00, 1.00},
@@ -278,6 +292,7 @@ static int select_variant_uncached(const Problem& q, bool fast, int count, size_
     if (t[i].kind == KIND_SPLITK &&
         skinny_workspace_bytes(q.M, q.N, q.K, t[i].BM, t[i].BN, t[i].BK) > ws_bytes)
       continue;
+    if (t[i].kind == KIND_F8K64 && f8k64_workspace_bytes(q.M, q.N, q.K, q.bpre) > ws_bytes) continue;
     int sp = 1;
     const double c = variant_cost(i, q, count, ws_bytes, &sp);
     if (best < 0 || c < best_cost) {
@@ -550,13 +565,24 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
     // prepared weights only have the fast kernels: fp32 A with 16-byte aligned rows, K a multiple
     // of the kernel's K step (checked per variant), and a buffer the 32-bit offsets can span
     if (!fast) return CASCMM_ERR_ALIGNMENT;
-    if (prepared_bytes(q.K, q.N, q.fmt, q.terms) > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+    if (prepared_bytes(q.K, q.N, q.fmt, q.terms, q.glu) > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
   }
 
   const auto& t = table();
   int splits = 1;
   if (variant < 0) {
     variant = select_variant(q, fast, count, workspace ? workspace_bytes : 0, &splits);
+    if (variant < 0 && count > 1) {
+      // no kernel takes these problems in one launch (the fp8-rate kernel runs one at a time): one
+      // launch each, in order on the stream, sharing the workspace
+      for (int i = 0; i < count; ++i) {
+        const void* bi = bias ? bias[i] : nullptr;
+        const int st1 = gemm_impl(1, A + i, B + i, C + i, bias ? &bi : nullptr, q, tensor_exps ? tensor_exps + 2 * i : nullptr,
+                                  workspace, workspace_bytes, stream, -1);
+        if (st1 != CASCMM_OK) return st1;
+      }
+      return CASCMM_OK;
+    }
     if (variant < 0) return variant;
   } else {
     splits = (variant >> 16) > 0 ? (variant >> 16) : 1;   // forced: kernel index | K splits << 16
@@ -566,7 +592,17 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
     if (!variant_matches(t[variant], q, fast)) return CASCMM_ERR_BAD_VARIANT;
   }
   const VariantDesc& v = t[variant];
-  if (count > 1 && !v.grouped) return CASCMM_ERR_BAD_VARIANT;
+  if (count > 1 && !v.grouped) {
+    // a forced kernel that runs one problem per launch: one launch each, in order on the stream
+    if (v.kind == KIND_SPLITK) return CASCMM_ERR_BAD_VARIANT;
+    for (int i = 0; i < count; ++i) {
+      const void* bi = bias ? bias[i] : nullptr;
+      const int st1 = gemm_impl(1, A + i, B + i, C + i, bias ? &bi : nullptr, q, tensor_exps ? tensor_exps + 2 * i : nullptr,
+                                workspace, workspace_bytes, stream, variant | (splits > 1 ? splits << 16 : 0));
+      if (st1 != CASCMM_OK) return st1;
+    }
+    return CASCMM_OK;
+  }
   GroupParams p;
   memset(&p, 0, sizeof(p));
   p.M = (int)q.M; p.N = (int)q.N; p.K = (int)q.K;
@@ -629,10 +665,17 @@ int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
     need = (size_t)prepared_bytes(K, N, fmt, 1);            // 16-bit tensors: B re-laid as operand slots
   } else if (A && B) {
     int splits = 1;
-    const int v = select_variant(q, fast_ok(q, A, B), 1, (size_t)-1, &splits);
+    int v = select_variant(q, fast_ok(q, A, B), 1, (size_t)-1, &splits);
     if (v < 0) return v;
+    if (table()[v].kind == KIND_F8K64 && f8k64_workspace_bytes(M, N, K, false) > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) {
+      // the fp8-rate kernel is a choice, not a need: without room for its operand slots the choice is
+      // made among the kernels that split inside the GEMM
+      v = select_variant(q, fast_ok(q, A, B), 1, (size_t)CASCMM_NOALLOC_SCRATCH_BYTES, &splits);
+      if (v < 0) return v;
+    }
     const VariantDesc& d = table()[v];
     if (d.kind == KIND_SPLITK) need = skinny_workspace_bytes(M, N, K, d.BM, d.BN, d.BK);
+    else if (d.kind == KIND_F8K64) need = f8k64_workspace_bytes(M, N, K, false);
     else if (splits > 1) need = (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
   }
   if (need > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) return CASCMM_ERR_SCRATCH_LIMIT;
@@ -673,7 +716,8 @@ int cascmm_gemm(const void* A, const void* B, void* C, const void* bias, int64_t
 size_t cascmm_prepared_bytes(int64_t K, int64_t N, int fmt, int terms) {
   if (K < 0 || N < 0 || terms < 1 || terms > 3) return 0;
   if (fmt != CASCMM_FMT_BF16 && fmt != CASCMM_FMT_FP16 && fmt != CASCMM_FMT_FP8) return 0;
-  return (size_t)prepared_bytes(K, N, fmt, terms);
+  // (three fp8 terms have two layouts, for the plain and the gated preparation: room for either)
+  return (size_t)std::max(prepared_bytes(K, N, fmt, terms, false), prepared_bytes(K, N, fmt, terms, true));
 }
 
 static int prepare_weight_impl(const void* B, int64_t K, int64_t N, int64_t ldb, int dtype, int fmt, int terms,
@@ -685,8 +729,15 @@ static int prepare_weight_impl(const void* B, int64_t K, int64_t N, int64_t ldb,
   if (K == 0 || N == 0) return CASCMM_OK;
   if (!B || !out) return CASCMM_ERR_NULL_POINTER;
   if (!aligned_to(out, 16)) return CASCMM_ERR_ALIGNMENT;
-  if (out_bytes < (size_t)prepared_bytes(K, N, fmt, terms)) return CASCMM_ERR_WORKSPACE;
+  if (out_bytes < (size_t)prepared_bytes(K, N, fmt, terms, glu != 0)) return CASCMM_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
+  if (prepared_as_k16_slots(K, fmt, terms, glu != 0)) {
+    // the layout of the fp8-rate kernel: [term][K/16][N] slots of 16 k
+    if (dtype != CASCMM_DT_F32) return CASCMM_ERR_BAD_DTYPE;
+    const int64_t units = (K >> 4) * N;
+    return launch_kernel(f8k64_split_cols_kernel<0>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, s, (const float*)B, (int)K,
+                         (int)N, ldb, tensor_exp, (u32x4*)out) == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+  }
   if (dtype == CASCMM_DT_F32) return launch_prepare_fmt<CASCMM_DT_F32>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s, glu);
   if (dtype == CASCMM_DT_F16) return launch_prepare_fmt<CASCMM_DT_F16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s, glu);
   if (dtype == CASCMM_DT_BF16) return launch_prepare_fmt<CASCMM_DT_BF16>(B, (int)K, (int)N, ldb, fmt, terms, tensor_exp, (u32x4*)out, s, glu);
@@ -743,6 +794,12 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
   for (const auto& v : table()) {
     if (v.kind != KIND_SPLITK || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
     const size_t n = skinny_workspace_bytes(M, N, K, v.BM, v.BN, v.BK);
+    need = n > need ? n : need;
+  }
+  // three fp8 terms on the fp8-rate kernel: the operand slots of A and B
+  for (const auto& v : table()) {
+    if (v.kind != KIND_F8K64 || v.bpre || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
+    const size_t n = f8k64_workspace_bytes(M, N, K, false);
     need = n > need ? n : need;
   }
   // 16-bit tensors as one term of their own format: room for B re-laid as operand slots

@@ -1,0 +1,269 @@
+// Three-term fp8 (e4m3) cascade on the fp8-rate MFMA of gfx950, v_mfma_scale_f32_32x32x64_f8f6f4.
+//
+// That instruction multiplies 32 x 64 by 64 x 32 fp8 values in 16 passes (64 cycles, measured): twice
+// the rate of the bf16 and legacy fp8 forms, so the six products of a three-term cascade cost what
+// the three products of the two-term bf16 cascade cost.  A lane supplies 32 consecutive k of its row
+// (column) in eight registers, lanes 0..31 the first half of the 64, lanes 32..63 the second, and one
+// E8M0 scale byte that the hardware applies to those 32 values.  The scales carry the term scaling:
+// term i of either operand is stored as lowp(r_i * 2^(e + 4 i)) and multiplied with scale 2^(-4 i),
+// so all six products of a block land in ONE accumulator with their weights 2^(-4 (i + j)) applied
+// before the addition (measured: a lane's scale applies to exactly its own 32 values; products are
+// added in fp32 with an alignment window of about 15 bits inside groups of neighbouring k and about
+// 18 bits across them, as in the legacy instruction).
+//
+// Both operands are split before the GEMM, by small kernels, into operand slots: 16 bytes = 16
+// consecutive k of one row (column) of one term, [term][K/16][rows].  Activations are split in every
+// call (their tensor scale is found first, by a pass of its own); a weight can be split once
+// (cascmm_prepare_weight writes this layout for three fp8 terms when K is a multiple of 64).  The
+// GEMM then moves nothing through registers but fragments: wave-wide `buffer_load ... lds` copies
+// slots to LDS (64 consecutive rows per instruction; rows past the edge are clamped to the last one),
+// a lane reads two slots per term and block, no VALU work is left in the loop.
+//
+// Workgroup: four waves (one per SIMD) stacked along M, tile 256 x 160, wave tile 64 x 160 (ten
+// accumulator blocks).  A stage is one MFMA deep (64 k): 78 KB of slots, double buffered; one barrier
+// per stage, 60 MFMAs = 3840 cycles per wave between barriers, the loads of the next stage issued in
+// the gaps (unconditionally: past the last stage the last one is fetched again).
+#pragma once
+#include "cascmm_tile_kernel.h"
+
+namespace cascmm {
+
+struct F8K64 {
+  static constexpr int BM = 256, BN = 160, BK = 64, NT = 256, TERMS = 3;
+  static constexpr int WTM = 64, MT = 2, NTL = 5;
+  static constexpr int KU = BK / 16;                       // 16-k slot columns per stage
+  static constexpr int A_STAGE = TERMS * KU * BM * 16;     // 48 KB
+  static constexpr int B_STAGE = TERMS * KU * BN * 16;     // 30 KB
+  static constexpr int STAGE = A_STAGE + B_STAGE;          // 78 KB
+  static constexpr int LDS_BYTES = 2 * STAGE;              // 156 KB
+  static constexpr int A_LOADS = TERMS * KU;               // per wave: its own 64 rows
+  static constexpr int B_SLOTS = TERMS * KU * BN;          // 1920 = 30 x 64
+  static constexpr int B_LOADS_MAX = 8;                    // 30 instructions over 4 waves: 8, 8, 7, 7
+};
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// bytes of the slots of an operand with `rows` rows (columns) and K (multiple of 16) deep
+inline __host__ __device__ int64_t f8k64_slot_bytes(int64_t rows, int64_t K) { return (int64_t)F8K64::TERMS * (K / 16) * rows * 16; }
+
+// Split of the LEFT operand: A [M, K] fp32 row-major -> slots[term][K/16][M].  A workgroup converts
+// 64 rows x 64 k (a thread: 16 consecutive k of a row) and transposes through LDS so that the slots
+// leave as 1 KB runs along M.
+template <int UNUSED>
+__global__ __launch_bounds__(256) void f8k64_split_rows_kernel(const float* __restrict__ A, int M, int K, int64_t lda,
+                                                              const int32_t* __restrict__ tensor_exp, u32x4* __restrict__ out) {
+  __shared__ u32x4 slots[3][4][64];
+  const int kus = K >> 4;
+  const int ku_tiles = (kus + 3) >> 2;
+  const int m0 = (blockIdx.x / ku_tiles) * 64, ku0 = (blockIdx.x % ku_tiles) * 4;
+  const float scale = tensor_exp ? __builtin_ldexpf(1.f, *tensor_exp) : 1.f;
+  {
+    const int row = threadIdx.x >> 2, ku = threadIdx.x & 3;
+    if (m0 + row < M && ku0 + ku < kus) {
+      const float* src = A + (int64_t)(m0 + row) * lda + (ku0 + ku) * 16;
+      u32x4 t[3];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const f32x4 v0 = *(const f32x4*)(src + 8 * h), v1 = *(const f32x4*)(src + 8 * h + 4);
+        float r[8] = {v0[0] * scale, v0[1] * scale, v0[2] * scale, v0[3] * scale, v1[0] * scale, v1[1] * scale, v1[2] * scale, v1[3] * scale};
+        const u32x2 t0 = Lowp<CASCMM_FMT_FP8>::peel<false>(r);
+        const u32x2 t1 = Lowp<CASCMM_FMT_FP8>::peel<false>(r);
+        const u32x2 t2 = Lowp<CASCMM_FMT_FP8>::peel<true>(r);
+        t[0][2 * h] = t0[0]; t[0][2 * h + 1] = t0[1];
+        t[1][2 * h] = t1[0]; t[1][2 * h + 1] = t1[1];
+        t[2][2 * h] = t2[0]; t[2][2 * h + 1] = t2[1];
+      }
+#pragma unroll
+      for (int i = 0; i < 3; ++i) slots[i][ku][row] = t[i];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const int v = threadIdx.x + 256 * i;
+    const int row = v & 63, ku = (v >> 6) & 3, term = v >> 8;
+    if (m0 + row < M && ku0 + ku < kus) out[((int64_t)term * kus + ku0 + ku) * M + m0 + row] = slots[term][ku][row];
+  }
+}
+
+// Split of the RIGHT operand: B [K, N] fp32 row-major -> slots[term][K/16][N]; thread (ku, n) walks
+// 16 rows of column n (consecutive threads: consecutive columns, coalesced both ways).
+template <int UNUSED>
+__global__ __launch_bounds__(256) void f8k64_split_cols_kernel(const float* __restrict__ B, int K, int N, int64_t ldb,
+                                                              const int32_t* __restrict__ tensor_exp, u32x4* __restrict__ out) {
+  const int kus = K >> 4;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)kus * N) return;
+  const int ku = (int)(i / N), n = (int)(i - (int64_t)ku * N);
+  const float scale = tensor_exp ? __builtin_ldexpf(1.f, *tensor_exp) : 1.f;
+  const float* src = B + (int64_t)ku * 16 * ldb + n;
+  u32x4 t[3];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = src[(int64_t)(8 * h + e) * ldb] * scale;
+    const u32x2 t0 = Lowp<CASCMM_FMT_FP8>::peel<false>(r);
+    const u32x2 t1 = Lowp<CASCMM_FMT_FP8>::peel<false>(r);
+    const u32x2 t2 = Lowp<CASCMM_FMT_FP8>::peel<true>(r);
+    t[0][2 * h] = t0[0]; t[0][2 * h + 1] = t0[1];
+    t[1][2 * h] = t1[0]; t[1][2 * h + 1] = t1[1];
+    t[2][2 * h] = t2[0]; t[2][2 * h + 1] = t2[1];
+  }
+#pragma unroll
+  for (int j = 0; j < 3; ++j) out[((int64_t)j * kus + ku) * N + n] = t[j];
+}
+
+struct F8K64Params {
+  const u32x4* a_slots;   // [3][K/16][M]
+  const u32x4* b_slots;   // [3][K/16][N]
+  float* C;
+  const float* bias;
+  const int32_t* tensor_exps;   // {e_A, e_B} or NULL
+  int M, N, K;
+  int64_t ldc;
+  int tiles_m, tiles_n;
+};
+
+typedef __attribute__((address_space(3))) void* f8k64_lds_ptr;
+
+// Host-checked: K % 64 == 0, the slot buffers below 2 GiB, C rows addressable with 32-bit byte offsets
+// inside a tile.
+template <int UNUSED>
+__global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_f8k64_kernel(const F8K64Params p) {
+  typedef F8K64 T;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char f8k64_smem[];
+  unsigned char* smem = f8k64_smem;
+  const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = wave * T::WTM;
+  int tm, tn;
+  tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * T::BM, n0 = tn * T::BN;
+  const int ksteps = p.K / T::BK;
+  const int kus = p.K >> 4;
+
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.a_slots, 0, 0x7FFFFFFF, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.b_slots, 0, 0x7FFFFFFF, 0x00020000);
+  // A: the wave's own 64 rows, one instruction per (term, ku); lane = row (clamped to the last valid one)
+  int a_row = m0 + wm0 + lane;
+  a_row = a_row < p.M ? a_row : p.M - 1;
+  const int a_voff = a_row * 16;
+  const int a_plane = kus * p.M * 16;          // bytes between terms
+  const int a_ku = p.M * 16;                   // bytes between 16-k slot columns
+  // B: the stage's 1920 slots as 30 runs of 64; this wave takes runs wave, wave + 4, ...
+  int b_voff[T::B_LOADS_MAX], b_lds[T::B_LOADS_MAX];
+#pragma unroll
+  for (int j = 0; j < T::B_LOADS_MAX; ++j) {
+    int run = wave + 4 * j;
+    run = run < 30 ? run : 29;                 // (waves 2 and 3 repeat their last run: same bytes to the same place)
+    const int s = run * 64 + lane;
+    const int term = s / (T::KU * T::BN), ku = (s / T::BN) % T::KU;
+    int col = n0 + s % T::BN;
+    col = col < p.N ? col : p.N - 1;
+    b_lds[j] = T::A_STAGE + run * 1024;
+    b_voff[j] = ((term * kus + ku) * p.N + col) * 16;
+  }
+  const int b_step = T::KU * p.N * 16;         // bytes per stage
+  auto issue_a = [&](int step_, int j) {      // j = term * 4 + ku
+    const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
+    const int term = j >> 2, ku = j & 3;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (f8k64_lds_ptr)(smem + (step_ & 1) * T::STAGE + (j * T::BM + wm0) * 16), 16, a_voff,
+                                             term * a_plane + (step * T::KU + ku) * a_ku, 0, 0);
+  };
+  auto issue_b = [&](int step_, int j) {
+    const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (f8k64_lds_ptr)(smem + (step_ & 1) * T::STAGE + b_lds[j]), 16, b_voff[j], step * b_step, 0, 0);
+  };
+
+  // fragment addresses inside a stage: lane (row l31, k half h) reads slots (term, ku = 2 h) and (term, 2 h + 1)
+  const int a_frag = (2 * h * T::BM + wm0 + l31) * 16;                  // + term * KU * BM * 16 + mi * 512, second slot + BM * 16
+  const int b_frag = T::A_STAGE + (2 * h * T::BN + l31) * 16;           // + term * KU * BN * 16 + ni * 512, second slot + BN * 16
+  const int scales = 0x00777B7F;                                        // E8M0 bytes 2^0, 2^-4, 2^-8: op_sel picks the term's
+
+  f32x16 acc[T::MT][T::NTL];
+#pragma unroll
+  for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
+
+#define F8K64_FENCE() __builtin_amdgcn_sched_barrier(0)
+  auto frag = [&](const unsigned char* base, int second) {
+    const u32x4 lo = *(const u32x4*)base, hi = *(const u32x4*)(base + second);
+    return (i32x8){(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+  };
+
+#pragma unroll
+  for (int j = 0; j < T::A_LOADS; ++j) issue_a(0, j);
+#pragma unroll
+  for (int j = 0; j < T::B_LOADS_MAX; ++j) issue_b(0, j);
+
+  for (int s = 0; s < ksteps; ++s) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this wave's loads of stage s have landed
+    __builtin_amdgcn_s_barrier();           // ... everybody's, and stage s - 1 has been read by all
+    const unsigned char* st = smem + (s & 1) * T::STAGE;
+    i32x8 a[T::TERMS][T::MT];
+#pragma unroll
+    for (int t = 0; t < T::TERMS; ++t)
+#pragma unroll
+      for (int mi = 0; mi < T::MT; ++mi) a[t][mi] = frag(st + a_frag + t * T::KU * T::BM * 16 + mi * 512, T::BM * 16);
+    i32x8 b[2][T::TERMS];
+#pragma unroll
+    for (int t = 0; t < T::TERMS; ++t) b[0][t] = frag(st + b_frag + t * T::KU * T::BN * 16, T::BN * 16);
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni) {
+      const int cur = ni & 1, nxt = cur ^ 1;
+      // products smallest first, the two row blocks alternating; 20 loads of the next stage and the
+      // fragments of the next column block go into the gaps
+      int n_issued = 0;
+      auto gap = [&]() {
+        F8K64_FENCE();
+        const int slot = ni * 12 + n_issued;        // 12 MFMA gaps per column block, 60 per stage
+        if (n_issued < 3 && ni + 1 < T::NTL) b[nxt][n_issued] = frag(st + b_frag + n_issued * T::KU * T::BN * 16 + (ni + 1) * 512, T::BN * 16);
+        if (slot % 3 == 1 && slot / 3 < T::A_LOADS) issue_a(s + 1, slot / 3);
+        if (slot % 3 == 2 && slot / 3 < T::B_LOADS_MAX) issue_b(s + 1, slot / 3);
+        F8K64_FENCE();
+        ++n_issued;
+      };
+      // (the term numbers are the instruction's op_sel fields: literals)
+#define F8K64_PRODUCT(I, J)                                                                                                          \
+  acc[0][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[I][0], b[cur][J], acc[0][ni], 0, 0, I, scales, J, scales);          \
+  gap();                                                                                                                             \
+  acc[1][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[I][1], b[cur][J], acc[1][ni], 0, 0, I, scales, J, scales);          \
+  gap();
+      F8K64_PRODUCT(0, 2)
+      F8K64_PRODUCT(1, 1)
+      F8K64_PRODUCT(2, 0)
+      F8K64_PRODUCT(0, 1)
+      F8K64_PRODUCT(1, 0)
+      F8K64_PRODUCT(0, 0)
+#undef F8K64_PRODUCT
+    }
+  }
+#undef F8K64_FENCE
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // the redundant loads of the last stage land before LDS is given up
+
+  // ---- epilogue: undo the tensor scales, add the bias; a lane holds column l31, rows 8 q + 4 h + e ----
+  float out_scale = 1.f;
+  if (p.tensor_exps) out_scale = __builtin_ldexpf(1.f, -(p.tensor_exps[0] + p.tensor_exps[1]));
+  const int row_base = m0 + wm0 + 4 * h;
+#pragma unroll
+  for (int ni = 0; ni < T::NTL; ++ni) {
+    const int col = n0 + ni * 32 + l31;
+    if (col >= p.N) continue;
+    const float bv = p.bias ? p.bias[col] : 0.f;
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int row = row_base + mi * 32 + q * 8 + e;
+          if (row < p.M) p.C[(int64_t)row * p.ldc + col] = acc[mi][ni][4 * q + e] * out_scale + bv;
+        }
+  }
+}
+
+}  // namespace cascmm

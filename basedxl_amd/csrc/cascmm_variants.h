@@ -5,11 +5,13 @@
 
 #include "cascmm_bdirect_kernel.h"
 #include "cascmm_w512_kernel.h"
+#include "cascmm_f8k64_kernel.h"
 
 namespace cascmm {
 
 // KIND_W512: the large-tile kernel (whole 256 x 320 tiles only, one problem per launch)
-enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2 };
+// KIND_F8K64: three fp8 terms on the fp8-rate MFMA; splits its operands into the workspace first
+enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3 };
 constexpr int kNumCUs = 256;  // MI355X: what the cost model's constants were measured on
 constexpr int kMaxDevices = 64;
 
@@ -201,6 +203,60 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
   if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
   return CASCMM_OK;
 }
+
+// Workspace of the fp8-rate kernel: the slots of A, and those of B unless B comes prepared (each
+// rounded up to 256 bytes so that the second buffer stays aligned)
+inline size_t f8k64_workspace_bytes(int64_t M, int64_t N, int64_t K, bool bpre) {
+  auto up = [](int64_t b) { return (size_t)((b + 255) / 256 * 256); };
+  return up(f8k64_slot_bytes(M, K)) + (bpre ? 0 : up(f8k64_slot_bytes(N, K)));
+}
+
+// the fp8-rate kernel: split A (and B) into operand slots, then the GEMM on the slots
+template <bool BPRE>
+int launch_f8k64(const GroupParams& p, hipStream_t stream) {
+  typedef F8K64 T;
+  if (p.count != 1 || p.glu || p.k_splits > 1 || p.K % T::BK != 0 || p.K == 0) return CASCMM_ERR_BAD_VARIANT;
+  const size_t need = f8k64_workspace_bytes(p.M, p.N, p.K, BPRE);
+  if (!p.workspace || p.workspace_bytes < need) return CASCMM_ERR_WORKSPACE;
+  if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
+  if (f8k64_slot_bytes(p.M, p.K) > 0x7FFFFFFF || f8k64_slot_bytes(p.N, p.K) > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  auto kfn = cascmm_f8k64_kernel<0>;
+  static bool lds_set[kMaxDevices] = {false};
+  const int d = device_index();
+  if (d < 0) return CASCMM_ERR_LAUNCH;
+  if (!lds_set[d]) {
+    if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
+    lds_set[d] = true;
+  }
+  u32x4* a_slots = (u32x4*)p.workspace;
+  const u32x4* b_slots = (const u32x4*)p.B[0];
+  const int kus = p.K >> 4;
+  const unsigned a_grid = (unsigned)(((p.M + 63) / 64) * ((kus + 3) / 4));
+  if (launch_kernel(f8k64_split_rows_kernel<0>, dim3(a_grid), dim3(256), 0, stream, (const float*)p.A[0], p.M, p.K, p.lda,
+                    p.tensor_exps, a_slots) != hipSuccess)
+    return CASCMM_ERR_LAUNCH;
+  if (!BPRE) {
+    u32x4* bs = (u32x4*)((char*)p.workspace + (f8k64_slot_bytes(p.M, p.K) + 255) / 256 * 256);
+    const int64_t units = (int64_t)kus * p.N;
+    if (launch_kernel(f8k64_split_cols_kernel<0>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, (const float*)p.B[0],
+                      p.K, p.N, p.ldb, p.tensor_exps ? p.tensor_exps + 1 : (const int32_t*)nullptr, bs) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
+    b_slots = bs;
+  }
+  F8K64Params q;
+  q.a_slots = a_slots; q.b_slots = b_slots; q.C = (float*)p.C[0]; q.bias = (const float*)p.bias[0];
+  q.tensor_exps = p.tensor_exps;
+  q.M = p.M; q.N = p.N; q.K = p.K; q.ldc = p.ldc;
+  q.tiles_m = (p.M + T::BM - 1) / T::BM; q.tiles_n = (p.N + T::BN - 1) / T::BN;
+  const unsigned grid = (unsigned)(q.tiles_m * q.tiles_n);
+  if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q) != hipSuccess) return CASCMM_ERR_LAUNCH;
+  return CASCMM_OK;
+}
+
+#define CASCMM_F8K64_VARIANT(NAME, BPRE)                                                                                  \
+  {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8K64::BM, F8K64::BN, F8K64::BK, F8K64::NT, F8K64::LDS_BYTES, \
+   true, false, &launch_f8k64<BPRE>, BPRE}
 
 #define CASCMM_W512_VARIANT(NAME)                                                                                   \
   {NAME, KIND_W512, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, W512::BM, W512::BN, 32, W512::NT, W512::LDS_BYTES, true, \

@@ -563,8 +563,8 @@ def test_tile_k_split_is_exact_and_ordered(gpu_device, shape):
     bias = _gpu(torch.arange(N, dtype=torch.float32))
     ran = 0
     for vi, name in _variants_for("bf16x2_tri"):
-        if name.startswith(("bd", "skinny")):
-            continue
+        if name.startswith(("bd", "skinny")) or "_w512_" in name or "f8k64" in name:
+            continue  # (kernels without the K split over work items)
         bk = int(name.split("_")[0].split("x")[2])
         steps = -(-K // bk)
         if "generic" not in name and K % bk:
@@ -630,7 +630,7 @@ def _fmt_of(name):
     return fmt, int(name.split(fmt + "x")[1][0])
 
 
-@pytest.mark.parametrize("shape", [(154, 64, 48), (256, 192, 160), (300, 128, 200), (96, 128, 384), (257, 64, 164)])
+@pytest.mark.parametrize("shape", [(154, 64, 48), (256, 192, 160), (300, 128, 200), (96, 128, 384), (257, 64, 164), (130, 96, 84)])
 def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
     M, K, N = shape
     a, b, want = _int_case(M, K, N, 100, seed=M + K + N)
@@ -639,13 +639,15 @@ def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
     for vi, name in enumerate(_lib.variant_names()):
         if "_bpre" not in name or "_io" in name or K % int(name.split("_")[0].split("x")[2]):
             continue
+        if "fp8x3" in name and "f8k64" not in name and K % 64 == 0:
+            continue  # three fp8 terms with K in steps of 64 are prepared for the fp8-rate kernel (another slot layout)
         fmt, terms = _fmt_of(name)
         _say("int-exact prepared", shape, name)
         w = PreparedWeight(_gpu(torch.tensor(b, dtype=torch.float32)), lowp=fmt, terms=terms)
         out = cascaded_lowp_matmul(_gpu(torch.tensor(a, dtype=torch.float32)), w, variant=vi)
         assert np.array_equal(out.cpu().numpy().astype(np.int64), want), (name, shape)
         ran += 1
-    assert ran >= 4
+    assert ran >= (4 if K % 64 == 0 else 2)
 
 
 def test_prepared_weight_equals_raw_weight_bit_for_bit(gpu_device):
@@ -722,6 +724,8 @@ def test_grouped_launch_equals_separate_launches(gpu_device):
         for vi, name in _variants_for("bf16x2_tri"):
             if name.startswith(("bd", "skinny")) or "generic" in name or K % int(name.split("_")[0].split("x")[2]):
                 continue
+            if "_w512_" in name and (M % 256 or N % 320):
+                continue  # whole 256 x 320 tiles only
             outs = cascaded_lowp_matmul_grouped([x, x, x, y], ws, biases=[bs[0], None, bs[2], None], variant=vi)
             for i, a in enumerate([x, x, x, y]):
                 single = cascaded_lowp_matmul(a, ws[i], bias=bs[i] if i in (0, 2) else None, variant=vi)
@@ -740,8 +744,8 @@ def test_more_tiles_than_resident_workgroups(gpu_device):
     want = a @ b
     at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
     for vi, name in _variants_for("bf16x2_tri"):
-        if name.startswith("skinny"):
-            continue
+        if name.startswith("skinny") or "_w512_" in name:
+            continue  # (the large-tile kernel: whole 256 x 320 tiles only, one per workgroup)
         _say("many-tiles", name)
         got = cascaded_lowp_matmul(at, bt, variant=vi).cpu().numpy().astype(np.int64)
         assert np.array_equal(got, want), name
