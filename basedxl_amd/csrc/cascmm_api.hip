@@ -120,9 +120,6 @@ static const TunedCost kTuned[] = {
     {"t128x128x64_w4x1x1_d2_p8_bf16x2_tri", 1.224, 6.84, 0.80, 0.70},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri", 3.250, 5.00, 0.70, 0.50},
     {"t256x320x32_w512_bf16x2_tri", 5.65, 16.0, 1.00, 1.00},
-    // (fixed part: the passes that split the operands)
-    {"t256x160x64_f8k64_fp8x3_tri", 2.6, 22.0, 0.80, 0.60},
-    {"t256x160x64_f8k64_fp8x3_tri_bpre", 2.6, 14.0, 0.80, 0.60},
     // three fp16 / bf16 terms
     {"t128x128x32_w4x2x1_d2_fp16x3_tri", 3.107, 7.22, 0.90, 0.80},
     {"t64x64x32_w2x2x1_d3_fp16x3_tri", 1.088, 2.27, 1.00, 1.00},
@@ -177,6 +174,17 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     // smaller row tile was faster wherever both were measured.
     if ((double)((q.M + 63) / 64) * (double)((q.N + 127) / 128) >= kNumCUs / 2) return 1e9;
     return 1e-6 * (double)(((q.M + v.BM - 1) / v.BM) * v.BM) + 1e-8 * v.BM;
+  }
+  if (v.kind == KIND_F8K64) {
+    // stages of 64 k at ~2.1 us per resident round, the K split the launcher will use, and the passes
+    // around the GEMM: the split of A (and of B unless prepared), the reduction of a K split
+    const int sp = f8k64_splits(q.M, q.N, q.K);
+    const double items = tiles * sp;
+    const double rounds_ = items <= kNumCUs ? 1.0 : (double)(int64_t)(items / kNumCUs) + ((int64_t)items % kNumCUs ? 0.8 : 0.0);
+    double us = rounds_ * ((double)(q.K / 64 / sp) * 2.1 + 6.0) + 6.0 + (double)q.M * q.K * 7.0 / 4.0e6;
+    if (!q.bpre) us += 3.0 + (double)q.K * q.N * 7.0 / 4.0e6;
+    if (sp > 1) us += 3.0 + (double)(sp + 1) * q.M * q.N * 4.0 / 4.0e6;
+    return us;
   }
   if (info.tuned) {
     const TunedCost& t = *info.tuned;
@@ -336,7 +344,17 @@ __device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64
     const int64_t total = rows * cols;
     if (IODT == CASCMM_DT_F32 && ((uintptr_t)x % 16) == 0) {
       const int64_t quads = total / 4;
-      for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += (int64_t)gridDim.x * blockDim.x) {
+      const int64_t step = (int64_t)gridDim.x * blockDim.x;
+      int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+      // four independent loads in flight per thread
+      for (; i + 3 * step < quads; i += 4 * step) {
+        f32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = ((const f32x4*)x)[i + u * step];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { fold(v[u][0]); fold(v[u][1]); fold(v[u][2]); fold(v[u][3]); }
+      }
+      for (; i < quads; i += step) {
         const f32x4 v = ((const f32x4*)x)[i];
         fold(v[0]); fold(v[1]); fold(v[2]); fold(v[3]);
       }
@@ -381,17 +399,18 @@ __global__ void amax_end_kernel(int32_t* exp_out) { *exp_out = exp_of_amax((unsi
 // every other workgroup's contribution, writes {e_x, *second} and leaves the scratch zeroed for the
 // next call.  No workgroup waits for another.
 template <int IODT>
-__global__ __launch_bounds__(256) void amax_single_launch_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld,
-                                                                 const int32_t* second, int32_t* exps_out, unsigned* scratch) {
-  __shared__ unsigned wave_best[4];
+__global__ __launch_bounds__(1024) void amax_single_launch_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld,
+                                                                  const int32_t* second, int32_t* exps_out, unsigned* scratch) {
+  __shared__ unsigned wave_best[16];
   const unsigned best = amax_scan<IODT>(x, rows, cols, ld);
   if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = best;
   __syncthreads();
   if (threadIdx.x != 0) return;
-  unsigned b = wave_best[0];
-#pragma unroll
-  for (int w = 1; w < 4; ++w) b = wave_best[w] > b ? wave_best[w] : b;
-  if (b != 0) atomicMax(&scratch[0], b);
+  unsigned b = 0;
+  for (unsigned w = 0; w < (blockDim.x >> 6); ++w) b = wave_best[w] > b ? wave_best[w] : b;
+  // atomics of all workgroups on one word run one after another: skip the one that cannot raise
+  // the maximum (the running value only grows within a call, so a stale read errs on the safe side)
+  if (b > __hip_atomic_load(&scratch[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&scratch[0], b);
   __threadfence();
   const unsigned ticket = atomicAdd(&scratch[1], 1u);
   if (ticket != gridDim.x - 1) return;
@@ -881,15 +900,16 @@ int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, in
   const int64_t total = rows * cols;
   // (an empty tensor: one workgroup that scans nothing and writes e = 0)
   hipError_t err = hipSuccess;
-  const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((total + 4095) / 4096, 1024));
+  // few, large workgroups: every workgroup ends in a ticket atomic on one word, and those serialise
+  const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>((total + 16383) / 16384, device_cus() / 2));
   if (dtype == CASCMM_DT_F32)
-    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_F32>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_F32>), dim3(grid), dim3(1024), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
   else if (dtype == CASCMM_DT_F16)
-    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_F16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_F16>), dim3(grid), dim3(1024), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
   else
-    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(256), 0, s, x, rows, cols, ld, second_exp,
+    CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(1024), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
   return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
 }

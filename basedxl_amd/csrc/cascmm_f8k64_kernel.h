@@ -22,8 +22,12 @@
 // Workgroup: four waves (one per SIMD) stacked along M, tile 256 x 160, wave tile 64 x 160 (ten
 // accumulator blocks).  A stage is one MFMA deep (64 k): 78 KB of slots, double buffered; one barrier
 // per stage, 60 MFMAs = 3840 cycles per wave between barriers, the loads of the next stage issued in
-// the gaps (unconditionally: past the last stage the last one is fetched again).
+// the gaps (unconditionally: past the last stage the last one is fetched again).  The barrier sits in
+// front of a stage's last column block, whose fragments are already in registers, so the first
+// fragments of the next stage are read behind that block's MFMAs.
 #pragma once
+#include <type_traits>
+
 #include "cascmm_tile_kernel.h"
 
 namespace cascmm {
@@ -123,6 +127,8 @@ struct F8K64Params {
   int M, N, K;
   int64_t ldc;
   int tiles_m, tiles_n;
+  int k_splits;           // > 1: workgroup (split, tile) multiplies K range split and writes partials[split][M][N]
+  float* partials;
 };
 
 typedef __attribute__((address_space(3))) void* f8k64_lds_ptr;
@@ -137,10 +143,13 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = wave * T::WTM;
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int split = p.k_splits > 1 ? (int)blockIdx.x / tiles : 0;
   int tm, tn;
-  tile_coords(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+  tile_coords((int)blockIdx.x - split * tiles, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * T::BM, n0 = tn * T::BN;
-  const int ksteps = p.K / T::BK;
+  const int ksteps = p.K / T::BK / (p.k_splits > 1 ? p.k_splits : 1);   // stages of this workgroup (the host picks a divisor)
+  const int step0 = split * ksteps;
   const int kus = p.K >> 4;
 
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.a_slots, 0, 0x7FFFFFFF, 0x00020000);
@@ -166,13 +175,13 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   }
   const int b_step = T::KU * p.N * 16;         // bytes per stage
   auto issue_a = [&](int step_, int j) {      // j = term * 4 + ku
-    const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
+    const int step = step0 + (step_ < ksteps - 1 ? step_ : ksteps - 1);
     const int term = j >> 2, ku = j & 3;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (f8k64_lds_ptr)(smem + (step_ & 1) * T::STAGE + (j * T::BM + wm0) * 16), 16, a_voff,
                                              term * a_plane + (step * T::KU + ku) * a_ku, 0, 0);
   };
   auto issue_b = [&](int step_, int j) {
-    const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
+    const int step = step0 + (step_ < ksteps - 1 ? step_ : ksteps - 1);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (f8k64_lds_ptr)(smem + (step_ & 1) * T::STAGE + b_lds[j]), 16, b_voff[j], step * b_step, 0, 0);
   };
 
@@ -190,6 +199,10 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
 
 #define F8K64_FENCE() __builtin_amdgcn_sched_barrier(0)
+  auto issue = [&](int step_, int k) {     // load k (0 .. 19) of a stage: 12 of A, then 8 of B
+    if (k < T::A_LOADS) issue_a(step_, k);
+    else issue_b(step_, k - T::A_LOADS);
+  };
   auto frag = [&](const unsigned char* base, int second) {
     const u32x4 lo = *(const u32x4*)base, hi = *(const u32x4*)(base + second);
     return (i32x8){(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
@@ -200,38 +213,66 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #pragma unroll
   for (int j = 0; j < T::B_LOADS_MAX; ++j) issue_b(0, j);
 
-  for (int s = 0; s < ksteps; ++s) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0): this wave's loads of stage s have landed
-    __builtin_amdgcn_s_barrier();           // ... everybody's, and stage s - 1 has been read by all
+  // Fragments: A of the whole stage (the wave's own rows), B of one column block, both double
+  // buffered in registers.  The barrier that opens stage s + 1 sits in front of the LAST column block
+  // of stage s: by then the wave has read everything it needs of stage s from LDS (the last block's
+  // fragments are prefetched during the block before), so the first fragments of stage s + 1 are read
+  // behind that block's MFMAs and no LDS latency is exposed after a barrier.
+  i32x8 a[2][T::TERMS][T::MT];
+  i32x8 b[2][T::TERMS];
+  auto read_a = [&](int buf, const unsigned char* st, int t) {
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi) a[buf][t][mi] = frag(st + a_frag + t * T::KU * T::BM * 16 + mi * 512, T::BM * 16);
+  };
+  auto read_b = [&](int buf, const unsigned char* st, int ni, int t) {
+    b[buf][t] = frag(st + b_frag + t * T::KU * T::BN * 16 + ni * 512, T::BN * 16);
+  };
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): stage 0 has landed
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int t = 0; t < T::TERMS; ++t) {
+    read_a(0, smem, t);
+    read_b(0, smem, 0, t);
+  }
+#pragma unroll
+  for (int k = 0; k < 6; ++k) issue(1, k);
+
+  // ksteps is even or odd: the stage loop is unrolled by two so that the register buffers are static
+  auto stage = [&](int s, auto BUF) {
+    constexpr int ab = decltype(BUF)::value;       // A buffer of this stage; B block ni uses buffer (ab * 5 + ni) & 1
     const unsigned char* st = smem + (s & 1) * T::STAGE;
-    i32x8 a[T::TERMS][T::MT];
-#pragma unroll
-    for (int t = 0; t < T::TERMS; ++t)
-#pragma unroll
-      for (int mi = 0; mi < T::MT; ++mi) a[t][mi] = frag(st + a_frag + t * T::KU * T::BM * 16 + mi * 512, T::BM * 16);
-    i32x8 b[2][T::TERMS];
-#pragma unroll
-    for (int t = 0; t < T::TERMS; ++t) b[0][t] = frag(st + b_frag + t * T::KU * T::BN * 16, T::BN * 16);
+    const unsigned char* st_next = smem + ((s + 1) & 1) * T::STAGE;
 #pragma unroll
     for (int ni = 0; ni < T::NTL; ++ni) {
-      const int cur = ni & 1, nxt = cur ^ 1;
-      // products smallest first, the two row blocks alternating; 20 loads of the next stage and the
-      // fragments of the next column block go into the gaps
+      const int cur = (ab * T::NTL + ni) & 1, nxt = cur ^ 1;
+      if (ni == T::NTL - 1) {
+        // everything this wave needs of stage s is in registers: open stage s + 1
+        __builtin_amdgcn_s_waitcnt(0x0F70);     // own loads of stage s + 1 have landed (issued ~2000 cycles ago)
+        __builtin_amdgcn_s_barrier();           // everybody's; and nobody reads stage s any more
+      }
       int n_issued = 0;
       auto gap = [&]() {
         F8K64_FENCE();
-        const int slot = ni * 12 + n_issued;        // 12 MFMA gaps per column block, 60 per stage
-        if (n_issued < 3 && ni + 1 < T::NTL) b[nxt][n_issued] = frag(st + b_frag + n_issued * T::KU * T::BN * 16 + (ni + 1) * 512, T::BN * 16);
-        if (slot % 3 == 1 && slot / 3 < T::A_LOADS) issue_a(s + 1, slot / 3);
-        if (slot % 3 == 2 && slot / 3 < T::B_LOADS_MAX) issue_b(s + 1, slot / 3);
+        if (ni < T::NTL - 1) {
+          if (n_issued < 3) read_b(nxt, st, ni + 1, n_issued);   // the fragments of the next column block
+          // loads 6 .. 19 of stage s + 1 (its buffer was given up at the barrier inside stage s - 1): gaps
+          // 3 .. 11 of block 0 and 3 .. 7 of block 1, which leaves them two and a half blocks to land
+          const int k = ni == 0 ? n_issued + 3 : ni == 1 ? n_issued + 12 : -1;
+          if (n_issued >= 3 && k >= 6 && k < 20) issue(s + 1, k);
+        } else {
+          // behind the last block: the first fragments of stage s + 1, then loads 0 .. 5 of stage s + 2
+          if (n_issued < 3) read_b(nxt, st_next, 0, n_issued);
+          else if (n_issued < 6) read_a(ab ^ 1, st_next, n_issued - 3);
+          else issue(s + 2, n_issued - 6);
+        }
         F8K64_FENCE();
         ++n_issued;
       };
       // (the term numbers are the instruction's op_sel fields: literals)
-#define F8K64_PRODUCT(I, J)                                                                                                          \
-  acc[0][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[I][0], b[cur][J], acc[0][ni], 0, 0, I, scales, J, scales);          \
-  gap();                                                                                                                             \
-  acc[1][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[I][1], b[cur][J], acc[1][ni], 0, 0, I, scales, J, scales);          \
+#define F8K64_PRODUCT(I, J)                                                                                                              \
+  acc[0][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[ab][I][0], b[cur][J], acc[0][ni], 0, 0, I, scales, J, scales);          \
+  gap();                                                                                                                                 \
+  acc[1][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[ab][I][1], b[cur][J], acc[1][ni], 0, 0, I, scales, J, scales);          \
   gap();
       F8K64_PRODUCT(0, 2)
       F8K64_PRODUCT(1, 1)
@@ -241,7 +282,13 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       F8K64_PRODUCT(0, 0)
 #undef F8K64_PRODUCT
     }
+  };
+  int s = 0;
+  for (; s + 2 <= ksteps; s += 2) {
+    stage(s, std::integral_constant<int, 0>{});
+    stage(s + 1, std::integral_constant<int, 1>{});
   }
+  if (s < ksteps) stage(s, std::integral_constant<int, 0>{});
 #undef F8K64_FENCE
   __builtin_amdgcn_s_waitcnt(0x0F70);       // the redundant loads of the last stage land before LDS is given up
 
@@ -249,11 +296,37 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   float out_scale = 1.f;
   if (p.tensor_exps) out_scale = __builtin_ldexpf(1.f, -(p.tensor_exps[0] + p.tensor_exps[1]));
   const int row_base = m0 + wm0 + 4 * h;
+  float* C = p.C;
+  int64_t ldc = p.ldc;
+  const float* bias = p.bias;
+  if (p.k_splits > 1) {   // partial result (scaled, no bias): the reduction kernel adds the splits in order
+    C = p.partials + (int64_t)split * p.M * p.N;
+    ldc = p.N;
+    bias = nullptr;
+  }
+  if (m0 + T::BM <= p.M && n0 + T::BN <= p.N && ldc * (int64_t)(T::BM * 4) < 0x7FFFFFFF) {
+    // whole tile inside C: buffer stores, the row as a scalar offset, nothing to mask
+    const i32x4 rc = make_rsrc(C + (int64_t)(m0 + wm0) * ldc + n0, 0x7FFFFFFF);
+    const int ldc_bytes = (int)ldc * 4;
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni) {
+      const float bv = bias ? bias[n0 + ni * 32 + l31] : 0.f;
+      const int voff = h * 4 * ldc_bytes + (ni * 32 + l31) * 4;
+#pragma unroll
+      for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            llvm_raw_buffer_store_f32(acc[mi][ni][4 * q + e] * out_scale + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+    }
+    return;
+  }
 #pragma unroll
   for (int ni = 0; ni < T::NTL; ++ni) {
     const int col = n0 + ni * 32 + l31;
     if (col >= p.N) continue;
-    const float bv = p.bias ? p.bias[col] : 0.f;
+    const float bv = bias ? bias[col] : 0.f;
 #pragma unroll
     for (int mi = 0; mi < T::MT; ++mi)
 #pragma unroll
@@ -261,7 +334,7 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int row = row_base + mi * 32 + q * 8 + e;
-          if (row < p.M) p.C[(int64_t)row * p.ldc + col] = acc[mi][ni][4 * q + e] * out_scale + bv;
+          if (row < p.M) C[(int64_t)row * ldc + col] = acc[mi][ni][4 * q + e] * out_scale + bv;
         }
   }
 }

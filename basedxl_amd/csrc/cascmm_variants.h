@@ -204,11 +204,31 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
   return CASCMM_OK;
 }
 
-// Workspace of the fp8-rate kernel: the slots of A, and those of B unless B comes prepared (each
-// rounded up to 256 bytes so that the second buffer stays aligned)
+// K split of the fp8-rate kernel for problems with fewer tiles than CUs: the split count that
+// minimises stages-per-workgroup x 2.1 us + the round trip of the partial results at ~4 TB/s
+inline int f8k64_splits(int64_t M, int64_t N, int64_t K) {
+  const int64_t tiles = ((M + F8K64::BM - 1) / F8K64::BM) * ((N + F8K64::BN - 1) / F8K64::BN);
+  const int64_t steps = K / F8K64::BK;
+  int best = 1;
+  double best_us = (double)steps * 2.1;
+  for (int sp = 2; sp <= 16; ++sp) {
+    if (steps % sp != 0 || tiles * sp > kNumCUs) continue;
+    const double us = (double)(steps / sp) * 2.1 + 3.0 + (double)(sp + 1) * (double)M * (double)N * 4.0 / 4.0e6;
+    if (us < best_us) {
+      best_us = us;
+      best = sp;
+    }
+  }
+  return best;
+}
+
+// Workspace of the fp8-rate kernel: the slots of A, those of B unless B comes prepared, and the
+// partial results of a K split (each rounded up to 256 bytes so that the next buffer stays aligned)
+inline size_t f8k64_up(int64_t b) { return (size_t)((b + 255) / 256 * 256); }
 inline size_t f8k64_workspace_bytes(int64_t M, int64_t N, int64_t K, bool bpre) {
-  auto up = [](int64_t b) { return (size_t)((b + 255) / 256 * 256); };
-  return up(f8k64_slot_bytes(M, K)) + (bpre ? 0 : up(f8k64_slot_bytes(N, K)));
+  const int sp = f8k64_splits(M, N, K);
+  return f8k64_up(f8k64_slot_bytes(M, K)) + (bpre ? 0 : f8k64_up(f8k64_slot_bytes(N, K))) +
+         (sp > 1 ? f8k64_up((int64_t)sp * M * N * 4) : 0);
 }
 
 // the fp8-rate kernel: split A (and B) into operand slots, then the GEMM on the slots
@@ -231,13 +251,15 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   }
   u32x4* a_slots = (u32x4*)p.workspace;
   const u32x4* b_slots = (const u32x4*)p.B[0];
+  char* ws_next = (char*)p.workspace + f8k64_up(f8k64_slot_bytes(p.M, p.K));
   const int kus = p.K >> 4;
   const unsigned a_grid = (unsigned)(((p.M + 63) / 64) * ((kus + 3) / 4));
   if (launch_kernel(f8k64_split_rows_kernel<0>, dim3(a_grid), dim3(256), 0, stream, (const float*)p.A[0], p.M, p.K, p.lda,
                     p.tensor_exps, a_slots) != hipSuccess)
     return CASCMM_ERR_LAUNCH;
   if (!BPRE) {
-    u32x4* bs = (u32x4*)((char*)p.workspace + (f8k64_slot_bytes(p.M, p.K) + 255) / 256 * 256);
+    u32x4* bs = (u32x4*)ws_next;
+    ws_next += f8k64_up(f8k64_slot_bytes(p.N, p.K));
     const int64_t units = (int64_t)kus * p.N;
     if (launch_kernel(f8k64_split_cols_kernel<0>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, (const float*)p.B[0],
                       p.K, p.N, p.ldb, p.tensor_exps ? p.tensor_exps + 1 : (const int32_t*)nullptr, bs) != hipSuccess)
@@ -249,8 +271,18 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   q.tensor_exps = p.tensor_exps;
   q.M = p.M; q.N = p.N; q.K = p.K; q.ldc = p.ldc;
   q.tiles_m = (p.M + T::BM - 1) / T::BM; q.tiles_n = (p.N + T::BN - 1) / T::BN;
-  const unsigned grid = (unsigned)(q.tiles_m * q.tiles_n);
+  q.k_splits = f8k64_splits(p.M, p.N, p.K);
+  q.partials = (float*)ws_next;
+  const unsigned grid = (unsigned)(q.tiles_m * q.tiles_n * q.k_splits);
   if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q) != hipSuccess) return CASCMM_ERR_LAUNCH;
+  if (q.k_splits > 1) {
+    const int64_t elems = (int64_t)p.M * p.N;
+    const int vec_out = p.ldc % 4 == 0 && p.N % 4 == 0 && (uintptr_t)p.C[0] % 16 == 0 && (uintptr_t)p.bias[0] % 16 == 0;
+    if (launch_kernel(splitk_reduce_kernel, dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, stream,
+                      (const float*)q.partials, q.k_splits, p.M, p.N, (const float*)p.bias[0], (float*)p.C[0], p.ldc,
+                      vec_out) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
+  }
   return CASCMM_OK;
 }
 
