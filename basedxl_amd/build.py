@@ -51,6 +51,12 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    # a kernel whose launch stub the compiler left out only shows up as an undefined symbol at load time
+    import ctypes
+    try:
+        ctypes.CDLL(LIB)
+    except OSError as e:
+        raise RuntimeError(f"{LIB} was linked but does not load: {e}") from None
     if verbose:
         print(f"built {LIB} from {len(srcs)} translation units")
     return LIB

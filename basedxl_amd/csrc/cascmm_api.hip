@@ -96,6 +96,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
     return false;
   if (v.bpre && v.kind != KIND_F8K64 && prepared_as_k16_slots(q.K, q.fmt, q.terms, q.glu)) return false;   // other layout
   if (v.kind == KIND_W512 && (q.M % v.BM != 0 || q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX)) return false;
+  if (v.kind == KIND_WAVEK && (q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX || q.K == 0)) return false;
   if (q.glu && !v.glu) return false;
   return true;
 }
@@ -157,6 +158,35 @@ static const std::vector<VariantInfo>& variant_info() {
   return info;
 }
 
+// The kernel that splits K over the waves of a workgroup (KIND_WAVEK) moves (32 + BN) x K x 4 bytes
+// into every workgroup and is bound by that: a CU pulled in 85 bytes per ns with the 32-wide and
+// 60 with the 64-wide tile, all CUs together 17 KB per ns (154 x 2048 x {640, 1280, 2560}); a launch
+// costs 2.5 us, prologue and the meeting of the partial tiles 0.6 us per round of workgroups.
+static bool wavek_eligible(const Problem& q) {
+  return q.dtype == CASCMM_DT_F32 && q.fmt == CASCMM_FMT_BF16 && q.terms == 2 && q.products == CASCMM_PROD_TRI && !q.bpre &&
+         !q.glu && q.K > 0 && q.K % 32 == 0 && q.N % 32 == 0 && q.M * q.lda * 4 <= INT32_MAX;
+}
+static double wavek_estimate_us(const Problem& q, int count, int bn) {
+  if (q.N % bn != 0) return 1e9;
+  const double items = (double)count * (double)((q.M + 31) / 32) * (double)(q.N / bn);
+  const double active = items < kNumCUs ? items : kNumCUs;
+  const double per_cu = bn == 32 ? 85.0e3 : 60.0e3;                       // bytes per us
+  const double rate = per_cu < 17.0e6 / active ? per_cu : 17.0e6 / active;
+  const double rounds = (double)(int64_t)((items + kNumCUs - 1) / kNumCUs);
+  return 2.5 + rounds * (0.6 + (double)(32 + bn) * (double)q.K * 4.0 / rate);
+}
+static double wavek_estimate_us(const Problem& q, int count) {
+  const double a = wavek_estimate_us(q, count, 32), b = wavek_estimate_us(q, count, 64);
+  return a < b ? a : b;
+}
+// The skinny split-K path for comparison (its 32-row variant, the one preferred among them): two
+// launches, a workgroup's (32 + 128) x K / splits x 4 bytes at 70 bytes per ns, the partial results
+// written and read back at about 4 TB/s (fitted on the same shapes).
+static double skinny_estimate_us(const Problem& q) {
+  const int sp = skinny_splits(q.M, q.N, q.K, 32, 128, 64);
+  return 8.5 + 160.0 * (double)(q.K / sp) * 4.0 / 70.0e3 + 2.0 * sp * (double)q.M * (double)q.N * 4.0 / 4.0e6;
+}
+
 // ws_bytes: workspace the caller brought; *splits_out: K split the cost was computed for (the
 // LDS-tiled two-term bf16 kernels may split K over up to kMaxTileSplits work items per tile when a
 // single problem has too few tiles to occupy the chip and the workspace holds the partials)
@@ -173,8 +203,11 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     // kernels would leave more than half of the CUs idle; among the split-K variants the
     // smaller row tile was faster wherever both were measured.
     if ((double)((q.M + 63) / 64) * (double)((q.N + 127) / 128) >= kNumCUs / 2) return 1e9;
+    // ... unless the one-launch kernel that splits K over its waves is expected to be faster
+    if (wavek_eligible(q) && wavek_estimate_us(q, count) < skinny_estimate_us(q)) return 1e9;
     return 1e-6 * (double)(((q.M + v.BM - 1) / v.BM) * v.BM) + 1e-8 * v.BM;
   }
+  if (v.kind == KIND_WAVEK) return wavek_estimate_us(q, count, v.BN);
   if (v.kind == KIND_F8K64) {
     // stages of 64 k at ~2.1 us per resident round, the K split the launcher will use, and the passes
     // around the GEMM: the split of A (and of B unless prepared), the reduction of a K split

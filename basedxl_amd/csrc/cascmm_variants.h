@@ -6,12 +6,14 @@
 #include "cascmm_bdirect_kernel.h"
 #include "cascmm_w512_kernel.h"
 #include "cascmm_f8k64_kernel.h"
+#include "cascmm_wavek_kernel.h"
 
 namespace cascmm {
 
 // KIND_W512: the large-tile kernel (whole 256 x 320 tiles only, one problem per launch)
 // KIND_F8K64: three fp8 terms on the fp8-rate MFMA; splits its operands into the workspace first
-enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3 };
+// KIND_WAVEK: skinny problems in one launch, K split over the waves of a workgroup (no workspace)
+enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3, KIND_WAVEK = 4 };
 constexpr int kNumCUs = 256;  // MI355X: what the cost model's constants were measured on
 constexpr int kMaxDevices = 64;
 
@@ -204,6 +206,31 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
   return CASCMM_OK;
 }
 
+// skinny problems, K split over the waves of a workgroup
+template <int NB>
+int launch_wavek(const GroupParams& p, hipStream_t stream) {
+  typedef WaveK<NB> T;
+  if (p.glu || p.k_splits > 1 || p.count < 1) return CASCMM_ERR_BAD_VARIANT;
+  if (p.N % T::BN != 0 || p.K % T::BK != 0) return CASCMM_ERR_BAD_VARIANT;
+  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  auto kfn = cascmm_wavek_kernel<NB>;
+  static bool lds_set[kMaxDevices] = {false};
+  const int d = device_index();
+  if (d < 0) return CASCMM_ERR_LAUNCH;
+  if (!lds_set[d]) {
+    if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
+    lds_set[d] = true;
+  }
+  GroupParams q = p;
+  q.tiles_m = (p.M + T::BM - 1) / T::BM;
+  q.tiles_n = p.N / T::BN;
+  const int64_t grid = (int64_t)q.count * q.tiles_m * q.tiles_n;
+  if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  if (launch_kernel(kfn, dim3((unsigned)grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q) != hipSuccess) return CASCMM_ERR_LAUNCH;
+  return CASCMM_OK;
+}
+
 // K split of the fp8-rate kernel for problems with fewer tiles than CUs: the split count that
 // minimises stages-per-workgroup x 2.1 us + the round trip of the partial results at ~4 TB/s
 inline int f8k64_splits(int64_t M, int64_t N, int64_t K) {
@@ -289,6 +316,10 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
 #define CASCMM_F8K64_VARIANT(NAME, BPRE)                                                                                  \
   {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8K64::BM, F8K64::BN, F8K64::BK, F8K64::NT, F8K64::LDS_BYTES, \
    true, false, &launch_f8k64<BPRE>, BPRE}
+
+#define CASCMM_WAVEK_VARIANT(NAME, NB)                                                                                \
+  {NAME, KIND_WAVEK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, WaveK<NB>::BM, WaveK<NB>::BN, WaveK<NB>::BK, WaveK<NB>::NT, \
+   WaveK<NB>::LDS_BYTES, true, true, &launch_wavek<NB>}
 
 #define CASCMM_W512_VARIANT(NAME)                                                                                   \
   {NAME, KIND_W512, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, W512::BM, W512::BN, 32, W512::NT, W512::LDS_BYTES, true, \

@@ -47,7 +47,7 @@ METRIC = {"ffn": "fp32-equiv TFLOP/s + % of MFMA roofline at SDXL FFN shape; rel
 # HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
 # summaries under profiles/ give the commands and the calibration); keyed by (workload, launch label).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    ("ffn", "ff.net.0.proj (W1)"): 2 * 92592.1 * 1024 + 89856.0 * 1024,
+    ("ffn", "ff.net.0.proj (W1)"): 2 * 72861.5 * 1024 + 83968.0 * 1024,
     ("attn", "to_q/to_k/to_v grouped"): 2 * 21930.0 * 1024 + 30720.0 * 1024,
 }
 

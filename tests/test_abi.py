@@ -89,7 +89,8 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
     names = _lib.variant_names()
     pick = lambda M, K, N: names[l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0) & 0xFFFF]
     assert pick(2048, 1280, 10240) == "t256x320x32_w512_bf16x2_tri"               # cfg3, first GEMM
-    assert pick(154, 2048, 1280).startswith("skinny") and pick(154, 2048, 640).startswith("skinny")   # cfg4
+    assert pick(154, 2048, 1280) == "t32x32x32_wavek_bf16x2_tri" and pick(154, 2048, 640) == "t32x32x32_wavek_bf16x2_tri"   # cfg4
+    assert pick(16, 2816, 1280).startswith("skinny")   # few tiles, deep K: split over workgroups
     grouped = names[l.cascmm_select_variant_grouped(3, 4096, 640, 640, 640, 640, 640, 0, 0, 2, 0) & 0xFFFF]
     assert grouped == "t256x128x32_w4x1x1_d2_bf16x2_tri"                           # cfg2, to_q / to_k / to_v
     assert pick(4096, 640, 640) == "t64x160x64_w2x1x2_d2_p8_bf16x2_tri"            # cfg2, to_out

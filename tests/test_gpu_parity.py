@@ -186,6 +186,8 @@ def test_integer_operands_are_exact_on_every_variant(gpu_device, shape):
             continue  # split-K variants take at most five row tiles and at least four K steps
         if "_w512_" in name and (M % 256 != 0 or N % 320 != 0 or K % 32 != 0):
             continue  # the large-tile kernel takes whole 256 x 320 tiles and K in steps of 32
+        if "_wavek_" in name and N % int(name.split("_")[0].split("x")[1]) != 0:
+            continue  # the kernel that splits K over its waves takes whole column tiles
         _say("int-exact", shape, name)
         out = cascaded_lowp_matmul(at7 if small else at, bt7 if small else bt, lowp=fmt, terms=terms, products=products,
                                    variant=vi)
@@ -414,26 +416,64 @@ def test_every_headline_variant_meets_the_bound(gpu_device):
         assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"], name
 
 
-@pytest.mark.parametrize("shape", [(154, 2048, 1280), (154, 2048, 640), (32, 1024, 384), (77, 768, 320)])
+@pytest.mark.parametrize("shape", [(154, 2048, 1280), (154, 2048, 640), (32, 1024, 384), (77, 768, 320), (16, 2816, 1280)])
 def test_skinny_split_k_meets_the_bound(gpu_device, shape):
-    """Text-token shapes (cross-attention K/V projections): the automatic choice is a split-K
-    variant, its result meets the bound and is bit-identical from launch to launch."""
+    """Text-token shapes (cross-attention K/V projections): the automatic choice is the one-launch
+    kernel that splits K over the waves of a workgroup, or a split-K variant with its reduction
+    pass; both meet the bound and are bit-identical from launch to launch."""
     M, K, N = shape
     a, b = oc.make_operands(M, K, N, seed=21, w_std=0.02)
     exp = oc.fp64_matmul(a, b)
     ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exp)
     ad, bd = _gpu(a), _gpu(b)
     l = _lib.lib()
+    names = _lib.variant_names()
     chosen = l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0)
-    assert _lib.variant_names()[chosen].startswith("skinny"), _lib.variant_names()[chosen]
+    assert names[chosen].startswith("skinny") or "_wavek_" in names[chosen], names[chosen]
     assert l.cascmm_workspace_bytes(M, N, K, 0, 0, 2, 0) >= M * N * 4
-    _say("skinny", shape, _lib.variant_names()[chosen])
     bias = _gpu(torch.randn(N))
-    first = cascaded_lowp_matmul(ad, bd, bias=bias).clone()
-    got = oc.error_metrics((first - bias).cpu(), exp)
-    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"] + 1e-6, (got, ref)
-    for _ in range(5):
-        assert torch.equal(cascaded_lowp_matmul(ad, bd, bias=bias), first)
+    candidates = [-1] + [vi for vi, name in _variants_for("bf16x2_tri")
+                         if (name.startswith("skinny32") and K >= 256 and K % 64 == 0) or
+                         ("_wavek_" in name and N % int(name.split("_")[0].split("x")[1]) == 0)]
+    assert len(candidates) >= 3
+    for vi in candidates:
+        _say("skinny", shape, names[chosen] if vi < 0 else names[vi])
+        first = cascaded_lowp_matmul(ad, bd, bias=bias, variant=vi).clone()
+        got = oc.error_metrics((first - bias).cpu(), exp)
+        assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"] + 1e-6, (got, ref)
+        for _ in range(5):
+            assert torch.equal(cascaded_lowp_matmul(ad, bd, bias=bias, variant=vi), first)
+
+
+@pytest.mark.parametrize("shape", [(154, 2048, 1280), (77, 64, 96), (2, 320, 1280), (33, 32, 32), (200, 2080, 64)])
+def test_wave_split_kernel_is_exact_on_integers_without_workspace(gpu_device, shape):
+    """The one-launch skinny kernel through the C ABI with no workspace at all (automatic choice, then
+    both of its tiles forced): exact on integer operands (ragged M, fewer K steps than waves, a K
+    whose steps do not divide by the eight waves), bias added, rows past M untouched."""
+    M, K, N = shape
+    a, b, want = _int_case(M, K, N, 30, seed=M + K + N)
+    at, bt = _gpu(torch.tensor(a, dtype=torch.float32)), _gpu(torch.tensor(b, dtype=torch.float32))
+    bias = _gpu(torch.arange(N, dtype=torch.float32))
+    l = _lib.lib()
+    out = torch.full((M + 3, N), -7.0, device=at.device)
+    picked = l.cascmm_select_variant(M, N, K, K, N, N, 0, 0, 2, 0)
+    _say("wavek", shape, _lib.variant_names()[picked])
+    st = l.cascmm_gemm(at.data_ptr(), bt.data_ptr(), out.data_ptr(), bias.data_ptr(), M, N, K, K, N, N, 0, 0, 2, 0, None, None, 0,
+                       torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(out[:M].cpu().numpy().astype(np.int64), want + np.arange(N)[None, :])
+    assert bool((out[M:] == -7.0).all())
+    for vi, name in _variants_for("bf16x2_tri"):
+        if "_wavek_" not in name or N % int(name.split("_")[0].split("x")[1]):
+            continue
+        out.fill_(-7.0)
+        st = l.cascmm_gemm_variant(at.data_ptr(), bt.data_ptr(), out.data_ptr(), bias.data_ptr(), M, N, K, K, N, N, 0, 0, 2, 0,
+                                   None, None, 0, torch.cuda.current_stream().cuda_stream, vi)
+        assert st == 0, name
+        torch.cuda.synchronize()
+        assert np.array_equal(out[:M].cpu().numpy().astype(np.int64), want + np.arange(N)[None, :]), name
+        assert bool((out[M:] == -7.0).all()), name
 
 
 def test_skinny_without_workspace_falls_back_or_reports(gpu_device):
@@ -563,7 +603,7 @@ def test_tile_k_split_is_exact_and_ordered(gpu_device, shape):
     bias = _gpu(torch.arange(N, dtype=torch.float32))
     ran = 0
     for vi, name in _variants_for("bf16x2_tri"):
-        if name.startswith(("bd", "skinny")) or "_w512_" in name or "f8k64" in name:
+        if name.startswith(("bd", "skinny")) or "_w512_" in name or "f8k64" in name or "_wavek_" in name:
             continue  # (kernels without the K split over work items)
         bk = int(name.split("_")[0].split("x")[2])
         steps = -(-K // bk)
@@ -726,6 +766,8 @@ def test_grouped_launch_equals_separate_launches(gpu_device):
                 continue
             if "_w512_" in name and (M % 256 or N % 320):
                 continue  # whole 256 x 320 tiles only
+            if "_wavek_" in name and N % int(name.split("_")[0].split("x")[1]):
+                continue  # whole column tiles only
             outs = cascaded_lowp_matmul_grouped([x, x, x, y], ws, biases=[bs[0], None, bs[2], None], variant=vi)
             for i, a in enumerate([x, x, x, y]):
                 single = cascaded_lowp_matmul(a, ws[i], bias=bs[i] if i in (0, 2) else None, variant=vi)
