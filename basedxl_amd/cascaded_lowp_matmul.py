@@ -92,10 +92,9 @@ def _check_bias(bias: Optional[torch.Tensor], like: torch.Tensor, n: int) -> Opt
 _exp_scratch: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
-def _activation_exps(a2: torch.Tensor, lda: int, second: Optional[torch.Tensor], out_ptr: int, stream: int) -> None:
-    """{e_A, e_B} at ``out_ptr`` (device int32[2]) in one launch: the fp8 scale exponent of ``a2`` found
-    on the device, next to the kept exponent ``second`` of the other operand (skipped when None)."""
-    dev = a2.device
+def _scale_scratch(dev: torch.device, stream: int) -> torch.Tensor:
+    """The two zeroed device int32 the one-launch scale search needs (it leaves them zeroed): one per
+    (device, stream) for eager launches, one per device for launches recorded into a device graph."""
     index = dev.index if dev.index is not None else torch.cuda.current_device()
     capturing = torch.cuda.is_current_stream_capturing()
     key = (index, "capture" if capturing else stream)
@@ -103,10 +102,35 @@ def _activation_exps(a2: torch.Tensor, lda: int, second: Optional[torch.Tensor],
         _exp_scratch[(index, "capture")] = torch.zeros(2, dtype=torch.int32, device=dev)
     scratch = _exp_scratch.get(key)
     if scratch is None:
-        scratch = _exp_scratch[key] = torch.zeros(2, dtype=torch.int32, device=dev)   # the kernel leaves it zeroed
+        scratch = _exp_scratch[key] = torch.zeros(2, dtype=torch.int32, device=dev)
+    return scratch
+
+
+def _activation_exps(a2: torch.Tensor, lda: int, second: Optional[torch.Tensor], out_ptr: int, stream: int) -> None:
+    """{e_A, e_B} at ``out_ptr`` (device int32[2]) in one launch: the fp8 scale exponent of ``a2`` found
+    on the device, next to the kept exponent ``second`` of the other operand (skipped when None)."""
+    scratch = _scale_scratch(a2.device, stream)
     _lib.check(_lib.lib().cascmm_tensor_exps(a2.data_ptr(), a2.shape[0], a2.shape[1], lda, _DTYPES[a2.dtype],
                                              second.data_ptr() if second is not None else None, out_ptr,
                                              scratch.data_ptr(), stream), "cascmm_tensor_exps")
+
+
+def _gemm_fp8_autoscale(a2: torch.Tensor, b_ptr: int, b_prepared: bool, out2: torch.Tensor, bias: Optional[torch.Tensor],
+                        M: int, N: int, K: int, lda: int, ldb: int, ldc: int, terms: int, products: int,
+                        b_exp: torch.Tensor) -> None:
+    """One fp8 GEMM on fp32 tensors whose activation scale is found inside the call (the weight's is
+    kept): cascmm_gemm_fp8_autoscale, which folds the search into the operand split of the fp8-rate
+    kernel and otherwise runs the one-launch search followed by the GEMM."""
+    dev = a2.device
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    ws = _workspace(dev, stream, _workspace_bytes(M, N, K, _lib.DT_F32, _lib.FMT_FP8, terms, products))
+    exps = torch.empty(2, dtype=torch.int32, device=dev)
+    scratch = _scale_scratch(dev, stream)
+    st = _lib.lib().cascmm_gemm_fp8_autoscale(
+        a2.data_ptr(), b_ptr, 1 if b_prepared else 0, out2.data_ptr(), bias.data_ptr() if bias is not None else None,
+        M, N, K, lda, ldb, ldc, terms, products, b_exp.data_ptr(), exps.data_ptr(), scratch.data_ptr(),
+        ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, stream)
+    _lib.check(st, "cascmm_gemm_fp8_autoscale")
 
 
 def _check_device_tensor(t: torch.Tensor, name: str) -> None:
@@ -284,6 +308,10 @@ def cascaded_lowp_matmul_prepared(a_list, w_list, *, outs=None, biases=None, pro
     pc = arr(*[t.data_ptr() for t in outs])
     pbias = arr(*[(None if bb is None else bb.data_ptr()) for bb in biases]) if biases is not None else None
     stream = torch.cuda.current_stream(dev).cuda_stream
+    if w0.fmt == _lib.FMT_FP8 and n == 1 and not w0.glu and adt == torch.float32 and variant < 0:
+        _gemm_fp8_autoscale(a2s[0], w0.slots.data_ptr(), True, outs[0], None if biases is None else biases[0], M, N, K,
+                            lda, N, max(NO, 1), w0.terms, _lib.PROD_BY_NAME[products], w0.exp)
+        return [outs[0].reshape(*a_list[0].shape[:-1], NO)]
     exps = None
     if w0.fmt == _lib.FMT_FP8:
         exps = torch.empty(2 * n, dtype=torch.int32, device=dev)
@@ -328,6 +356,10 @@ def _gemm_2d(a2: torch.Tensor, b2: torch.Tensor, out2: torch.Tensor, bias: Optio
         if tensor_exps.dtype != torch.int32 or tensor_exps.numel() != 2 or not tensor_exps.is_cuda:
             raise ValueError("tensor_exps must be a device int32 tensor {e_A, e_B}")
         exps = tensor_exps.contiguous()
+    elif fmt == _lib.FMT_FP8 and b_exp is not None and variant < 0 and a2.dtype == torch.float32:
+        _gemm_fp8_autoscale(a2, b2.data_ptr(), False, out2, bias, M, N, K, a2.stride(0) if M > 1 else max(K, 1),
+                            b2.stride(0) if K > 1 else max(N, 1), out2.stride(0) if M > 1 else max(N, 1), terms, products, b_exp)
+        return
     elif fmt == _lib.FMT_FP8:
         exps = torch.empty(2, dtype=torch.int32, device=a2.device)
         _activation_exps(a2, a2.stride(0) if M > 1 else max(K, 1), b_exp, exps.data_ptr(), stream)

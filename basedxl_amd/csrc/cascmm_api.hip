@@ -211,10 +211,11 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
   if (v.kind == KIND_F8K64) {
     // stages of 64 k at ~2.1 us per resident round, the K split the launcher will use, and the passes
     // around the GEMM: the split of A (and of B unless prepared), the reduction of a K split
-    const int sp = f8k64_splits(q.M, q.N, q.K);
+    const int sp = f8k64_splits(q.M, q.N, q.K, v.BM);
     const double items = tiles * sp;
     const double rounds_ = items <= kNumCUs ? 1.0 : (double)(int64_t)(items / kNumCUs) + ((int64_t)items % kNumCUs ? 0.8 : 0.0);
-    double us = rounds_ * ((double)(q.K / 64 / sp) * 2.1 + 6.0) + 6.0 + (double)q.M * q.K * 7.0 / 4.0e6;
+    double us = rounds_ * ((double)(q.K / 64 / sp) * f8k64_stage_us(v.BM) + (v.BM == 256 ? 6.0 : 4.0)) + 6.0 +
+                (double)q.M * q.K * 7.0 / 4.0e6;
     if (!q.bpre) us += 3.0 + (double)q.K * q.N * 7.0 / 4.0e6;
     if (sp > 1) us += 3.0 + (double)(sp + 1) * q.M * q.N * 4.0 / 4.0e6;
     return us;
@@ -333,7 +334,7 @@ static int select_variant_uncached(const Problem& q, bool fast, int count, size_
     if (t[i].kind == KIND_SPLITK &&
         skinny_workspace_bytes(q.M, q.N, q.K, t[i].BM, t[i].BN, t[i].BK) > ws_bytes)
       continue;
-    if (t[i].kind == KIND_F8K64 && f8k64_workspace_bytes(q.M, q.N, q.K, q.bpre) > ws_bytes) continue;
+    if (t[i].kind == KIND_F8K64 && f8k64_workspace_bytes(q.M, q.N, q.K, q.bpre, t[i].BM) > ws_bytes) continue;
     int sp = 1;
     const double c = variant_cost(i, q, count, ws_bytes, &sp);
     if (best < 0 || c < best_cost) {
@@ -361,63 +362,6 @@ __global__ void fill_bias_kernel(void* C, const void* bias, int M, int N, int64_
 // pattern of max|x| (non-negative floats order like their bit patterns), turn it into the
 // exponent e with max|x| * 2^e in (224, 448]
 __global__ void amax_begin_kernel(int32_t* exp_out) { *exp_out = 0; }
-
-// bit pattern of max|x| over the elements this thread visits, reduced over its wave
-template <int IODT>
-__device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64_t cols, int64_t ld) {
-  typedef typename IoType<IODT>::T T;
-  const T* src = (const T*)x;
-  unsigned best = 0;
-  auto fold = [&](float v) {
-    const unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7FFFFFFFu;
-    best = bits > best ? bits : best;
-  };
-  if (ld == cols) {
-    // contiguous: one flat range, 16-byte loads where the element type and alignment allow
-    const int64_t total = rows * cols;
-    if (IODT == CASCMM_DT_F32 && ((uintptr_t)x % 16) == 0) {
-      const int64_t quads = total / 4;
-      const int64_t step = (int64_t)gridDim.x * blockDim.x;
-      int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-      // four independent loads in flight per thread
-      for (; i + 3 * step < quads; i += 4 * step) {
-        f32x4 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = ((const f32x4*)x)[i + u * step];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) { fold(v[u][0]); fold(v[u][1]); fold(v[u][2]); fold(v[u][3]); }
-      }
-      for (; i < quads; i += step) {
-        const f32x4 v = ((const f32x4*)x)[i];
-        fold(v[0]); fold(v[1]); fold(v[2]); fold(v[3]);
-      }
-      if (blockIdx.x == 0 && threadIdx.x < total - quads * 4) fold(IoType<IODT>::load(src + quads * 4 + threadIdx.x));
-    } else {
-      for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x)
-        fold(IoType<IODT>::load(src + i));
-    }
-  } else {
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x)
-      for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) fold(IoType<IODT>::load(src + r * ld + c));
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    const unsigned other = (unsigned)__shfl_xor((int)best, off, 64);
-    best = other > best ? other : best;
-  }
-  return best;
-}
-
-// the exponent e with max|x| * 2^e in (224, 448], from the bit pattern of max|x|
-__device__ __forceinline__ int exp_of_amax(unsigned bits) {
-  int e = 0;
-  if (bits != 0 && bits < 0x7F800000u) {   // finite and non-zero
-    int ex;
-    const float m = frexpf(__builtin_bit_cast(float, bits), &ex);   // m in [0.5, 1)
-    e = m <= 0.875f ? 9 - ex : 8 - ex;                              // 448 = 0.875 * 2^9
-  }
-  return e;
-}
 
 template <int IODT>
 __global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t rows, int64_t cols, int64_t ld, int32_t* exp_out) {
@@ -555,9 +499,11 @@ static bool onthefly_prepare_ok(const Problem& q, int count, const void* const* 
 }
 
 // One launch for `count` problems of one shape (count == 1: a plain GEMM).
+// exps_dyn (fp8-rate kernel only, count == 1): the launch finds the left operand's scale exponent
+// itself and leaves {e_A, *b_exp_src} there; CASCMM_ERR_BAD_VARIANT when another kernel is selected.
 static int gemm_impl(int count, const void* const* A, const void* const* B, void* const* C, const void* const* bias,
                      const Problem& q, const int32_t* tensor_exps, void* workspace, size_t workspace_bytes,
-                     hipStream_t stream, int variant) {
+                     hipStream_t stream, int variant, int32_t* exps_dyn = nullptr, const int32_t* b_exp_src = nullptr) {
   int st = check_problem(q);
   if (st != CASCMM_OK) return st;
   if (count < 1 || count > kMaxGroup) return CASCMM_ERR_BAD_SHAPE;
@@ -644,6 +590,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
     if (!variant_matches(t[variant], q, fast)) return CASCMM_ERR_BAD_VARIANT;
   }
   const VariantDesc& v = t[variant];
+  if (exps_dyn && (v.kind != KIND_F8K64 || count != 1)) return CASCMM_ERR_BAD_VARIANT;
   if (count > 1 && !v.grouped) {
     // a forced kernel that runs one problem per launch: one launch each, in order on the stream
     if (v.kind == KIND_SPLITK) return CASCMM_ERR_BAD_VARIANT;
@@ -668,6 +615,8 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   p.k_splits = v.kind == KIND_TILE ? splits : 1;
   p.tensor_exps = q.fmt == CASCMM_FMT_FP8 ? tensor_exps : nullptr;
   p.glu = q.glu ? 1 : 0;
+  p.exps_dyn = exps_dyn;
+  p.b_exp_src = b_exp_src;
   for (int i = 0; i < count; ++i) {
     p.A[i] = A[i]; p.B[i] = B[i]; p.C[i] = C[i]; p.bias[i] = bias ? bias[i] : nullptr;
   }
@@ -719,7 +668,7 @@ int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
     int splits = 1;
     int v = select_variant(q, fast_ok(q, A, B), 1, (size_t)-1, &splits);
     if (v < 0) return v;
-    if (table()[v].kind == KIND_F8K64 && f8k64_workspace_bytes(M, N, K, false) > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) {
+    if (table()[v].kind == KIND_F8K64 && f8k64_workspace_bytes(M, N, K, false, table()[v].BM) > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) {
       // the fp8-rate kernel is a choice, not a need: without room for its operand slots the choice is
       // made among the kernels that split inside the GEMM
       v = select_variant(q, fast_ok(q, A, B), 1, (size_t)CASCMM_NOALLOC_SCRATCH_BYTES, &splits);
@@ -727,7 +676,7 @@ int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
     }
     const VariantDesc& d = table()[v];
     if (d.kind == KIND_SPLITK) need = skinny_workspace_bytes(M, N, K, d.BM, d.BN, d.BK);
-    else if (d.kind == KIND_F8K64) need = f8k64_workspace_bytes(M, N, K, false);
+    else if (d.kind == KIND_F8K64) need = f8k64_workspace_bytes(M, N, K, false, d.BM);
     else if (splits > 1) need = (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
   }
   if (need > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) return CASCMM_ERR_SCRATCH_LIMIT;
@@ -851,7 +800,7 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
   // three fp8 terms on the fp8-rate kernel: the operand slots of A and B
   for (const auto& v : table()) {
     if (v.kind != KIND_F8K64 || v.bpre || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
-    const size_t n = f8k64_workspace_bytes(M, N, K, false);
+    const size_t n = f8k64_workspace_bytes(M, N, K, false, v.BM);
     need = n > need ? n : need;
   }
   // 16-bit tensors as one term of their own format: room for B re-laid as operand slots
@@ -945,6 +894,37 @@ int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, in
     CASCMM_LAUNCH(err, (amax_single_launch_kernel<CASCMM_DT_BF16>), dim3(grid), dim3(1024), 0, s, x, rows, cols, ld, second_exp,
                        exps_out, (unsigned*)scratch);
   return err == hipSuccess ? CASCMM_OK : CASCMM_ERR_LAUNCH;
+}
+
+int cascmm_gemm_fp8_autoscale(const void* A, const void* B, int b_prepared, void* C, const void* bias, int64_t M, int64_t N,
+                              int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int terms, int products, const int32_t* b_exp,
+                              int32_t* exps_out, int32_t* scratch, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!exps_out || !scratch) return CASCMM_ERR_NULL_POINTER;
+  Problem q{M, N, K, lda, b_prepared ? N : ldb, ldc, CASCMM_DT_F32, CASCMM_FMT_FP8, terms, products};
+  q.bpre = b_prepared != 0;
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  const void* bias1 = bias;
+  if (M > 0 && N > 0 && K > 0 && A && B) {
+    // the fp8-rate kernel splits A in a pass of its own anyway: the search rides on it
+    const bool fast = fast_ok(q, A, q.bpre ? nullptr : B);
+    if (!q.bpre || fast) {
+      const int v = select_variant(q, fast, 1, workspace ? workspace_bytes : 0);
+      if (v >= 0 && table()[v].kind == KIND_F8K64)
+        return gemm_impl(1, &A, &B, &C, bias ? &bias1 : nullptr, q, nullptr, workspace, workspace_bytes, (hipStream_t)stream, v,
+                         exps_out, b_exp);
+    }
+  }
+  // any other kernel: the one-launch search, then the GEMM with its result
+  const int se = cascmm_tensor_exps(A, M, K, lda, CASCMM_DT_F32, b_exp, exps_out, scratch, stream);
+  if (se != CASCMM_OK) return se;
+  if (!b_exp) {
+    // (exps_out[1] must be defined: a NULL b_exp means e_B = 0)
+    hipError_t err = hipSuccess;
+    CASCMM_LAUNCH(err, amax_begin_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, exps_out + 1);
+    if (err != hipSuccess) return CASCMM_ERR_LAUNCH;
+  }
+  return gemm_impl(1, &A, &B, &C, bias ? &bias1 : nullptr, q, exps_out, workspace, workspace_bytes, (hipStream_t)stream, -1);
 }
 
 int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms, int tensor_exp,

@@ -224,6 +224,66 @@ template <int FMT, int TERMS, bool FULL> struct AccClasses {
   static constexpr int kChunkK = 256;
 };
 
+// ---------------------------------------------------------------------------------------
+// fp8 tensor scale: max|x| as a bit pattern (non-negative floats order like their bit patterns)
+// ---------------------------------------------------------------------------------------
+// bit pattern of max|x| over the elements this thread visits, reduced over its wave
+template <int IODT>
+__device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64_t cols, int64_t ld) {
+  typedef typename IoType<IODT>::T T;
+  const T* src = (const T*)x;
+  unsigned best = 0;
+  auto fold = [&](float v) {
+    const unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7FFFFFFFu;
+    best = bits > best ? bits : best;
+  };
+  if (ld == cols) {
+    // contiguous: one flat range, 16-byte loads where the element type and alignment allow
+    const int64_t total = rows * cols;
+    if (IODT == CASCMM_DT_F32 && ((uintptr_t)x % 16) == 0) {
+      const int64_t quads = total / 4;
+      const int64_t step = (int64_t)gridDim.x * blockDim.x;
+      int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+      // four independent loads in flight per thread
+      for (; i + 3 * step < quads; i += 4 * step) {
+        f32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = ((const f32x4*)x)[i + u * step];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { fold(v[u][0]); fold(v[u][1]); fold(v[u][2]); fold(v[u][3]); }
+      }
+      for (; i < quads; i += step) {
+        const f32x4 v = ((const f32x4*)x)[i];
+        fold(v[0]); fold(v[1]); fold(v[2]); fold(v[3]);
+      }
+      if (blockIdx.x == 0 && threadIdx.x < total - quads * 4) fold(IoType<IODT>::load(src + quads * 4 + threadIdx.x));
+    } else {
+      for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x)
+        fold(IoType<IODT>::load(src + i));
+    }
+  } else {
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x)
+      for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) fold(IoType<IODT>::load(src + r * ld + c));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned other = (unsigned)__shfl_xor((int)best, off, 64);
+    best = other > best ? other : best;
+  }
+  return best;
+}
+
+// the exponent e with max|x| * 2^e in (224, 448], from the bit pattern of max|x|
+__device__ __forceinline__ int exp_of_amax(unsigned bits) {
+  int e = 0;
+  if (bits != 0 && bits < 0x7F800000u) {   // finite and non-zero
+    int ex;
+    const float m = frexpf(__builtin_bit_cast(float, bits), &ex);   // m in [0.5, 1)
+    e = m <= 0.875f ? 9 - ex : 8 - ex;                              // 448 = 0.875 * 2^9
+  }
+  return e;
+}
+
 struct GemmParams {
   const void* A;
   const void* B;
@@ -258,6 +318,11 @@ struct GroupParams {
   // "gate" columns; C has N/2 columns, C[m][32 j + l] = (h[m][64 j + l] + bias[32 j + l]) *
   // gelu(h[m][64 j + 32 + l] + bias[N/2 + 32 j + l]) with h = A x B.
   int glu;
+  // fp8-rate kernel only: the left operand's scale exponent is found inside the launch (two kernels:
+  // per-workgroup maxima, then the operand split reduces them) and written, with *b_exp_src, to
+  // exps_dyn[0..1], which the GEMM then reads instead of tensor_exps
+  int32_t* exps_dyn;
+  const int32_t* b_exp_src;
 };
 
 }  // namespace cascmm

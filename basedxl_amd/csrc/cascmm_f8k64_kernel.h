@@ -25,6 +25,11 @@
 // the gaps (unconditionally: past the last stage the last one is fetched again).  The barrier sits in
 // front of a stage's last column block, whose fragments are already in registers, so the first
 // fragments of the next stage are read behind that block's MFMAs.
+// A second instantiation has half the rows (tile 128 x 160, wave tile 32 x 160, 30 MFMAs per stage):
+// twice the tiles for problems that would otherwise leave CUs idle or need their K split over
+// workgroups (and its partial results written out and added by a second kernel).  Its stages are too
+// short to spread the loads: all loads of stage s + 2 are issued right behind the barrier that frees
+// their buffer, a whole stage before they are needed.
 #pragma once
 #include <type_traits>
 
@@ -32,35 +37,80 @@
 
 namespace cascmm {
 
-struct F8K64 {
-  static constexpr int BM = 256, BN = 160, BK = 64, NT = 256, TERMS = 3;
-  static constexpr int WTM = 64, MT = 2, NTL = 5;
+template <int MT_>
+struct F8K64T {
+  static constexpr int MT = MT_, NTL = 5;                  // 32 x 32 accumulator blocks of a wave: MT x NTL
+  static constexpr int WTM = 32 * MT, BM = 4 * WTM, BN = 160, BK = 64, NT = 256, TERMS = 3;
   static constexpr int KU = BK / 16;                       // 16-k slot columns per stage
-  static constexpr int A_STAGE = TERMS * KU * BM * 16;     // 48 KB
+  static constexpr int A_STAGE = TERMS * KU * BM * 16;     // 48 KB (24 KB)
   static constexpr int B_STAGE = TERMS * KU * BN * 16;     // 30 KB
-  static constexpr int STAGE = A_STAGE + B_STAGE;          // 78 KB
-  static constexpr int LDS_BYTES = 2 * STAGE;              // 156 KB
-  static constexpr int A_LOADS = TERMS * KU;               // per wave: its own 64 rows
+  static constexpr int STAGE = A_STAGE + B_STAGE;          // 78 KB (54 KB)
+  static constexpr int LDS_BYTES = 2 * STAGE;              // 156 KB (108 KB)
+  static constexpr int A_LOADS = TERMS * KU * BM / 64 / 4; // per wave: the stage's runs of 64 rows, dealt round robin
   static constexpr int B_SLOTS = TERMS * KU * BN;          // 1920 = 30 x 64
   static constexpr int B_LOADS_MAX = 8;                    // 30 instructions over 4 waves: 8, 8, 7, 7
+  static constexpr int LOADS = A_LOADS + B_LOADS_MAX;      // 20 (14)
+  static constexpr int GB = 6 * MT;                        // MFMAs (and the gaps behind them) per column block
 };
+typedef F8K64T<2> F8K64;   // the 256 x 160 tile; what is common to both (BN, BK, slot layout) is read from it
 
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // bytes of the slots of an operand with `rows` rows (columns) and K (multiple of 16) deep
 inline __host__ __device__ int64_t f8k64_slot_bytes(int64_t rows, int64_t K) { return (int64_t)F8K64::TERMS * (K / 16) * rows * 16; }
 
+// max|a| of this workgroup's share of A [M, K] (bit pattern) -> amax_out[blockIdx.x]; no atomics, no
+// meeting point: the kernel that splits A reduces the gridDim.x values.
+template <int UNUSED>
+__global__ __launch_bounds__(1024) void f8k64_amax_kernel(const float* __restrict__ A, int64_t M, int64_t K, int64_t lda,
+                                                         unsigned* __restrict__ amax_out) {
+  __shared__ unsigned wave_best[16];
+  const unsigned best = amax_scan<CASCMM_DT_F32>(A, M, K, lda);
+  if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  unsigned b = 0;
+  for (unsigned w = 0; w < (blockDim.x >> 6); ++w) b = wave_best[w] > b ? wave_best[w] : b;
+  amax_out[blockIdx.x] = b;
+}
+
 // Split of the LEFT operand: A [M, K] fp32 row-major -> slots[term][K/16][M].  A workgroup converts
 // 64 rows x 64 k (a thread: 16 consecutive k of a row) and transposes through LDS so that the slots
 // leave as 1 KB runs along M.
+// The scale exponent is *tensor_exp (NULL: 0), or, when `amax` is given, found here: amax[0 .. n_amax)
+// are the per-workgroup maxima |a| (bit patterns) of a preceding f8k64_amax_kernel; every workgroup
+// reduces them itself (1 KB from L2, behind its loads of A), and the first one leaves {e_A, *b_exp}
+// in exps_out for the GEMM.
 template <int UNUSED>
 __global__ __launch_bounds__(256) void f8k64_split_rows_kernel(const float* __restrict__ A, int M, int K, int64_t lda,
-                                                              const int32_t* __restrict__ tensor_exp, u32x4* __restrict__ out) {
+                                                              const int32_t* __restrict__ tensor_exp, u32x4* __restrict__ out,
+                                                              const unsigned* __restrict__ amax, int n_amax,
+                                                              const int32_t* __restrict__ b_exp, int32_t* __restrict__ exps_out) {
   __shared__ u32x4 slots[3][4][64];
+  __shared__ int e_found;
   const int kus = K >> 4;
   const int ku_tiles = (kus + 3) >> 2;
   const int m0 = (blockIdx.x / ku_tiles) * 64, ku0 = (blockIdx.x % ku_tiles) * 4;
-  const float scale = tensor_exp ? __builtin_ldexpf(1.f, *tensor_exp) : 1.f;
+  int e = tensor_exp ? *tensor_exp : 0;
+  if (amax) {   // (uniform over the grid)
+    if (threadIdx.x < 64) {
+      unsigned best = 0;
+      for (int i = threadIdx.x; i < n_amax; i += 64) best = amax[i] > best ? amax[i] : best;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const unsigned other = (unsigned)__shfl_xor((int)best, off, 64);
+        best = other > best ? other : best;
+      }
+      if (threadIdx.x == 0) e_found = exp_of_amax(best);
+    }
+    __syncthreads();
+    e = e_found;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      exps_out[0] = e;
+      exps_out[1] = b_exp ? *b_exp : 0;
+    }
+  }
+  const float scale = __builtin_ldexpf(1.f, e);
   {
     const int row = threadIdx.x >> 2, ku = threadIdx.x & 3;
     if (m0 + row < M && ku0 + ku < kus) {
@@ -133,11 +183,18 @@ struct F8K64Params {
 
 typedef __attribute__((address_space(3))) void* f8k64_lds_ptr;
 
+// 64 lanes x 16 bytes from a buffer straight into LDS at dst + 16 lane.  (A function of its own: in a
+// call whose arguments depend on a template parameter the host pass of the compiler rejects the
+// builtin without a message and then leaves out the kernel's launch stub.)
+__device__ __forceinline__ void f8k64_load_lds(__amdgpu_buffer_rsrc_t rsrc, unsigned char* dst, int voffset, int soffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (f8k64_lds_ptr)dst, 16, voffset, soffset, 0, 0);
+}
+
 // Host-checked: K % 64 == 0, the slot buffers below 2 GiB, C rows addressable with 32-bit byte offsets
-// inside a tile.
-template <int UNUSED>
-__global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_f8k64_kernel(const F8K64Params p) {
-  typedef F8K64 T;
+// inside a tile.  MT = 2: 256 x 160 tile, MT = 1: 128 x 160.
+template <int MT>
+__global__ __launch_bounds__(F8K64T<MT>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_f8k64_kernel(const F8K64Params p) {
+  typedef F8K64T<MT> T;
   extern __shared__ __attribute__((aligned(1024))) unsigned char f8k64_smem[];
   unsigned char* smem = f8k64_smem;
   const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, h = lane >> 5;
@@ -154,12 +211,21 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.a_slots, 0, 0x7FFFFFFF, 0x00020000);
   const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.b_slots, 0, 0x7FFFFFFF, 0x00020000);
-  // A: the wave's own 64 rows, one instruction per (term, ku); lane = row (clamped to the last valid one)
-  int a_row = m0 + wm0 + lane;
-  a_row = a_row < p.M ? a_row : p.M - 1;
-  const int a_voff = a_row * 16;
+  // A: a stage holds, per (term, ku), BM slots = BM / 64 runs of 64 rows, run r at byte r * 1024; this
+  // wave loads runs wave, wave + 4, ...; lane = row inside the run (clamped to the last valid row)
   const int a_plane = kus * p.M * 16;          // bytes between terms
   const int a_ku = p.M * 16;                   // bytes between 16-k slot columns
+  constexpr int CH = T::BM / 64;               // runs per (term, ku)
+  int a_voff[T::A_LOADS], a_soff[T::A_LOADS];
+#pragma unroll
+  for (int j = 0; j < T::A_LOADS; ++j) {
+    const int run = wave + 4 * j;
+    const int tk = run / CH, chunk = run % CH;           // tk = term * KU + ku
+    int row = m0 + chunk * 64 + lane;
+    row = row < p.M ? row : p.M - 1;
+    a_voff[j] = row * 16;
+    a_soff[j] = (tk / T::KU) * a_plane + (tk % T::KU) * a_ku;
+  }
   // B: the stage's 1920 slots as 30 runs of 64; this wave takes runs wave, wave + 4, ...
   int b_voff[T::B_LOADS_MAX], b_lds[T::B_LOADS_MAX];
 #pragma unroll
@@ -174,15 +240,13 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     b_voff[j] = ((term * kus + ku) * p.N + col) * 16;
   }
   const int b_step = T::KU * p.N * 16;         // bytes per stage
-  auto issue_a = [&](int step_, int j) {      // j = term * 4 + ku
+  auto issue_a = [&](int step_, int j) {
     const int step = step0 + (step_ < ksteps - 1 ? step_ : ksteps - 1);
-    const int term = j >> 2, ku = j & 3;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (f8k64_lds_ptr)(smem + (step_ & 1) * T::STAGE + (j * T::BM + wm0) * 16), 16, a_voff,
-                                             term * a_plane + (step * T::KU + ku) * a_ku, 0, 0);
+    f8k64_load_lds(ra, smem + (step_ & 1) * T::STAGE + (wave + 4 * j) * 1024, a_voff[j], a_soff[j] + step * T::KU * a_ku);
   };
   auto issue_b = [&](int step_, int j) {
     const int step = step0 + (step_ < ksteps - 1 ? step_ : ksteps - 1);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (f8k64_lds_ptr)(smem + (step_ & 1) * T::STAGE + b_lds[j]), 16, b_voff[j], step * b_step, 0, 0);
+    f8k64_load_lds(rb, smem + (step_ & 1) * T::STAGE + b_lds[j], b_voff[j], step * b_step);
   };
 
   // fragment addresses inside a stage: lane (row l31, k half h) reads slots (term, ku = 2 h) and (term, 2 h + 1)
@@ -199,7 +263,7 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
 
 #define F8K64_FENCE() __builtin_amdgcn_sched_barrier(0)
-  auto issue = [&](int step_, int k) {     // load k (0 .. 19) of a stage: 12 of A, then 8 of B
+  auto issue = [&](int step_, int k) {     // load k (0 .. LOADS - 1) of a stage: those of A, then 8 of B
     if (k < T::A_LOADS) issue_a(step_, k);
     else issue_b(step_, k - T::A_LOADS);
   };
@@ -209,9 +273,7 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   };
 
 #pragma unroll
-  for (int j = 0; j < T::A_LOADS; ++j) issue_a(0, j);
-#pragma unroll
-  for (int j = 0; j < T::B_LOADS_MAX; ++j) issue_b(0, j);
+  for (int k = 0; k < T::LOADS; ++k) issue(0, k);
 
   // Fragments: A of the whole stage (the wave's own rows), B of one column block, both double
   // buffered in registers.  The barrier that opens stage s + 1 sits in front of the LAST column block
@@ -234,8 +296,11 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     read_a(0, smem, t);
     read_b(0, smem, 0, t);
   }
+  // Loads of stage s + 1 that are issued before stage s begins (the others follow inside stage s):
+  // MT = 2: the first six; MT = 1: all of them
+  constexpr int EARLY = MT == 2 ? 6 : T::LOADS;
 #pragma unroll
-  for (int k = 0; k < 6; ++k) issue(1, k);
+  for (int k = 0; k < EARLY; ++k) issue(1, k);
 
   // ksteps is even or odd: the stage loop is unrolled by two so that the register buffers are static
   auto stage = [&](int s, auto BUF) {
@@ -247,7 +312,7 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       const int cur = (ab * T::NTL + ni) & 1, nxt = cur ^ 1;
       if (ni == T::NTL - 1) {
         // everything this wave needs of stage s is in registers: open stage s + 1
-        __builtin_amdgcn_s_waitcnt(0x0F70);     // own loads of stage s + 1 have landed (issued ~2000 cycles ago)
+        __builtin_amdgcn_s_waitcnt(0x0F70);     // own loads of stage s + 1 have landed (issued a stage ago)
         __builtin_amdgcn_s_barrier();           // everybody's; and nobody reads stage s any more
       }
       int n_issued = 0;
@@ -255,25 +320,34 @@ __global__ __launch_bounds__(F8K64::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         F8K64_FENCE();
         if (ni < T::NTL - 1) {
           if (n_issued < 3) read_b(nxt, st, ni + 1, n_issued);   // the fragments of the next column block
-          // loads 6 .. 19 of stage s + 1 (its buffer was given up at the barrier inside stage s - 1): gaps
-          // 3 .. 11 of block 0 and 3 .. 7 of block 1, which leaves them two and a half blocks to land
-          const int k = ni == 0 ? n_issued + 3 : ni == 1 ? n_issued + 12 : -1;
-          if (n_issued >= 3 && k >= 6 && k < 20) issue(s + 1, k);
-        } else {
+          if (MT == 2) {
+            // loads 6 .. 19 of stage s + 1 (its buffer was given up at the barrier inside stage s - 1): gaps
+            // 3 .. 11 of block 0 and 3 .. 7 of block 1, which leaves them two and a half blocks to land
+            const int k = ni == 0 ? n_issued + 3 : ni == 1 ? n_issued + 12 : -1;
+            if (n_issued >= 3 && k >= 6 && k < T::LOADS) issue(s + 1, k);
+          }
+        } else if (MT == 2) {
           // behind the last block: the first fragments of stage s + 1, then loads 0 .. 5 of stage s + 2
           if (n_issued < 3) read_b(nxt, st_next, 0, n_issued);
           else if (n_issued < 6) read_a(ab ^ 1, st_next, n_issued - 3);
           else issue(s + 2, n_issued - 6);
+        } else {
+          // six gaps: a fragment read and up to three loads of stage s + 2 in each (all fourteen)
+          if (n_issued < 3) read_b(nxt, st_next, 0, n_issued);
+          else read_a(ab ^ 1, st_next, n_issued - 3);
+#pragma unroll
+          for (int u = 0; u < 3; ++u)
+            if (n_issued * 3 + u < T::LOADS) issue(s + 2, n_issued * 3 + u);
         }
         F8K64_FENCE();
         ++n_issued;
       };
       // (the term numbers are the instruction's op_sel fields: literals)
 #define F8K64_PRODUCT(I, J)                                                                                                              \
-  acc[0][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[ab][I][0], b[cur][J], acc[0][ni], 0, 0, I, scales, J, scales);          \
-  gap();                                                                                                                                 \
-  acc[1][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[ab][I][1], b[cur][J], acc[1][ni], 0, 0, I, scales, J, scales);          \
-  gap();
+  _Pragma("unroll") for (int mi = 0; mi < T::MT; ++mi) {                                                                                 \
+    acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[ab][I][mi], b[cur][J], acc[mi][ni], 0, 0, I, scales, J, scales);     \
+    gap();                                                                                                                               \
+  }
       F8K64_PRODUCT(0, 2)
       F8K64_PRODUCT(1, 1)
       F8K64_PRODUCT(2, 0)

@@ -231,16 +231,18 @@ int launch_wavek(const GroupParams& p, hipStream_t stream) {
   return CASCMM_OK;
 }
 
-// K split of the fp8-rate kernel for problems with fewer tiles than CUs: the split count that
-// minimises stages-per-workgroup x 2.1 us + the round trip of the partial results at ~4 TB/s
-inline int f8k64_splits(int64_t M, int64_t N, int64_t K) {
-  const int64_t tiles = ((M + F8K64::BM - 1) / F8K64::BM) * ((N + F8K64::BN - 1) / F8K64::BN);
+// K split of the fp8-rate kernel (row tile bm = 256 or 128) for problems with fewer tiles than CUs:
+// the split count that minimises stages-per-workgroup x the stage time + the round trip of the
+// partial results at ~4 TB/s
+inline double f8k64_stage_us(int bm) { return bm == 256 ? 2.1 : 1.15; }
+inline int f8k64_splits(int64_t M, int64_t N, int64_t K, int bm) {
+  const int64_t tiles = ((M + bm - 1) / bm) * ((N + F8K64::BN - 1) / F8K64::BN);
   const int64_t steps = K / F8K64::BK;
   int best = 1;
-  double best_us = (double)steps * 2.1;
+  double best_us = (double)steps * f8k64_stage_us(bm);
   for (int sp = 2; sp <= 16; ++sp) {
     if (steps % sp != 0 || tiles * sp > kNumCUs) continue;
-    const double us = (double)(steps / sp) * 2.1 + 3.0 + (double)(sp + 1) * (double)M * (double)N * 4.0 / 4.0e6;
+    const double us = (double)(steps / sp) * f8k64_stage_us(bm) + 3.0 + (double)(sp + 1) * (double)M * (double)N * 4.0 / 4.0e6;
     if (us < best_us) {
       best_us = us;
       best = sp;
@@ -249,25 +251,27 @@ inline int f8k64_splits(int64_t M, int64_t N, int64_t K) {
   return best;
 }
 
-// Workspace of the fp8-rate kernel: the slots of A, those of B unless B comes prepared, and the
-// partial results of a K split (each rounded up to 256 bytes so that the next buffer stays aligned)
+// Workspace of the fp8-rate kernel: the slots of A, those of B unless B comes prepared, the partial
+// results of a K split (each rounded up to 256 bytes so that the next buffer stays aligned), and the
+// per-workgroup maxima of a scale search done inside the launch
+constexpr int kF8K64AmaxGroups = 256;
 inline size_t f8k64_up(int64_t b) { return (size_t)((b + 255) / 256 * 256); }
-inline size_t f8k64_workspace_bytes(int64_t M, int64_t N, int64_t K, bool bpre) {
-  const int sp = f8k64_splits(M, N, K);
+inline size_t f8k64_workspace_bytes(int64_t M, int64_t N, int64_t K, bool bpre, int bm) {
+  const int sp = f8k64_splits(M, N, K, bm);
   return f8k64_up(f8k64_slot_bytes(M, K)) + (bpre ? 0 : f8k64_up(f8k64_slot_bytes(N, K))) +
-         (sp > 1 ? f8k64_up((int64_t)sp * M * N * 4) : 0);
+         (sp > 1 ? f8k64_up((int64_t)sp * M * N * 4) : 0) + kF8K64AmaxGroups * sizeof(unsigned);
 }
 
 // the fp8-rate kernel: split A (and B) into operand slots, then the GEMM on the slots
-template <bool BPRE>
+template <bool BPRE, int MT>
 int launch_f8k64(const GroupParams& p, hipStream_t stream) {
-  typedef F8K64 T;
+  typedef F8K64T<MT> T;
   if (p.count != 1 || p.glu || p.k_splits > 1 || p.K % T::BK != 0 || p.K == 0) return CASCMM_ERR_BAD_VARIANT;
-  const size_t need = f8k64_workspace_bytes(p.M, p.N, p.K, BPRE);
+  const size_t need = f8k64_workspace_bytes(p.M, p.N, p.K, BPRE, T::BM);
   if (!p.workspace || p.workspace_bytes < need) return CASCMM_ERR_WORKSPACE;
   if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
   if (f8k64_slot_bytes(p.M, p.K) > 0x7FFFFFFF || f8k64_slot_bytes(p.N, p.K) > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
-  auto kfn = cascmm_f8k64_kernel<0>;
+  auto kfn = cascmm_f8k64_kernel<MT>;
   static bool lds_set[kMaxDevices] = {false};
   const int d = device_index();
   if (d < 0) return CASCMM_ERR_LAUNCH;
@@ -281,24 +285,41 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   char* ws_next = (char*)p.workspace + f8k64_up(f8k64_slot_bytes(p.M, p.K));
   const int kus = p.K >> 4;
   const unsigned a_grid = (unsigned)(((p.M + 63) / 64) * ((kus + 3) / 4));
+  const int32_t* exps = p.tensor_exps;
+  const int32_t* b_exp = p.tensor_exps ? p.tensor_exps + 1 : (const int32_t*)nullptr;
+  const unsigned* amax = nullptr;
+  int n_amax = 0;
+  if (p.exps_dyn) {
+    // the scale of A is not known yet: per-workgroup maxima now, reduced by the split of A, which
+    // leaves {e_A, e_B} in exps_dyn for the GEMM (no atomics, no pass of its own for the reduction)
+    unsigned* am = (unsigned*)((char*)p.workspace + need - kF8K64AmaxGroups * sizeof(unsigned));
+    const int64_t total = (int64_t)p.M * p.K;
+    n_amax = (int)std::max<int64_t>(1, std::min<int64_t>((total + 8191) / 8192, kF8K64AmaxGroups));
+    if (launch_kernel(f8k64_amax_kernel<0>, dim3((unsigned)n_amax), dim3(1024), 0, stream, (const float*)p.A[0], (int64_t)p.M,
+                      (int64_t)p.K, p.lda, am) != hipSuccess)
+      return CASCMM_ERR_LAUNCH;
+    amax = am;
+    exps = p.exps_dyn;
+    b_exp = p.b_exp_src;
+  }
   if (launch_kernel(f8k64_split_rows_kernel<0>, dim3(a_grid), dim3(256), 0, stream, (const float*)p.A[0], p.M, p.K, p.lda,
-                    p.tensor_exps, a_slots) != hipSuccess)
+                    p.exps_dyn ? (const int32_t*)nullptr : p.tensor_exps, a_slots, amax, n_amax, b_exp, p.exps_dyn) != hipSuccess)
     return CASCMM_ERR_LAUNCH;
   if (!BPRE) {
     u32x4* bs = (u32x4*)ws_next;
     ws_next += f8k64_up(f8k64_slot_bytes(p.N, p.K));
     const int64_t units = (int64_t)kus * p.N;
     if (launch_kernel(f8k64_split_cols_kernel<0>, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, stream, (const float*)p.B[0],
-                      p.K, p.N, p.ldb, p.tensor_exps ? p.tensor_exps + 1 : (const int32_t*)nullptr, bs) != hipSuccess)
+                      p.K, p.N, p.ldb, b_exp, bs) != hipSuccess)
       return CASCMM_ERR_LAUNCH;
     b_slots = bs;
   }
   F8K64Params q;
   q.a_slots = a_slots; q.b_slots = b_slots; q.C = (float*)p.C[0]; q.bias = (const float*)p.bias[0];
-  q.tensor_exps = p.tensor_exps;
+  q.tensor_exps = exps;
   q.M = p.M; q.N = p.N; q.K = p.K; q.ldc = p.ldc;
   q.tiles_m = (p.M + T::BM - 1) / T::BM; q.tiles_n = (p.N + T::BN - 1) / T::BN;
-  q.k_splits = f8k64_splits(p.M, p.N, p.K);
+  q.k_splits = f8k64_splits(p.M, p.N, p.K, T::BM);
   q.partials = (float*)ws_next;
   const unsigned grid = (unsigned)(q.tiles_m * q.tiles_n * q.k_splits);
   if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q) != hipSuccess) return CASCMM_ERR_LAUNCH;
@@ -313,9 +334,9 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   return CASCMM_OK;
 }
 
-#define CASCMM_F8K64_VARIANT(NAME, BPRE)                                                                                  \
-  {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8K64::BM, F8K64::BN, F8K64::BK, F8K64::NT, F8K64::LDS_BYTES, \
-   true, false, &launch_f8k64<BPRE>, BPRE}
+#define CASCMM_F8K64_VARIANT(NAME, BPRE, MT)                                                                                  \
+  {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8K64T<MT>::BM, F8K64T<MT>::BN, F8K64T<MT>::BK, F8K64T<MT>::NT, \
+   F8K64T<MT>::LDS_BYTES, true, false, &launch_f8k64<BPRE, MT>, BPRE}
 
 #define CASCMM_WAVEK_VARIANT(NAME, NB)                                                                                \
   {NAME, KIND_WAVEK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, WaveK<NB>::BM, WaveK<NB>::BN, WaveK<NB>::BK, WaveK<NB>::NT, \

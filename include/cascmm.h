@@ -216,6 +216,24 @@ int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int
 int cascmm_tensor_exps(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype,
                        const int32_t* second_exp, int32_t* exps_out, int32_t* scratch, void* stream);
 
+/* A three-term (or any) fp8 GEMM on fp32 tensors that finds the scale of its left operand itself:
+ * the same result, bit for bit, as cascmm_tensor_exps(A, ..., b_exp, exps_out, scratch) followed by
+ * cascmm_gemm (b_prepared == 0) or cascmm_gemm_prepared with count 1 (b_prepared != 0: B is a buffer
+ * written by cascmm_prepare_weight, ldb is ignored) with tensor_exps = exps_out, for the case every
+ * Linear layer of a model is in: activations whose scale changes from call to call times a weight
+ * whose scale e_B = *b_exp is kept (b_exp NULL: 0), the counterpart of the per-call cast of the
+ * activations at basedxl/triton/cascaded_lowp_matmul.py:101-103 next to the one-time weight
+ * preparation of basedxl/modules/lowp_linear.py:12.  exps_out (two device int32) receives
+ * {e_A, e_B}.  When the kernel that runs splits A in a pass of its own (the fp8-rate kernel:
+ * three terms, K a multiple of 64), the search costs no reduction pass: a first kernel leaves
+ * per-workgroup maxima in the workspace and the split reduces them.  Otherwise the function makes
+ * exactly the two calls named above.  scratch: as for cascmm_tensor_exps.  workspace: as for
+ * cascmm_gemm (cascmm_workspace_bytes covers it). */
+int cascmm_gemm_fp8_autoscale(const void* A, const void* B, int b_prepared, void* C, const void* bias,
+                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                              int terms, int products, const int32_t* b_exp, int32_t* exps_out,
+                              int32_t* scratch, void* workspace, size_t workspace_bytes, void* stream);
+
 /* The operand split alone (a test hook for parity of the split with the CPU oracle):
  * out is fp32 [terms][n]; term i holds lowp(r_i * 2^(tensor_exp + shift*i)) upcast to fp32
  * with r_0 = x, r_{i+1} = r_i - t_i / 2^(tensor_exp + shift*i); shift = 0 / 11 / 4 for
