@@ -199,7 +199,8 @@ def bench_kv(dev, check=True):
     return out
 
 
-def bench_unet(dev, cascades=(("bf16", 2), ("fp8", 3)), latents=(("full latent", None), ("half-latent share", 64)), forward=True):
+def bench_unet(dev, cascades=(("bf16", 2, None), ("fp8", 3, None), ("bf16", 2, True), ("fp8", 3, True)),
+               latents=(("full latent", None), ("half-latent share", 64)), forward=True):
     """cfg5: the routed layers of one UNet step.  The module tree is built on the GPU with random
     weights and patched through the config switch; one forward pass records every routed call; those
     calls are then replayed in call order on resident inputs from ONE HIP graph, so the figure is the
@@ -211,9 +212,9 @@ def bench_unet(dev, cascades=(("bf16", 2), ("fp8", 3)), latents=(("full latent",
     from basedxl_amd.utils import BasedXLConfig
 
     rows = []
-    for lowp, terms in cascades:
+    for lowp, terms, prepared in cascades:
         model = SDXLUNetSkeleton(device=dev, seed=SEED)
-        unet = BasedXLUnet(model, BasedXLConfig(fp16_acc_matmul=True, lowp=lowp, terms=terms))
+        unet = BasedXLUnet(model, BasedXLConfig(fp16_acc_matmul=True, lowp=lowp, terms=terms, prepared=prepared))
         for label, latent_rows in latents:
             inp = synthetic_inputs(model, latent=128, latent_rows=latent_rows, seed=SEED, device=dev)
             calls = routed_calls(unet, *inp)
@@ -229,7 +230,7 @@ def bench_unet(dev, cascades=(("bf16", 2), ("fp8", 3)), latents=(("full latent",
             with torch.no_grad():
                 us = _graph_time_us(path, reps=1, replays=3, spin_s=0.3)
                 fwd_ms = None
-                if forward:
+                if forward and not prepared:
                     unet(*inp)
                     torch.cuda.synchronize()
                     t0 = time.perf_counter()
@@ -238,7 +239,8 @@ def bench_unet(dev, cascades=(("bf16", 2), ("fp8", 3)), latents=(("full latent",
                     torch.cuda.synchronize()
                     fwd_ms = (time.perf_counter() - t0) * 1e3 / 2
             flops = sum(2.0 * c["M"] * c["K"] * c["N"] for c in calls)
-            rows.append({"cascade": f"{lowp}x{terms} tri", "latent": label, "routed_calls": len(calls), "distinct_shapes": len(shapes),
+            rows.append({"cascade": f"{lowp}x{terms} tri", "weights": "kept split (prepared once)" if prepared else "split in every call",
+                         "latent": label, "routed_calls": len(calls), "distinct_shapes": len(shapes),
                          "gflop_fp32_equiv": round(flops * 1e-9, 1), "linear_path_ms_per_step": round(us * 1e-3, 3),
                          "fp32_equiv_tflops": round(flops / us * 1e-6, 1),
                          "whole_forward_ms_eager": None if fwd_ms is None else round(fwd_ms, 1)})
@@ -247,8 +249,43 @@ def bench_unet(dev, cascades=(("bf16", 2), ("fp8", 3)), latents=(("full latent",
         torch.cuda.empty_cache()
     return {"workload": "cfg5: every nn.Linear and 1x1 convolution of one SDXL UNet denoising step (latent 2x4x128x128, text "
                         "context 2x77x2048, weights ~N(0,0.02)) through the patched module tree (fused to_k/to_v, bias in the "
-                        "store, fp8 activation scale found in every call, weight scales kept); one HIP graph of all routed calls",
+                        "store, fp8 activation scale found in every call, weight scales kept); one HIP graph of all routed calls; "
+                        "activations are split in every call, weights either in every call too or once (a labelled mode)",
             "configs": rows}
+
+
+def bench_sweep(dev, sizes=(256, 512, 1024, 2048, 4096, 8192)):
+    """The reference's self-benchmark (basedxl/triton/cascaded_lowp_matmul.py:204-242): square
+    problems M = N = K against the vendor GEMM.  Here: the two-term bf16 cascade on fp32 tensors
+    (three products, both operands split inside the timed kernel) next to torch.matmul on the same
+    fp32 tensors and on their bf16 roundings (one product, no split); HIP-graph replay."""
+    import torch
+    from basedxl_amd import cascaded_lowp_matmul, _lib
+
+    rows = []
+    l = _lib.lib()
+    for n in sizes:
+        g = torch.Generator(device=dev).manual_seed(SEED + n)
+        a = torch.randn(n, n, device=dev, generator=g)
+        b = torch.randn(n, n, device=dev, generator=g) * 0.02
+        a16, b16 = a.bfloat16(), b.bfloat16()
+        o, o16 = torch.empty(n, n, device=dev), torch.empty(n, n, device=dev, dtype=torch.bfloat16)
+        reps = 20 if n <= 2048 else 5
+        us = _graph_time_us(lambda: cascaded_lowp_matmul(a, b, out=o), reps=reps)
+        us32 = _graph_time_us(lambda: torch.matmul(a, b, out=o), reps=reps)
+        us16 = _graph_time_us(lambda: torch.matmul(a16, b16, out=o16), reps=reps)
+        flop = 2.0 * n ** 3
+        ref = a.double() @ b.double()
+        err = lambda x: float((x.double() - ref).norm() / ref.norm())   # noqa: E731
+        e_c, e_32, e_16 = err(cascaded_lowp_matmul(a, b)), err(torch.matmul(a, b)), err(torch.matmul(a16, b16))
+        rows.append({"n": n, "kernel": l.cascmm_variant_name(l.cascmm_select_variant(n, n, n, n, n, n, 0, 0, 2, 0)).decode(),
+                     "cascade_bf16x2_us": round(us, 2), "cascade_fp32_equiv_tflops": round(flop / us * 1e-6, 1),
+                     "cascade_mfma_tflops": round(3 * flop / us * 1e-6, 1), "cascade_rel_fro": e_c,
+                     "torch_fp32_us": round(us32, 2), "torch_fp32_tflops": round(flop / us32 * 1e-6, 1), "torch_fp32_rel_fro": e_32,
+                     "torch_bf16_us": round(us16, 2), "torch_bf16_tflops": round(flop / us16 * 1e-6, 1), "torch_bf16_rel_fro": e_16})
+        del a, b, a16, b16, o, o16, ref
+    return {"workload": "square sweep M = N = K: two-term bf16 cascade of fp32 tensors vs torch.matmul (fp32 tensors; bf16 tensors)",
+            "sizes": rows}
 
 
 def bench_eager_launch(dev):
@@ -281,10 +318,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["ffn", "attn", "kv", "unet"], default="ffn",
+    ap.add_argument("--workload", choices=["ffn", "attn", "kv", "unet", "sweep"], default="ffn",
                     help="ffn: the two GEMMs of the 32x32-stage GEGLU feed-forward block (the shape the metric is quoted on); "
                          "attn: the four 64x64-stage self-attention projections of one GPU's patch share; kv: the skinny "
-                         "cross-attention K/V projections (GB/s); unet: the Linear path of one whole UNet step")
+                         "cross-attention K/V projections (GB/s); unet: the Linear path of one whole UNet step; sweep: square "
+                         "problems 256 .. 8192 against torch.matmul")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="ffn only: leave the kv / unet / eager-launch figures out of the line (they add about a minute)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -313,7 +351,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
-    if args.workload in ("kv", "unet"):
+    if args.workload in ("kv", "unet", "sweep"):
         base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
                 "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
         if args.workload == "kv":
@@ -326,6 +364,12 @@ def main():
                                             "unit": "GB/s", "frac": worst["frac_of_8TBs"], "traffic": KV_TRAFFIC_BYTES.get(worst["N"]),
                                             "launch_us": worst["launch_us"], "algorithmic_bytes_per_launch": worst["algorithmic_bytes"]},
                                   gemms=kv["gemms"])))
+        elif args.workload == "sweep":
+            sw = bench_sweep(dev)
+            head = sw["sizes"][-1]
+            print(json.dumps(dict(base, metric="fp32-equiv TFLOP/s of the two-term bf16 cascade on square problems",
+                                  value=head["cascade_fp32_equiv_tflops"], unit="TFLOP/s", ms_per_step=round(head["cascade_bf16x2_us"] * 1e-3, 5),
+                                  config={"workload": sw["workload"], "headline": f"n = {head['n']}"}, sizes=sw["sizes"])))
         else:
             un = bench_unet(dev)
             head = un["configs"][0]

@@ -188,7 +188,7 @@ def test_fp8_gemm_that_finds_its_activation_scale_equals_the_two_calls(gpu_devic
     # the operator takes the same route (a kept weight scale, the activation scale found per call)
     via_op = cascaded_lowp_matmul(ad, w if prepared else bd, bias=bias, lowp="fp8", terms=3, b_exp=w.exp)
     assert torch.equal(via_op, outs[0])
-    if M * N * K <= 2048 * 1280 * 1280:
+    if M * N * K <= 2048 * 1280 * 1280 and M * N >= 16384:   # (an error norm over a handful of results says nothing)
         exp64 = oc.fp64_matmul(a, b) + bias.cpu().double()
         ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "fp8", 3, "tri") + bias.cpu(), exp64)
         got = oc.error_metrics(outs[0].cpu(), exp64)
