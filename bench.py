@@ -47,7 +47,7 @@ METRIC = {"ffn": "fp32-equiv TFLOP/s + % of MFMA roofline at SDXL FFN shape; rel
 # HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
 # summaries under profiles/ give the commands and the calibration); keyed by (workload, launch label).
 TRAFFIC_BYTES_PER_LAUNCH = {
-    ("ffn", "ff.net.0.proj (W1)"): 2 * 72861.5 * 1024 + 83968.0 * 1024,
+    ("ffn", "ff.net.0.proj (W1)"): 2 * 72854.0 * 1024 + 83968.0 * 1024,
     ("attn", "to_q/to_k/to_v grouped"): 2 * 21930.0 * 1024 + 30720.0 * 1024,
 }
 
@@ -157,7 +157,7 @@ def _graph_time_us(fn, reps, replays=5, spin_s=0.2):
     return e0.elapsed_time(e1) * 1e3 / (replays * reps)
 
 
-KV_TRAFFIC_BYTES = {1280: None, 640: None}   # HBM-side bytes per launch from rocprofv3 counters (see profiles/), when measured
+KV_TRAFFIC_BYTES = {1280: 21034047.0, 640: 18076444.0}   # HBM-side bytes per launch from rocprofv3 counters (see profiles/), when measured
 
 
 def bench_kv(dev, check=True):
@@ -576,35 +576,39 @@ def main():
                   "kernel_max_abs": err_k["max_abs"], "oracle_max_abs": err_o["max_abs"]},
     }
     if args.workload == "ffn" and not args.no_graph:
-        # cfg3 also names the 3-term fp16 cascade (six products): the same two GEMMs, reported beside
-        # the headline, not part of `value`
-        other = {"cascade": "fp16x3 tri", "gemms": []}
-        for i, ln in enumerate(launches):
-            a, w, o = sets[0][0][ln.a_idx[0]], sets[0][1][ln.w_idx[0]], sets[0][2][i][0]
-            cascaded_lowp_matmul(a, w, out=o, lowp="fp16", terms=3)
-            g3 = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g3):
-                for _ in range(REPS):
-                    cascaded_lowp_matmul(a, w, out=o, lowp="fp16", terms=3)
-            for _ in range(3):
-                g3.replay()
-            torch.cuda.synchronize()
-            k0, k1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            k0.record()
-            for _ in range(5):
-                g3.replay()
-            k1.record()
-            torch.cuda.synchronize()
-            us = k0.elapsed_time(k1) * 1e3 / (5 * REPS)
-            other["gemms"].append({"launch": ln.label, "launch_us": round(us, 2), "fp32_equiv_tflops": round(ln.flops / us * 1e-6, 1),
-                                   "mfma_tflops": round(6 * ln.flops / us * 1e-6, 1)})
-        exp = oc.fp64_matmul(a_chk, w_chk)
-        e3 = oc.error_metrics(sets[0][2][-1][-1].cpu(), exp)
-        e3o = oc.error_metrics(oc.cascade_matmul_ref(a_chk, w_chk, "fp16", 3, "tri"), exp)
-        del exp
-        other["error"] = {"checked_gemm": chk.label, "kernel_rel_fro": e3["rel_fro"], "oracle_rel_fro": e3o["rel_fro"],
-                          "kernel_max_abs": e3["max_abs"], "oracle_max_abs": e3o["max_abs"]}
-        result["other_cascades"] = [other]
+        # cfg3 also names the 3-term fp16 cascade, and the fp8 comparison of cfg5 starts at this shape: the
+        # same two GEMMs with six products each, reported beside the headline, not part of `value`.  fp8:
+        # both operands raw fp32, the weight's scale kept (found once, as a layer does), the activation's
+        # found inside every call; its MFMA rate is priced against the fp8 peak.
+        from basedxl_amd import tensor_scale_exp
+        others = []
+        for lowp, peak in (("fp16", PEAK_BF16_TFLOPS), ("fp8", 5000.0)):
+            other = {"cascade": f"{lowp}x3 tri", "mfma_peak_tflops": peak, "gemms": []}
+            for i, ln in enumerate(launches):
+                a, w, o = sets[0][0][ln.a_idx[0]], sets[0][1][ln.w_idx[0]], sets[0][2][i][0]
+                kw = {"b_exp": tensor_scale_exp(w)} if lowp == "fp8" else {}
+                us = _graph_time_us(lambda: cascaded_lowp_matmul(a, w, out=o, lowp=lowp, terms=3, **kw), reps=REPS, spin_s=0.05)
+                other["gemms"].append({"launch": ln.label, "launch_us": round(us, 2), "fp32_equiv_tflops": round(ln.flops / us * 1e-6, 1),
+                                       "mfma_tflops": round(6 * ln.flops / us * 1e-6, 1),
+                                       "frac_of_mfma_peak": round(6 * ln.flops / us * 1e-6 / peak, 4)})
+            exp = oc.fp64_matmul(a_chk, w_chk)
+            e3 = oc.error_metrics(sets[0][2][-1][-1].cpu(), exp)
+            e3o = oc.error_metrics(oc.cascade_matmul_ref(a_chk, w_chk, lowp, 3, "tri"), exp)
+            del exp
+            other["error"] = {"checked_gemm": chk.label, "kernel_rel_fro": e3["rel_fro"], "oracle_rel_fro": e3o["rel_fro"],
+                              "kernel_max_abs": e3["max_abs"], "oracle_max_abs": e3o["max_abs"]}
+            others.append(other)
+        result["other_cascades"] = others
+    elif args.workload == "ffn":
+        # (--no-graph is how the counter runs of a profiler are made: let them see the other cascades' kernels too)
+        from basedxl_amd import tensor_scale_exp
+        for lowp in ("fp16", "fp8"):
+            for i, ln in enumerate(launches):
+                a, w, o = sets[0][0][ln.a_idx[0]], sets[0][1][ln.w_idx[0]], sets[0][2][i][0]
+                kw = {"b_exp": tensor_scale_exp(w)} if lowp == "fp8" else {}
+                for _ in range(3):
+                    cascaded_lowp_matmul(a, w, out=o, lowp=lowp, terms=3, **kw)
+        torch.cuda.synchronize()
     if args.workload == "ffn" and not args.no_graph and not args.no_other_workloads:
         del sets, a_dev, w_dev
         torch.cuda.empty_cache()
