@@ -51,6 +51,7 @@ SIGNATURES = {
     "cascmm_gemm_fp8_autoscale": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p] + [c_int64] * 6 + [c_int, c_int]
                                   + [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "cascmm_split_terms": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
+    "cascmm_selftest": (c_int, []),
     "cascmm_strerror": (c_char_p, [c_int]),
     "cascmm_version": (c_int, []),
 }

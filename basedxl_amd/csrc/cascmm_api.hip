@@ -58,7 +58,10 @@ static bool prepared_as_k16_slots(int64_t K, int fmt, int terms, bool glu) {
 static int64_t prepared_bytes(int64_t K, int64_t N, int fmt, int terms, bool glu = false) {
   if (prepared_as_k16_slots(K, fmt, terms, glu)) return f8k64_slot_bytes(N, K);
   const int planes = fmt == CASCMM_FMT_FP8 ? (terms + 1) / 2 : terms;
-  return (int64_t)planes * ((K + 7) / 8) * N * 16;
+  int64_t slots = 0, bytes = 0;   // (saturates instead of overflowing: callers compare the result with limits)
+  if (__builtin_mul_overflow((int64_t)planes * ((K + 7) / 8), N, &slots) || __builtin_mul_overflow(slots, (int64_t)16, &bytes))
+    return INT64_MAX;
+  return bytes;
 }
 
 static int check_problem(const Problem& q) {
@@ -955,6 +958,19 @@ const char* cascmm_strerror(int status) {
     case CASCMM_ERR_SCRATCH_LIMIT: return "problem needs more scratch than the library's built-in buffer holds (use cascmm_gemm with a workspace)";
     default: return "unknown status";
   }
+}
+
+int cascmm_selftest(void) {
+  int bad = 0;
+  const auto& t = table();
+  for (const TunedCost& c : kTuned) {
+    int hits = 0;
+    for (const VariantDesc& d : t) hits += strcmp(c.name, d.name) == 0 ? 1 : 0;
+    bad += hits == 1 ? 0 : 1;
+  }
+  for (size_t i = 0; i < t.size(); ++i)
+    for (size_t j = i + 1; j < t.size(); ++j) bad += strcmp(t[i].name, t[j].name) == 0 ? 1 : 0;
+  return bad;
 }
 
 int cascmm_version(void) { return CASCMM_VERSION; }

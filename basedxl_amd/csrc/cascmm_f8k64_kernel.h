@@ -57,7 +57,13 @@ typedef F8K64T<2> F8K64;   // the 256 x 160 tile; what is common to both (BN, BK
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // bytes of the slots of an operand with `rows` rows (columns) and K (multiple of 16) deep
-inline __host__ __device__ int64_t f8k64_slot_bytes(int64_t rows, int64_t K) { return (int64_t)F8K64::TERMS * (K / 16) * rows * 16; }
+// (saturates instead of overflowing: callers compare the result with limits)
+inline __host__ __device__ int64_t f8k64_slot_bytes(int64_t rows, int64_t K) {
+  int64_t slots = 0, bytes = 0;
+  if (__builtin_mul_overflow((int64_t)F8K64::TERMS * (K / 16), rows, &slots) || __builtin_mul_overflow(slots, (int64_t)16, &bytes))
+    return INT64_MAX;
+  return bytes;
+}
 
 // max|a| of this workgroup's share of A [M, K] (bit pattern) -> amax_out[blockIdx.x]; no atomics, no
 // meeting point: the kernel that splits A reduces the gridDim.x values.

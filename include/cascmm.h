@@ -241,6 +241,12 @@ int cascmm_gemm_fp8_autoscale(const void* A, const void* B, int b_prepared, void
 int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms,
                        int tensor_exp, void* stream);
 
+/* Consistency of the library's own tables (no counterpart in the reference): the number of entries of
+ * the measured-cost table that do not name exactly one compiled kernel variant, plus the number of
+ * variant names that occur twice; 0 for a sound build.  (A cost entry whose kernel was renamed would
+ * silently leave that kernel to the analytic cost estimate.)  Host only, launches nothing. */
+int cascmm_selftest(void);
+
 const char* cascmm_strerror(int status);
 int cascmm_version(void);
 

@@ -147,3 +147,11 @@ def test_fast_kernels_are_not_chosen_when_offsets_would_overflow():
     big = l.cascmm_select_variant(4096, 32768, 32768, 32768, 32768, 32768, 0, 0, 2, 0)
     assert ok >= 0 and "generic" not in names[ok]
     assert big >= 0 and "generic" in names[big]
+
+
+def test_library_tables_are_consistent():
+    """Every entry of the measured-cost table names exactly one compiled variant (a renamed kernel
+    would otherwise fall back to the analytic estimate without a word), and no variant name repeats."""
+    assert _lib.lib().cascmm_selftest() == 0
+    names = _lib.variant_names()
+    assert len(names) == len(set(names))

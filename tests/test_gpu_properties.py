@@ -189,6 +189,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
     x = {"tile": rn(2048, 640), "ksplit": rn(1024, 5120), "skinny": rn(154, 2048), "h": rn(1024, 640).half(),
          "glu": rn(512, 640), "fp8": rn(512, 320)}
     pw, pg = PreparedWeight(w["tile"]), PreparedWeight(w["glu"], glu=True)
+    p8 = PreparedWeight(w["fp8"], lowp="fp8", terms=3)   # (holds the weight's kept scale exponent too)
 
     def run():
         return [
@@ -200,6 +201,9 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
             cascaded_lowp_matmul(x["tile"], pw),
             cascaded_lowp_matmul(x["glu"], pg),
             cascaded_lowp_matmul(x["fp8"], w["fp8"], lowp="fp8", terms=3),
+            # the activation scale found inside the call (maxima, split, GEMM: all on the stream), weight raw / kept split
+            cascaded_lowp_matmul(x["fp8"], w["fp8"], lowp="fp8", terms=3, b_exp=p8.exp),
+            cascaded_lowp_matmul(x["fp8"], p8),
         ]
 
     run()                                            # warm-up: workspaces exist before the capture
@@ -218,7 +222,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
         outs = run()
     grown = torch.cuda.memory_allocated() - before
     assert {k: v.data_ptr() for k, v in _workspaces.items()} == ws_before        # no workspace was created or replaced
-    # what the capture allocated: the eight results plus the grouped launches' other results and the
+    # what the capture allocated: the ten results plus the grouped launches' other results and the
     # two-int exponent tensor, each rounded up to the allocator's 512-byte granule -- far below the
     # 21 MB K-split workspace a capture-time allocation would add
     results = sum(o.numel() * o.element_size() for o in outs)
