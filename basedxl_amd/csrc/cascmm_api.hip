@@ -143,6 +143,7 @@ static const TunedCost kTuned[] = {
     {"t64x64x64_w2x2x1_d3_bf16x2_tri_bpre", 0.515, 2.08, 1.00, 1.00},
     {"t64x256x32_w1x4x1_d3_bf16x2_tri_bpre", 1.250, 5.89, 0.80, 0.50},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri_bpre", 2.837, 12.00, 0.60, 0.50},
+    {"t256x320x32_w512_bf16x2_tri_bpre", 5.50, 16.0, 1.00, 1.00},
 };
 
 constexpr int kMaxTileSplits = 4;

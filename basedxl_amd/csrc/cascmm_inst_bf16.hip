@@ -19,7 +19,7 @@ static const VariantDesc kTable[] = {
     // (its permuted B columns are staged in 8 x 2 blocks: every producer thread gets the same units; 3 % faster here)
     CASCMM_TILE_VARIANT_PAIRS("t256x160x32_w4x1x1_d2_bf16x2_tri", 256, 160, 32, 4, 1, 1, 2, 4, F32, BF, 2, false, true),
     // four waves of 512 registers, 256 x 320 tile (needs the workspace for the left operand's slots)
-    CASCMM_W512_VARIANT("t256x320x32_w512_bf16x2_tri"),
+    CASCMM_W512_VARIANT("t256x320x32_w512_bf16x2_tri", 0),
     // K split over the eight waves of a workgroup: one launch, no workspace
     CASCMM_WAVEK_VARIANT("t32x32x32_wavek_bf16x2_tri", 1),
     CASCMM_WAVEK_VARIANT("t32x64x32_wavek_bf16x2_tri", 2),

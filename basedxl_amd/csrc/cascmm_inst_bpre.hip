@@ -17,6 +17,8 @@ static const VariantDesc kTable[] = {
     CASCMM_TILE_VARIANT_BPRE("t64x64x64_w2x2x1_d3_bf16x2_tri_bpre", 64, 64, 64, 2, 2, 1, 3, 4, BF, 2, false),
     CASCMM_TILE_VARIANT_BPRE("t64x256x32_w1x4x1_d3_bf16x2_tri_bpre", 64, 256, 32, 1, 4, 1, 3, 4, BF, 2, false),
     CASCMM_TILE_VARIANT_BPRE("t256x160x32_w4x1x1_d2_bf16x2_tri_bpre", 256, 160, 32, 4, 1, 1, 2, 4, BF, 2, false),
+    // the large-tile kernel fed with prepared slots of B (A still raw fp32, split at fragment-read time)
+    CASCMM_W512_VARIANT("t256x320x32_w512_bf16x2_tri_bpre", 1),
     CASCMM_TILE_VARIANT_BPRE("t128x128x32_w4x2x1_d2_bf16x3_tri_bpre", 128, 128, 32, 4, 2, 1, 2, 4, BF, 3, false),
     CASCMM_TILE_VARIANT_BPRE("t128x128x32_w4x2x1_d2_fp16x3_tri_bpre", 128, 128, 32, 4, 2, 1, 2, 4, FP, 3, false),
     CASCMM_TILE_VARIANT_BPRE("t128x128x32_w4x2x1_d2_fp8x3_tri_bpre", 128, 128, 32, 4, 2, 1, 2, 4, F8, 3, false),

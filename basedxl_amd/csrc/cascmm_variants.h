@@ -184,15 +184,15 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   return CASCMM_OK;
 }
 
-// the large-tile kernel
-template <int UNUSED>
+// the large-tile kernel (BPRE = 1: right operand prepared)
+template <int BPRE>
 int launch_w512(const GroupParams& p, hipStream_t stream) {
   typedef W512 T;
   if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
   if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
-  auto kfn = cascmm_w512_kernel<UNUSED>;
+  auto kfn = cascmm_w512_kernel<BPRE>;
   static bool lds_set[kMaxDevices] = {false};
   const int d = device_index();
   if (d < 0) return CASCMM_ERR_LAUNCH;
@@ -342,9 +342,9 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   {NAME, KIND_WAVEK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, WaveK<NB>::BM, WaveK<NB>::BN, WaveK<NB>::BK, WaveK<NB>::NT, \
    WaveK<NB>::LDS_BYTES, true, true, &launch_wavek<NB>}
 
-#define CASCMM_W512_VARIANT(NAME)                                                                                   \
+#define CASCMM_W512_VARIANT(NAME, BPRE)                                                                             \
   {NAME, KIND_W512, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, W512::BM, W512::BN, 32, W512::NT, W512::LDS_BYTES, true, \
-   false, &launch_w512<0>}
+   false, &launch_w512<BPRE>, BPRE != 0}
 
 // eight producer waves, every B column loaded singly (all producer threads share A and B evenly)
 #define CASCMM_TILE_VARIANT_PS(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)          \

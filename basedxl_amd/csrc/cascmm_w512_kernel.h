@@ -58,8 +58,13 @@ __device__ __forceinline__ f32x16 w512_mfma_a(u32x4 a, u32x4 b, f32x16 c) {
 // Host-checked: M % 256 == 0, N % 320 == 0, K % 32 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
 // aligned, M * lda * 4 and K * ldb * 4 below 2 GiB, C rows addressable with 32-bit byte offsets
 // inside a tile.
+// BPRE = 1: the right operand comes already split (cascmm_prepare_weight: 16-byte slots of 8 k of one
+// column of one term, [term][K/8][N], below 2 GiB).  A stage then holds the same 20 KB of B as slots
+// [term][k group][320], copied by the same twenty 1 KB loads; a lane reads its two operands with two
+// 16-byte reads instead of eight 4-byte ones, and the split of B, 55 % of the kernel's VALU work,
+// is gone.  Same terms, same order of products: the results equal the raw kernel's bit for bit.
 // (a template, so that only the translation unit that lists the variant compiles it)
-template <int UNUSED>
+template <int BPRE>
 __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_w512_kernel(const GroupParams p) {
   typedef W512 T;
   extern __shared__ __attribute__((aligned(1024))) unsigned char w512_smem[];
@@ -90,13 +95,20 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
   for (int j = 0; j < 5; ++j) {
     const int inst = wave * 5 + j;
-    const int f = inst * 256 + lane * 4;
-    const int k = f / T::BN, pos = f % T::BN;
-    int n = pos - 32 * ((k >> 3) & 1);
-    n = n < 0 ? n + T::BN : n;
     b_lds[j] = T::A_STAGE + inst * 1024;
-    b_voff[j] = k * ldb_bytes + (n0 + n) * 4;
+    if (BPRE) {
+      // run inst = (term * 2 + k group) * 5 + run of 64 columns; lane = column inside the run
+      const int tk = inst / 5, run = inst % 5;
+      b_voff[j] = (((tk >> 1) * (p.K >> 3) + (tk & 1)) * p.N + n0 + run * 64 + lane) * 16;
+    } else {
+      const int f = inst * 256 + lane * 4;
+      const int k = f / T::BN, pos = f % T::BN;
+      int n = pos - 32 * ((k >> 3) & 1);
+      n = n < 0 ? n + T::BN : n;
+      b_voff[j] = k * ldb_bytes + (n0 + n) * 4;
+    }
   }
+  const int b_step = BPRE ? 2 * p.N * 16 : T::BK * ldb_bytes;   // bytes of B per stage
   auto issue1 = [&](int step_, int j) {
     const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
     const int st = step_ % T::NS;
@@ -104,7 +116,7 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
       __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (w512_lds_ptr)(smem + st * T::STAGE + a_lds[j]), 16, a_voff[j], step * T::BK * 4, 0, 0);
     else
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (w512_lds_ptr)(smem + st * T::STAGE + b_lds[j - 4]), 16, b_voff[j - 4],
-                                               step * T::BK * ldb_bytes, 0, 0);
+                                               step * b_step, 0, 0);
   };
 
   // fragment addresses (bytes inside a stage)
@@ -117,6 +129,8 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
     int pos = wn0 + ni * 32 + l31 + 32 * g;
     pos = pos >= T::BN ? pos - T::BN : pos;
     b_frag[ni] = T::A_STAGE + (8 * g * T::BN + pos) * 4;   // + e * BN * 4
+    // prepared: slot (term 0, k group g, column) -- term 1 is 2 * BN slots further
+    if (BPRE) b_frag[ni] = T::A_STAGE + (g * T::BN + wn0 + ni * 32 + l31) * 16;
   }
 
   f32x16 acc[T::MT][T::NTL];
@@ -144,6 +158,9 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
     for (int e = e0; e < e1; ++e) dst[e] = *(const float*)(stp + b_frag[ni] + e * T::BN * 4);
   };
+  // prepared B: the two terms of a block (the second term is needed four MFMAs later than the first)
+  auto read_slot_hi = [&](int buf, const unsigned char* stp, int ni) { H[buf] = *(const u32x4*)(stp + b_frag[ni]); };
+  auto read_slot_lo = [&](int buf, const unsigned char* stp, int ni) { L[buf] = *(const u32x4*)(stp + b_frag[ni] + 2 * T::BN * 16); };
   // the split of one pair of consecutive k in two halves of three VALU instructions each
   auto split_1 = [&](float (&x)[8], u32x4& hi, int e) {
     const f32x2v v = {x[2 * e], x[2 * e + 1]};
@@ -173,12 +190,17 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
         split_2(x, Af[0][0][mi], Af[0][1][mi], e);
       }
     }
-    read_raw(R[0], smem, 0, 0, 8);
-    read_raw(R[1], smem, 1, 0, 8);
+    if (BPRE) {
+      read_slot_hi(0, smem, 0);
+      read_slot_lo(0, smem, 0);
+    } else {
+      read_raw(R[0], smem, 0, 0, 8);
+      read_raw(R[1], smem, 1, 0, 8);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      split_1(R[0], H[0], e);
-      split_2(R[0], H[0], L[0], e);
+      for (int e = 0; e < 4; ++e) {
+        split_1(R[0], H[0], e);
+        split_2(R[0], H[0], L[0], e);
+      }
     }
   }
 
@@ -196,6 +218,8 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
         const int cur = t & 1, nxt = cur ^ 1;
         const int n2 = (ni + 2) % T::NTL;
         const unsigned char* st2 = (ni + 2 < T::NTL) ? st0 : st1;
+        const int n1 = (ni + 1) % T::NTL;                                  // prepared B: the next block's slots are read whole
+        const unsigned char* stn = (ni + 1 < T::NTL) ? st0 : st1;
         u32x4(&Ah)[T::MT] = Af[j][0];
         u32x4(&Al)[T::MT] = Af[j][1];
         // products lo.hi, hi.lo, hi.hi of the four row blocks: smallest first, consecutive MFMAs on
@@ -212,9 +236,11 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
           if (slot < T::LOADS) issue1(s + j + T::NS - 1, slot);
         };
         mm(0); W512_FENCE();
-        read_raw(R[cur], st2, n2, 0, 4); W512_FENCE();
+        if (!BPRE) read_raw(R[cur], st2, n2, 0, 4);
+        W512_FENCE();
         mm(1); W512_FENCE();
-        read_raw(R[cur], st2, n2, 4, 8); dl(0); W512_FENCE();
+        if (!BPRE) read_raw(R[cur], st2, n2, 4, 8);
+        dl(0); W512_FENCE();
         mm(2); W512_FENCE();
         if (ni < 4) {   // row block ni of the next stage
           const f32x4 x0 = *(const f32x4*)(st1 + a_frag0 + ni * 2048), x1 = *(const f32x4*)(st1 + a_frag1 + ni * 2048);
@@ -228,12 +254,14 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
         mm(3); W512_FENCE();
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          split_1(R[nxt], H[nxt], e);
+          if (!BPRE) split_1(R[nxt], H[nxt], e);
           if (ni < 4) split_1(RA, Af[j ^ 1][0][ni], e);
           W512_FENCE();
           mm(4 + 2 * e); W512_FENCE();
-          split_2(R[nxt], H[nxt], L[nxt], e);
+          if (!BPRE) split_2(R[nxt], H[nxt], L[nxt], e);
           if (ni < 4) split_2(RA, Af[j ^ 1][0][ni], Af[j ^ 1][1][ni], e);
+          if (BPRE && e == 0) read_slot_hi(nxt, stn, n1);     // behind MFMA 4: seven MFMAs before the next block's first
+          if (BPRE && e == 2) read_slot_lo(nxt, stn, n1);
           if (e == 3) dl(1);
           W512_FENCE();
           mm(5 + 2 * e); W512_FENCE();

@@ -728,7 +728,8 @@ def _fmt_of(name):
     return fmt, int(name.split(fmt + "x")[1][0])
 
 
-@pytest.mark.parametrize("shape", [(154, 64, 48), (256, 192, 160), (300, 128, 200), (96, 128, 384), (257, 64, 164), (130, 96, 84)])
+@pytest.mark.parametrize("shape", [(154, 64, 48), (256, 192, 160), (300, 128, 200), (96, 128, 384), (257, 64, 164), (130, 96, 84),
+                                   (256, 64, 320), (512, 96, 640)])
 def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
     M, K, N = shape
     a, b, want = _int_case(M, K, N, 100, seed=M + K + N)
@@ -739,6 +740,8 @@ def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
             continue
         if "fp8x3" in name and "f8k64" not in name and K % 64 == 0:
             continue  # three fp8 terms with K in steps of 64 are prepared for the fp8-rate kernel (another slot layout)
+        if "_w512_" in name and (M % 256 != 0 or N % 320 != 0):
+            continue  # the large-tile kernel takes whole 256 x 320 tiles
         fmt, terms = _fmt_of(name)
         _say("int-exact prepared", shape, name)
         w = PreparedWeight(_gpu(torch.tensor(b, dtype=torch.float32)), lowp=fmt, terms=terms)
@@ -750,12 +753,14 @@ def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
 
 def test_prepared_weight_equals_raw_weight_bit_for_bit(gpu_device):
     """Same tile, same consumer layout: the prepared path does the same split and accumulates
-    in the same order as the on-the-fly path, so the bits agree."""
+    in the same order as the on-the-fly path, so the bits agree (the large-tile kernel, which takes
+    whole 256 x 320 tiles, on operands of its own)."""
     names = _lib.variant_names()
-    a, b = oc.make_operands(1000, 640, 640, seed=31, w_std=0.02)
-    ad, bd = _gpu(a), _gpu(b)
-    bias = _gpu(torch.randn(640))
-    w = PreparedWeight(bd)
+    cases = {}
+    for big, (M, K, N) in ((False, (1000, 640, 640)), (True, (512, 1280, 640))):
+        a, b = oc.make_operands(M, K, N, seed=31, w_std=0.02)
+        ad, bd = _gpu(a), _gpu(b)
+        cases[big] = (ad, bd, _gpu(torch.randn(N)), PreparedWeight(bd))
     pairs = 0
     for vi, name in enumerate(names):
         if not name.endswith("bf16x2_tri_bpre"):
@@ -764,11 +769,12 @@ def test_prepared_weight_equals_raw_weight_bit_for_bit(gpu_device):
         if raw not in names:
             continue
         _say("prepared == raw", name)
+        ad, bd, bias, w = cases["_w512_" in name]
         got = cascaded_lowp_matmul(ad, w, bias=bias, variant=vi)
         ref = cascaded_lowp_matmul(ad, bd, bias=bias, variant=names.index(raw))
         assert torch.equal(got, ref), name
         pairs += 1
-    assert pairs >= 2
+    assert pairs >= 3 and any("_w512_" in n and n.endswith("_bpre") for n in names)
 
 
 @pytest.mark.parametrize("fmt,terms", [("bf16", 2), ("bf16", 3), ("fp16", 3), ("fp8", 3)])
