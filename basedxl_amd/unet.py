@@ -25,7 +25,7 @@ def patch_unet(model: nn.Module, cfg: BasedXLConfig) -> nn.Module:
     kw = cfg.cascade_kwargs()
     lin_kw = dict(kw, prepared=cfg.prepared)
     if cfg.fuse_kv:
-        fuse_kv_projections(model, cache_cross=cfg.cache_cross_kv, **lin_kw)
+        fuse_kv_projections(model, cache_cross=cfg.cache_cross_kv, fuse_q=cfg.fuse_qkv, **lin_kw)
     if cfg.fuse_geglu:
         fuse_geglu_layers(model, **kw)
     patch_linear_layers(model, **lin_kw)

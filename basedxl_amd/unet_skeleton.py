@@ -25,7 +25,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .modules.fused_kv import BasedXLFusedKV
+from .modules.fused_kv import BasedXLFusedKV, BasedXLFusedQKV
 from .modules.geglu import BasedXLLowPGEGLU
 
 W_STD = 0.02   # every weight ~ N(0, 0.02); biases zero-mean with the same spread
@@ -54,7 +54,8 @@ class FeedForward(nn.Module):
 
 class Attention(nn.Module):
     """Multi-head attention with separate to_q / to_k / to_v Linear layers (no bias) and an output
-    Linear; after :func:`fuse_kv_projections` the key and value come from one ``to_kv`` module."""
+    Linear; after :func:`fuse_kv_projections` the key and value come from one ``to_kv`` module, or
+    (self-attention, ``fuse_q``) query, key and value from one ``to_qkv`` module."""
 
     def __init__(self, query_dim: int, cross_dim: Optional[int], heads: int):
         super().__init__()
@@ -68,11 +69,14 @@ class Attention(nn.Module):
 
     def forward(self, x, context=None):
         src = x if context is None else context
-        q = self.to_q(x)
-        if hasattr(self, "to_kv"):
-            k, v = self.to_kv(src)
+        if hasattr(self, "to_qkv"):
+            q, k, v = self.to_qkv(x)
         else:
-            k, v = self.to_k(src), self.to_v(src)
+            q = self.to_q(x)
+            if hasattr(self, "to_kv"):
+                k, v = self.to_kv(src)
+            else:
+                k, v = self.to_k(src), self.to_v(src)
         B, T, C = q.shape
         h = self.heads
 
@@ -303,16 +307,24 @@ def synthetic_inputs(model: SDXLUNetSkeleton, *, batch: int = 2, latent: int = 1
 # ---------------------------------------------------------------------------------------------
 # patchers beyond the reference's Linear walk, and the record of what a forward pass routes
 # ---------------------------------------------------------------------------------------------
-def fuse_kv_projections(model: nn.Module, *, cache_cross: bool = False, **cascade_kwargs) -> nn.Module:
+def fuse_kv_projections(model: nn.Module, *, cache_cross: bool = False, fuse_q: bool = False, **cascade_kwargs) -> nn.Module:
     """Every attention module with ``to_k`` / ``to_v`` Linear children gets one ``to_kv``
     (:class:`BasedXLFusedKV`) instead, as basedxl/modules/attn.py:16-39 does; with ``cache_cross``
-    the cross-attention modules (``is_cross``) keep their result like attn.py:57,74-78.  Call it
-    BEFORE patch_linear_layers (it takes the plain Linear layers)."""
+    the cross-attention modules (``is_cross``) keep their result like attn.py:57,74-78.  With
+    ``fuse_q`` the self-attention modules (not ``is_cross``: query, key and value read the same tokens)
+    get one ``to_qkv`` (:class:`BasedXLFusedQKV`) for all three.  Call it BEFORE patch_linear_layers
+    (it takes the plain Linear layers)."""
     for module in list(model.modules()):
-        to_k, to_v = getattr(module, "to_k", None), getattr(module, "to_v", None)
-        if isinstance(to_k, nn.Linear) and isinstance(to_v, nn.Linear):
-            module.to_kv = BasedXLFusedKV(to_k, to_v, cache=cache_cross and bool(getattr(module, "is_cross", False)),
-                                          **cascade_kwargs)
+        to_q, to_k, to_v = getattr(module, "to_q", None), getattr(module, "to_k", None), getattr(module, "to_v", None)
+        if not (isinstance(to_k, nn.Linear) and isinstance(to_v, nn.Linear)):
+            continue
+        is_cross = bool(getattr(module, "is_cross", False))
+        if (fuse_q and not is_cross and hasattr(module, "is_cross") and isinstance(to_q, nn.Linear)
+                and to_q.in_features == to_k.in_features):
+            module.to_qkv = BasedXLFusedQKV(to_q, to_k, to_v, **cascade_kwargs)
+            del module.to_q, module.to_k, module.to_v
+        else:
+            module.to_kv = BasedXLFusedKV(to_k, to_v, cache=cache_cross and is_cross, **cascade_kwargs)
             del module.to_k, module.to_v
     return model
 

@@ -29,6 +29,8 @@ class BasedXLConfig:
     fuse_kv: bool = True
     #: ... whose cross-attention result is kept between denoising steps (attn.py:57,74-78)
     cache_cross_kv: bool = False
+    #: with fuse_kv: in self-attention, where all three read the same tokens, to_q too (one GEMM instead of two)
+    fuse_qkv: bool = True
     #: GEGLU gate applied in the store of the projection GEMM (weights kept split)
     fuse_geglu: bool = False
     #: keep the weights of the Linear layers split (None: the module's default for its dtype)

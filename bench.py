@@ -248,7 +248,8 @@ def bench_unet(dev, cascades=(("bf16", 2, None), ("fp8", 3, None), ("bf16", 2, T
         del unet, model
         torch.cuda.empty_cache()
     return {"workload": "cfg5: every nn.Linear and 1x1 convolution of one SDXL UNet denoising step (latent 2x4x128x128, text "
-                        "context 2x77x2048, weights ~N(0,0.02)) through the patched module tree (fused to_k/to_v, bias in the "
+                        "context 2x77x2048, weights ~N(0,0.02)) through the patched module tree (to_q/to_k/to_v of self-attention as one "
+                        "GEMM, to_k/to_v of cross-attention as one, bias in the "
                         "store, fp8 activation scale found in every call, weight scales kept); one HIP graph of all routed calls; "
                         "activations are split in every call, weights either in every call too or once (a labelled mode)",
             "configs": rows}

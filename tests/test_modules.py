@@ -33,6 +33,18 @@ def test_pointwise_predicate_and_patcher():
         BasedXLLowPConv1x1(torch.nn.Conv2d(8, 16, 3))
 
 
+def test_fused_qkv_weight_is_the_concatenation():
+    """Self-attention: query, key and value read the same tokens, so the three weights stack into one."""
+    from basedxl_amd.modules import BasedXLFusedQKV
+    to_q, to_k, to_v = (torch.nn.Linear(12, 8, bias=False) for _ in range(3))
+    mod = BasedXLFusedQKV(to_q, to_k, to_v)
+    assert mod.to_qkv.weight.shape == (12, 24) and mod.to_qkv.bias is None
+    for i, lin in enumerate((to_q, to_k, to_v)):
+        assert torch.equal(mod.to_qkv.weight[:, 8 * i:8 * i + 8], lin.weight.detach().T)
+    with pytest.raises(AssertionError):
+        BasedXLFusedQKV(to_q, torch.nn.Linear(16, 8, bias=False), torch.nn.Linear(16, 8, bias=False))   # cross-attention
+
+
 def test_pointwise_conv_holds_both_weight_layouts():
     conv = torch.nn.Conv2d(6, 10, 1)
     mod = BasedXLLowPConv1x1(conv)
@@ -129,6 +141,25 @@ def test_fused_kv_equals_separate_projections_and_caches(gpu_device):
     assert mod.kv_cache is None
     k4, _ = BasedXLFusedKV(to_k, to_v)(ctx)
     assert torch.equal(k4, k)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("lowp,terms,atol", [("bf16", 2, 3e-5), ("fp8", 3, 3e-4)])
+def test_fused_qkv_equals_the_oracle_of_each_projection(gpu_device, lowp, terms, atol):
+    from basedxl_amd.modules import BasedXLFusedQKV
+    torch.manual_seed(34)
+    lins = [torch.nn.Linear(640, 640, bias=False).to("cuda:0") for _ in range(3)]
+    x = torch.randn(2, 512, 640, device="cuda:0")
+    mod = BasedXLFusedQKV(*lins, lowp=lowp, terms=terms)
+    outs = mod(x)
+    assert all(o.shape == (2, 512, 640) for o in outs)
+    # the fp8 cascade scales the stacked weight as one tensor: the oracle gets that exponent
+    kw = {}
+    if lowp == "fp8":
+        kw = {"b_exp": oc.tensor_scale_exp(torch.cat([l.weight.detach().cpu() for l in lins]), "fp8")}
+    for got, lin in zip(outs, lins):
+        want = oc.cascade_matmul_ref(x.cpu().reshape(-1, 640), lin.weight.detach().cpu().T.contiguous(), lowp, terms, "tri", **kw)
+        torch.testing.assert_close(got.cpu().reshape(-1, 640), want, rtol=0, atol=atol)
 
 
 # ---------------------------------------------------------------------------------- gated projection

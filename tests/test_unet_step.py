@@ -79,10 +79,19 @@ def test_config_switch_off_leaves_the_model_alone_and_on_swaps_every_linear():
     assert not any(isinstance(x, nn.Linear) for x in full.modules())
     assert sum(isinstance(x, BasedXLLowPConv1x1) for x in full.modules()) == n_pw
     assert sum(isinstance(x, BasedXLLowPGEGLU) for x in full.modules()) == n_glu
-    assert sum(isinstance(x, BasedXLLowPLinear) for x in full.modules()) == n_linear - n_attn - n_glu   # k + v -> kv
+    n_self = sum(type(x).__name__ == "Attention" and not x.is_cross for x in m.modules())
+    # cross-attention: k + v -> kv; self-attention: q + k + v -> qkv
+    assert sum(isinstance(x, BasedXLLowPLinear) for x in full.modules()) == n_linear - (n_attn - n_self) - 2 * n_self - n_glu
     assert all((x.lowp, x.terms) == ("fp8", 3) for x in full.modules() if is_routed(x))
     kv = [x for x in full.modules() if type(x).__name__ == "BasedXLFusedKV"]
-    assert len(kv) == n_attn and not any(hasattr(a, "to_k") for a in full.modules() if type(a).__name__ == "Attention")
+    qkv = [x for x in full.modules() if type(x).__name__ == "BasedXLFusedQKV"]
+    assert len(kv) == n_attn - n_self and len(qkv) == n_self and 0 < n_self < n_attn
+    assert not any(hasattr(a, "to_k") for a in full.modules() if type(a).__name__ == "Attention")
+    assert all(hasattr(a, "to_q") == a.is_cross for a in full.modules() if type(a).__name__ == "Attention")
+    # the reference's own fusion only (attn.py:23-39)
+    kv_only = patch_unet(copy.deepcopy(m), BasedXLConfig(fp16_acc_matmul=True, fuse_qkv=False))
+    assert sum(type(x).__name__ == "BasedXLFusedKV" for x in kv_only.modules()) == n_attn
+    assert not any(type(x).__name__ == "BasedXLFusedQKV" for x in kv_only.modules())
 
 
 def test_bad_bias_is_refused_before_any_launch(monkeypatch):
@@ -207,7 +216,7 @@ def test_small_patched_unet_matches_the_oracle_layer_by_layer(gpu_device, fmt, t
     with torch.no_grad():
         exact = copy.deepcopy(base).double()(*[t.double() if torch.is_tensor(t) and t.is_floating_point() else t for t in inp[:3]],
                                              {k: v.double() for k, v in inp[3].items()})
-    cfg = BasedXLConfig(fp16_acc_matmul=True, lowp=fmt, terms=terms, fuse_kv=fused, fuse_geglu=fused, cache_cross_kv=fused)
+    cfg = BasedXLConfig(fp16_acc_matmul=True, lowp=fmt, terms=terms, fuse_kv=fused, fuse_qkv=fused, fuse_geglu=fused, cache_cross_kv=fused)
     unet = BasedXLUnet(copy.deepcopy(base).to(gpu_device), cfg)
     dev_in = synthetic_inputs(base, latent=16, text_tokens=7, seed=5, device=gpu_device)
     seen, hooks = [], []
