@@ -318,7 +318,9 @@ __global__ __launch_bounds__(F8K64T<MT>::NT) __attribute__((amdgpu_waves_per_eu(
       const int cur = (ab * T::NTL + ni) & 1, nxt = cur ^ 1;
       if (ni == T::NTL - 1) {
         // everything this wave needs of stage s is in registers: open stage s + 1
-        __builtin_amdgcn_s_waitcnt(0x0F70);     // own loads of stage s + 1 have landed (issued a stage ago)
+        // own loads of stage s + 1 have landed (issued a stage ago), and own reads of stage s have returned
+        // (the last of them were issued three MFMAs ago: the loads that follow the barrier overwrite that buffer)
+        __builtin_amdgcn_s_waitcnt(0x0070);     // vmcnt(0), lgkmcnt(0)
         __builtin_amdgcn_s_barrier();           // everybody's; and nobody reads stage s any more
       }
       int n_issued = 0;
