@@ -337,6 +337,9 @@ def main():
     ap.add_argument("--rotate", type=int, default=1,
                     help="number of distinct input/weight/output buffer sets the steps cycle through (1 = the same buffers "
                          "every step, resident in the Infinity Cache; 8 = every step reads HBM-cold data)")
+    ap.add_argument("--unet-select", default="",
+                    help="unet only: run one configuration instead of all eight, as cascade:weights:latent, e.g. "
+                         "bf16x2:raw:full or fp8x3:prepared:half (what a profiler run wants)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -372,7 +375,13 @@ def main():
                                   value=head["cascade_fp32_equiv_tflops"], unit="TFLOP/s", ms_per_step=round(head["cascade_bf16x2_us"] * 1e-3, 5),
                                   config={"workload": sw["workload"], "headline": f"n = {head['n']}"}, sizes=sw["sizes"])))
         else:
-            un = bench_unet(dev)
+            if args.unet_select:
+                casc, wts, lat = args.unet_select.split(":")
+                lowp, terms = casc.split("x")
+                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts == "prepared" else None),),
+                                latents=(("full latent", None),) if lat == "full" else (("half-latent share", 64),), forward=False)
+            else:
+                un = bench_unet(dev)
             head = un["configs"][0]
             print(json.dumps(dict(base, metric="fp32-equiv TFLOP/s of the Linear / 1x1-convolution path of one SDXL UNet step",
                                   value=head["fp32_equiv_tflops"], unit="TFLOP/s", ms_per_step=head["linear_path_ms_per_step"],
