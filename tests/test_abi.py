@@ -166,3 +166,25 @@ def test_library_tables_are_consistent():
     assert _lib.lib().cascmm_selftest() == 0
     names = _lib.variant_names()
     assert len(names) == len(set(names))
+
+
+def test_product_package_never_touches_the_oracle_or_the_reference_tree():
+    """The oracle is test infrastructure: nothing under basedxl_amd/ (Python or HIP sources) imports,
+    names or opens it, and nothing there reads the reference's tree; importing the package must not
+    pull the oracle in either."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    pkg = os.path.join(root, "basedxl_amd")
+    for dirpath, _dirs, files in os.walk(pkg):
+        if os.path.basename(dirpath) in ("build", "__pycache__"):
+            continue
+        for f in files:
+            if not f.endswith((".py", ".h", ".hip")):
+                continue
+            text = open(os.path.join(dirpath, f), encoding="utf-8").read()
+            assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), f
+            assert "oracle/" not in text and "/root/reference" not in text, f
+    code = "import sys, basedxl_amd, basedxl_amd.modules, basedxl_amd.unet, basedxl_amd.unet_skeleton; " \
+           "sys.exit(1 if any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules) else 0)"
+    assert subprocess.run([sys.executable, "-c", code], cwd=root).returncode == 0
