@@ -5,7 +5,9 @@ AddressSanitizer and UndefinedBehaviorSanitizer.
 is left alone), linked with the library's other objects and a small driver
 (`host_sanitizer_driver.cpp`) that walks the selection and size functions over a grid of shapes up
 to 2**40 and calls the launching entry points with arguments they must refuse before any HIP call.
-Nothing here needs a GPU.
+A second build, under ThreadSanitizer, is driven by `host_threads_driver.cpp`: eight threads ask for
+kernels and sizes at once (the selection keeps a table of earlier answers behind a lock) and must get
+what one thread gets.  Nothing here needs a GPU.
 """
 import glob
 import os
@@ -39,3 +41,23 @@ def test_host_layer_is_clean_under_asan_and_ubsan(tmp_path):
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
     r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0 and "OK (0 failures)" in r.stdout, (r.stdout[-1500:], r.stderr[-1500:])
+
+
+def test_concurrent_callers_are_clean_under_tsan_and_agree(tmp_path):
+    objs = [o for o in glob.glob(os.path.join(CSRC, "build", "*.o")) if not o.endswith("cascmm_api.o")]
+    if not os.path.exists(HIPCC) or shutil.which("g++") is None or len(objs) < 5:
+        pytest.skip("needs hipcc, g++ and the library's object files (python -m basedxl_amd.build)")
+    api, drv, exe = str(tmp_path / "api_tsan.o"), str(tmp_path / "driver.o"), str(tmp_path / "driver")
+    flags = ["-O1", "-g", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument"]
+    r = subprocess.run([HIPCC, *flags, "-Xarch_host", "-fsanitize=thread", "-c", os.path.join(CSRC, "cascmm_api.hip"), "-o", api],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fsanitize=thread", "-I", os.path.join(ROOT, "include"), "-c",
+                        os.path.join(HERE, "host_threads_driver.cpp"), "-o", drv], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-fsanitize=thread", "-fno-gpu-sanitize", "-o", exe, drv, api, *objs],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "OK (0 failures" in r.stdout and "ThreadSanitizer" not in r.stderr, (r.stdout[-1500:], r.stderr[-1500:])
