@@ -46,6 +46,7 @@ SIGNATURES = {
     "cascmm_select_variant_grouped": (c_int, [c_int] + [c_int64] * 6 + [c_int] * 4),
     "cascmm_variant_count": (c_int, []),
     "cascmm_variant_name": (c_char_p, [c_int]),
+    "cascmm_variant_kernel": (c_char_p, [c_int]),
     "cascmm_tensor_exp": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
     "cascmm_tensor_exps": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "cascmm_gemm_fp8_autoscale": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p] + [c_int64] * 6 + [c_int, c_int]

@@ -62,5 +62,41 @@ def build(verbose: bool = True, jobs: int = 8) -> str:
     return LIB
 
 
+def _listing(src: str) -> str:
+    """Assembly listing of one translation unit's device code (kept beside the objects, redone when a
+    source under csrc/ is newer)."""
+    out = os.path.join(OBJ, src[:-4] + ".gfx950.s")
+    newest = max(os.path.getmtime(os.path.join(CSRC, f)) for f in os.listdir(CSRC) if f.endswith((".hip", ".h")))
+    if not os.path.exists(out) or os.path.getmtime(out) < newest:
+        os.makedirs(OBJ, exist_ok=True)
+        cmd = [HIPCC, *FLAGS, "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc -S failed on {src}:\n{r.stderr[-2000:]}")
+    return out
+
+
+def kernel_isa(symbol: str, jobs: int = 8) -> str:
+    """gfx950 assembly of one kernel of the library, from its label to the end of its
+    `.amdhsa_kernel` block (register counts, LDS and scratch sizes), compiled from the sources under
+    csrc/ with the flags of the build.  `symbol` is what `cascmm_variant_kernel` returns."""
+    srcs = [f for f in sources() if f.startswith("cascmm_inst_")] + [f for f in sources() if not f.startswith("cascmm_inst_")]
+    with ThreadPoolExecutor(max_workers=min(jobs, len(srcs))) as ex:
+        listings = list(ex.map(_listing, srcs))
+    label, end = symbol + ":", ".end_amdhsa_kernel"
+    for path in listings:
+        with open(path) as f:
+            text = f.read()
+        at = text.find("\n" + label)
+        if at < 0:
+            continue
+        meta = text.find("\t.amdhsa_kernel " + symbol + "\n", at)
+        stop = text.find(end, meta if meta >= 0 else at)
+        if stop < 0:
+            continue
+        return f"; {os.path.basename(path)}\n" + text[at + 1:stop + len(end)] + "\n"
+    raise KeyError(f"no kernel {symbol} in the listings of {', '.join(srcs)}")
+
+
 if __name__ == "__main__":
     build()

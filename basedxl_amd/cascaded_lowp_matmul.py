@@ -474,6 +474,22 @@ def _rows(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def kernel_listing(variant: int) -> str:
+    """What `dump_ptx=True` writes: the variant's name, its kernel's symbol and the kernel's gfx950
+    assembly (compiled from the library's sources on first use; without a compiler the two header
+    lines and the reason)."""
+    l = _lib.lib()
+    name, sym = l.cascmm_variant_name(variant), l.cascmm_variant_kernel(variant)
+    head = f"// gfx950 kernel variant: {name.decode() if name else variant}\n// kernel: {sym.decode() if sym else '?'}\n"
+    if not sym:
+        return head
+    from . import build
+    try:
+        return head + build.kernel_isa(sym.decode())
+    except (OSError, RuntimeError, KeyError) as e:
+        return head + f"// no listing: {e}\n"
+
+
 def cascaded_lowp_matmul(
     a: torch.Tensor,
     b: torch.Tensor,
@@ -550,13 +566,12 @@ def cascaded_lowp_matmul(
     _gemm_2d(a2, b, out2, bias, fmt, terms, prod, variant, b_exp, tensor_exps)
 
     if dump_ptx:
-        # the reference writes the kernel's PTX (cascaded_lowp_matmul.py:170-171); there is no
-        # PTX here, so the file names the gfx950 kernel variant that ran instead
+        # the reference writes the PTX of the kernel it launched (cascaded_lowp_matmul.py:170-171);
+        # here the file holds the gfx950 assembly of the GEMM kernel that ran
         l = _lib.lib()
         v = variant if variant >= 0 else l.cascmm_select_variant(
             M, N, K, a2.stride(0), b.stride(0), out2.stride(0), _DTYPES[a.dtype], fmt, terms, prod)
-        name = l.cascmm_variant_name(v)
         with open("dump.ptx", "w") as f:
-            f.write(f"// gfx950 kernel variant: {name.decode() if name else v}\n")
+            f.write(kernel_listing(v & 0xFFFF))
 
     return out.reshape(*batch_dims, N)

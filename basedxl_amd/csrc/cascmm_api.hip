@@ -2,6 +2,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <dlfcn.h>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -850,6 +851,19 @@ int cascmm_variant_count(void) { return (int)table().size(); }
 const char* cascmm_variant_name(int variant) {
   if (variant < 0 || variant >= (int)table().size()) return nullptr;
   return table()[variant].name;
+}
+
+const char* cascmm_variant_kernel(int variant) {
+  if (variant < 0 || variant >= (int)table().size()) return nullptr;
+  const void* handle = nullptr;
+  GroupParams p;
+  memset(&p, 0, sizeof(p));
+  p.kernel_out = &handle;
+  if (table()[variant].launch(p, nullptr) != CASCMM_OK || !handle) return nullptr;
+  // the handle of a kernel is an exported object of this library that carries the kernel's name
+  Dl_info info;
+  if (!dladdr(handle, &info) || !info.dli_sname || info.dli_saddr != handle) return nullptr;
+  return info.dli_sname;
 }
 
 int cascmm_tensor_exp(const void* x, int64_t rows, int64_t cols, int64_t ld, int dtype, int32_t* exp_out,

@@ -323,6 +323,9 @@ struct GroupParams {
   // exps_dyn[0..1], which the GEMM then reads instead of tensor_exps
   int32_t* exps_dyn;
   const int32_t* b_exp_src;
+  // host side only: when set, the variant's launch function stores the handle of its GEMM kernel here
+  // and returns without checking or launching anything (the library names its kernels this way)
+  const void** kernel_out;
 };
 
 }  // namespace cascmm

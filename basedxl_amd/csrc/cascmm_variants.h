@@ -55,6 +55,7 @@ struct VariantDesc {
 template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST, bool BPRE = false>
 int launch_tile(const GroupParams& p, hipStream_t stream) {
   auto kfn = cascmm_tile_kernel<TL, IODT, FMT, TERMS, FULL, FAST, BPRE>;
+  if (p.kernel_out) { *p.kernel_out = (const void*)kfn; return CASCMM_OK; }
   constexpr int lds = LdsLayout<TL, Lowp<FMT>::planes(TERMS)>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
@@ -140,6 +141,7 @@ inline size_t skinny_workspace_bytes(int64_t M, int64_t N, int64_t K, int bm, in
 
 template <class TL, int FMT, int TERMS, bool FULL, bool SPLITK>
 int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
+  if (gp.kernel_out) { *gp.kernel_out = (const void*)cascmm_bdirect_kernel<TL, FMT, TERMS, FULL, SPLITK>; return CASCMM_OK; }
   if (gp.count != 1) return CASCMM_ERR_BAD_VARIANT;
   GemmParams p;
   memset(&p, 0, sizeof(p));
@@ -188,6 +190,7 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
 template <int BPRE>
 int launch_w512(const GroupParams& p, hipStream_t stream) {
   typedef W512 T;
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_w512_kernel<BPRE>; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
   if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
@@ -210,6 +213,7 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
 template <int NB>
 int launch_wavek(const GroupParams& p, hipStream_t stream) {
   typedef WaveK<NB> T;
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_wavek_kernel<NB>; return CASCMM_OK; }
   if (p.glu || p.k_splits > 1 || p.count < 1) return CASCMM_ERR_BAD_VARIANT;
   if (p.N % T::BN != 0 || p.K % T::BK != 0) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
@@ -266,6 +270,7 @@ inline size_t f8k64_workspace_bytes(int64_t M, int64_t N, int64_t K, bool bpre, 
 template <bool BPRE, int MT>
 int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   typedef F8K64T<MT> T;
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_f8k64_kernel<MT>; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1 || p.K % T::BK != 0 || p.K == 0) return CASCMM_ERR_BAD_VARIANT;
   const size_t need = f8k64_workspace_bytes(p.M, p.N, p.K, BPRE, T::BM);
   if (!p.workspace || p.workspace_bytes < need) return CASCMM_ERR_WORKSPACE;

@@ -200,6 +200,12 @@ int cascmm_variant_count(void);
 /* Static string: the device function name of the variant's kernel is a template
  * instantiation whose text contains this name (for filtering rocprof output), or NULL. */
 const char* cascmm_variant_name(int variant);
+/* The symbol (mangled device function name) of the GEMM kernel that the variant launches, as the
+ * code object, a profiler's kernel trace and an assembly listing of the library's sources spell it;
+ * static string, NULL for an index outside the table.  Works without a GPU.  Stands where the
+ * reference reads its compiled kernel back from the launch (`kernel.asm["ptx"]`,
+ * basedxl/triton/cascaded_lowp_matmul.py:163-171): the wrapper's `dump_ptx` looks this symbol up. */
+const char* cascmm_variant_kernel(int variant);
 
 /* fp8 tensor scale: writes to *exp_out (device int32) the exponent e with
  * max|x| * 2^e in (224, 448] (0 for an all-zero tensor).  x is [rows, cols] with leading

@@ -9,7 +9,8 @@ int main() {
   expect(cascmm_selftest() == 0, "selftest");
   const int n = cascmm_variant_count();
   expect(n > 50, "variant count");
-  for (int i = -2; i < n + 2; ++i) { const char* s = cascmm_variant_name(i); expect((s != nullptr) == (i >= 0 && i < n), "variant name range"); }
+  for (int i = -2; i < n + 2; ++i) { const char* s = cascmm_variant_name(i); expect((s != nullptr) == (i >= 0 && i < n), "variant name range");
+    const char* k = cascmm_variant_kernel(i); expect((k != nullptr) == (i >= 0 && i < n), "variant kernel range"); }
   const int64_t dims[] = {0, 1, 2, 31, 32, 33, 154, 640, 1280, 2048, 5120, 10240, 32768, (1ll << 31) - 1, 1ll << 31, 1ll << 40, -1};
   for (int64_t M : dims) for (int64_t N : dims) for (int64_t K : dims)
     for (int dt = -1; dt < 4; ++dt) for (int fmt = -1; fmt < 4; ++fmt) for (int terms = 0; terms < 5; ++terms) for (int pr = 0; pr < 2; ++pr) {

@@ -43,6 +43,30 @@ def test_variant_table():
     assert _lib.lib().cascmm_variant_name(len(names)) is None
 
 
+def test_every_variant_names_its_kernel_and_the_kernel_has_a_listing():
+    """`cascmm_variant_kernel` gives the device function's symbol without a GPU; the listing that
+    `dump_ptx=True` writes (the counterpart of the reference's PTX dump,
+    basedxl/triton/cascaded_lowp_matmul.py:170-171) is that function's gfx950 assembly."""
+    from basedxl_amd.cascaded_lowp_matmul import kernel_listing
+    l = _lib.lib()
+    names = _lib.variant_names()
+    kinds = {"_w512_": "cascmm_w512_kernel", "_wavek_": "cascmm_wavek_kernel", "_f8k64_": "cascmm_f8k64_kernel"}
+    for i, n in enumerate(names):
+        sym = l.cascmm_variant_kernel(i)
+        assert sym and sym.decode().startswith("_ZN6cascmm"), n
+        for tag, fn in kinds.items():
+            assert (tag in n) == (fn in sym.decode()), (n, sym)
+    assert l.cascmm_variant_kernel(-1) is None and l.cascmm_variant_kernel(len(names)) is None
+    if not os.path.exists(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")):
+        pytest.skip("the listing needs hipcc")
+    v = names.index("t256x320x32_w512_bf16x2_tri")
+    text = kernel_listing(v)
+    assert text.startswith("// gfx950 kernel variant: t256x320x32_w512_bf16x2_tri\n// kernel: _ZN6cascmm18cascmm_w512_kernelILi0E")
+    assert "no listing" not in text and "s_endpgm" in text
+    assert text.count("v_mfma_f32_32x32x16_bf16") == 120          # 20 blocks x 3 products x 2 k halves of a stage
+    assert ".amdhsa_next_free_vgpr 512" in text                      # the whole register file of a SIMD
+
+
 def _gemm(M, N, K, lda=None, ldb=None, ldc=None, dtype=0, fmt=0, terms=2, products=0, A=8, B=8, C=8):
     l = _lib.lib()
     return l.cascmm_gemm(A, B, C, None, M, N, K, lda if lda is not None else K, ldb if ldb is not None else N,

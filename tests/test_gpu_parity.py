@@ -580,6 +580,24 @@ def test_reference_shape_cases(gpu_device, shape_a, shape_b):
     assert torch.allclose(out.cpu(), torch.matmul(a, b), rtol=0.001, atol=0.35)
 
 
+def test_dump_ptx_writes_the_listing_of_the_kernel_that_ran(gpu_device, tmp_path, monkeypatch):
+    """The reference's `dump_ptx=True` writes `dump.ptx` into the working directory
+    (basedxl/triton/cascaded_lowp_matmul.py:170-171); here the file holds the variant's name, its
+    kernel's symbol and that kernel's gfx950 assembly, and the result is what it is without the dump."""
+    from basedxl_amd import _lib
+    monkeypatch.chdir(tmp_path)
+    g = torch.Generator().manual_seed(13)
+    a, b = _gpu(torch.randn(154, 2048, generator=g)), _gpu(torch.randn(2048, 1280, generator=g) * 0.02)
+    out = cascaded_lowp_matmul(a, b, dump_ptx=True)
+    assert torch.equal(out, cascaded_lowp_matmul(a, b))
+    text = (tmp_path / "dump.ptx").read_text()
+    l = _lib.lib()
+    v = l.cascmm_select_variant(154, 1280, 2048, 2048, 1280, 1280, 0, 0, 2, 0)
+    assert text.startswith(f"// gfx950 kernel variant: {l.cascmm_variant_name(v).decode()}\n// kernel: {l.cascmm_variant_kernel(v).decode()}\n")
+    if os.path.exists(os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")):    # (without a compiler: the two header lines and the reason)
+        assert "no listing" not in text and "v_mfma_f32_32x32x16_bf16" in text and "s_endpgm" in text
+
+
 def test_out_argument_strided_input_and_bias(gpu_device):
     g = torch.Generator().manual_seed(12)
     big = _gpu(torch.randn(64, 200, generator=g))

@@ -35,9 +35,10 @@ def test_host_layer_is_clean_under_asan_and_ubsan(tmp_path):
     r = subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-I", os.path.join(ROOT, "include"), "-c",
                         os.path.join(HERE, "host_sanitizer_driver.cpp"), "-o", drv], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
-    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined", "-fno-gpu-sanitize", "-o", exe, drv, api,
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined", "-fno-gpu-sanitize", "-rdynamic", "-o", exe, drv, api,
                         *objs], capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
+    # (-rdynamic: the library finds its kernels' names among its exported symbols, which an executable only has with it)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
     r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0 and "OK (0 failures)" in r.stdout, (r.stdout[-1500:], r.stderr[-1500:])
