@@ -6,6 +6,8 @@ operands whose partial sums stay below 2**24); for random fp32 operands the erro
 fp64 product must be no worse than 1.25x the oracle cascade's error (max-abs and relative
 Frobenius), same split and same product set.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
