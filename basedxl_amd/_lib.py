@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libcascmm.so")
 DT_F32, DT_F16, DT_BF16 = 0, 1, 2
 FMT_BF16, FMT_FP16, FMT_FP8 = 0, 1, 2
 PROD_TRI, PROD_FULL = 0, 1
+ERR_BAD_FORMAT = -4   # CASCMM_ERR_BAD_FORMAT: no kernel for this (dtype, format, terms, products, shape)
 
 FMT_BY_NAME = {"bf16": FMT_BF16, "fp16": FMT_FP16, "fp8": FMT_FP8}
 PROD_BY_NAME = {"tri": PROD_TRI, "full": PROD_FULL}
@@ -41,6 +42,8 @@ SIGNATURES = {
     "cascmm_gemm_prepared_glu": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p] + [c_int64] * 5 + [c_int] * 4
                                  + [c_void_p, c_void_p, c_int]),
     "cascmm_select_variant_prepared": (c_int, [c_int] + [c_int64] * 5 + [c_int] * 4),
+    "cascmm_select_variant_glu": (c_int, [c_int64] * 6 + [c_int] * 4),
+    "cascmm_gemm_glu": (c_int, [c_void_p] * 4 + [c_int64] * 6 + [c_int] * 4 + [c_void_p, c_int]),
     "cascmm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int]),
     "cascmm_select_variant": (c_int, [c_int64] * 6 + [c_int] * 4),
     "cascmm_select_variant_grouped": (c_int, [c_int] + [c_int64] * 6 + [c_int] * 4),

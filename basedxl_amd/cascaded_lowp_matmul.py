@@ -474,6 +474,64 @@ def _rows(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def gated_variant(a: torch.Tensor, b: torch.Tensor, *, lowp: Optional[str] = None, terms: Optional[int] = None,
+                  products: str = "tri") -> int:
+    """Index of the kernel that computes ``value * gelu(gate)`` of ``a @ b`` from the RAW ``[K, 2 * inner]``
+    weight in its store, or a negative status when there is none for these tensors (then the caller runs
+    the plain product and applies the gate)."""
+    if not (a.is_cuda and b.is_cuda and a.dtype == b.dtype == torch.float32 and b.dim() == 2 and b.is_contiguous()):
+        return _lib.ERR_BAD_FORMAT
+    d_lowp, d_terms = default_cascade(a.dtype)
+    lowp, terms = d_lowp if lowp is None else lowp, d_terms if terms is None else terms
+    K, N = b.shape
+    M = a.numel() // K if K else 0
+    if a.shape[-1] != K or M == 0 or N % 2 != 0:
+        return _lib.ERR_BAD_FORMAT
+    a2 = a.reshape(M, K)
+    if a2.stride(1) != 1 or a2.data_ptr() % 16 != 0 or b.data_ptr() % 16 != 0:
+        return _lib.ERR_BAD_FORMAT
+    return _lib.lib().cascmm_select_variant_glu(M, N, K, a2.stride(0), N, N // 2, _DTYPES[a.dtype], _lib.FMT_BY_NAME[lowp],
+                                                terms, _lib.PROD_BY_NAME[products])
+
+
+def cascaded_lowp_matmul_glu(a: torch.Tensor, b: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+                             out: Optional[torch.Tensor] = None, lowp: Optional[str] = None, terms: Optional[int] = None,
+                             products: str = "tri", variant: int = -1) -> torch.Tensor:
+    """``h = a @ b + bias; value, gate = h.chunk(2, -1); return value * gelu(gate)`` (diffusers' GEGLU around
+    one of the nn.Linear layers the reference routes, basedxl/unet.py:81-87) in ONE kernel on the raw
+    weight ``b`` ``[K, 2 * inner]``: ``h`` never reaches memory.  Only where :func:`gated_variant` finds a
+    kernel (fp32 tensors, two bf16 terms, rows % 256 == 0, inner % 160 == 0, K % 32 == 0); raises otherwise."""
+    assert a.shape[-1] == b.shape[-2], "Incompatible dimensions"
+    assert b.is_contiguous(), "Matrix B must be contiguous"
+    _check_device_tensor(a, "a")
+    _check_device_tensor(b, "b")
+    d_lowp, d_terms = default_cascade(a.dtype)
+    lowp, terms = d_lowp if lowp is None else lowp, d_terms if terms is None else terms
+    K, N = b.shape
+    if N % 2 != 0:
+        raise ValueError("a gated projection has an even number of columns")
+    bias = _check_bias(bias, a, N)
+    batch_dims = a.shape[:-1]
+    M = batch_dims.numel()
+    a2 = _rows(a.reshape(M, K))
+    inner = N // 2
+    if out is None:
+        out = torch.empty((M, inner), device=a.device, dtype=a.dtype)
+    else:
+        _check_device_tensor(out, "out")
+        if out.dtype != a.dtype or out.numel() != M * inner:
+            raise ValueError(f"out must hold {M * inner} elements of {a.dtype}")
+    out2 = out if out.dim() == 2 and out.shape == (M, inner) else out.view(M, inner)
+    if inner > 1 and out2.stride(1) != 1:
+        raise ValueError("out must have unit stride along its columns")
+    stream = torch.cuda.current_stream(a.device).cuda_stream
+    st = _lib.lib().cascmm_gemm_glu(a2.data_ptr(), b.data_ptr(), out2.data_ptr(), None if bias is None else bias.data_ptr(),
+                                    M, N, K, a2.stride(0) if M > 1 else max(K, 1), N, out2.stride(0) if M > 1 else max(inner, 1),
+                                    _DTYPES[a.dtype], _lib.FMT_BY_NAME[lowp], terms, _lib.PROD_BY_NAME[products], stream, variant)
+    _lib.check(st, "cascmm_gemm_glu")
+    return out.reshape(*batch_dims, inner)
+
+
 def kernel_listing(variant: int) -> str:
     """What `dump_ptx=True` writes: the variant's name, its kernel's symbol and the kernel's gfx950
     assembly (compiled from the library's sources on first use; without a compiler the two header

@@ -518,7 +518,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
     if (!C[i]) return CASCMM_ERR_NULL_POINTER;
     if (!aligned_to(C[i], es) || (bias && !aligned_to(bias[i], es))) return CASCMM_ERR_ALIGNMENT;
   }
-  if (q.glu && (!q.bpre || q.N % 64 != 0 || q.K == 0)) return CASCMM_ERR_BAD_SHAPE;
+  if (q.glu && (q.N % 64 != 0 || q.K == 0)) return CASCMM_ERR_BAD_SHAPE;
   if (q.K == 0) {
     const int64_t total = q.M * q.N;
     const unsigned grid = (unsigned)((total + 255) / 256);
@@ -710,6 +710,37 @@ int cascmm_gemm_grouped(int count, const void* const* A, const void* const* B, v
   if (!A || !B || !C) return CASCMM_ERR_NULL_POINTER;
   const Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
   return gemm_impl(count, A, B, C, bias, q, tensor_exps, workspace, workspace_bytes, (hipStream_t)stream, variant);
+}
+
+int cascmm_select_variant_glu(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt,
+                              int terms, int products) {
+  Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  q.glu = true;
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  if (N % 64 != 0 || K == 0) return CASCMM_ERR_BAD_SHAPE;
+  const bool fast = fast_ok(q, nullptr, nullptr);
+  const int v = select_variant(q, fast, 1);
+  if (v < 0) return v;
+  // worth it?  The alternative is the best plain kernel for the product plus the caller's gate, which
+  // reads M x N values and writes half as many (measured at about 3.5 TB/s, two launches); the kernel
+  // with the gated store may be a poor fit for the shape (too few tiles for the chip).
+  Problem plain = q;
+  plain.glu = false;
+  plain.ldc = N;
+  const int vp = select_variant(plain, fast, 1);
+  if (vp >= 0) {
+    const double gate_us = 2.0 + (double)M * (double)N * 6.0 / 3.5e6;
+    if (variant_cost(v, q, 1) > variant_cost(vp, plain, 1) + gate_us) return CASCMM_ERR_BAD_FORMAT;
+  }
+  return v;
+}
+
+int cascmm_gemm_glu(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K, int64_t lda,
+                    int64_t ldb, int64_t ldc, int dtype, int fmt, int terms, int products, void* stream, int variant) {
+  Problem q{M, N, K, lda, ldb, ldc, dtype, fmt, terms, products};
+  q.glu = true;
+  return gemm_impl(1, &A, &B, &C, bias ? &bias : nullptr, q, nullptr, nullptr, 0, (hipStream_t)stream, variant);
 }
 
 int cascmm_gemm(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K, int64_t lda,

@@ -301,6 +301,32 @@ struct GemmParams {
 // A group of GEMMs of one shape launched as one kernel (count == 1 for a plain GEMM).  Work
 // item i = problem i / tiles, tile i % tiles; workgroup w runs items w, w + grid, w + 2 grid ...
 constexpr int kMaxGroup = 8;
+// gelu(g) = 0.5 g (1 + erf(g / sqrt 2)) = 0.5 g erfc(-g / sqrt 2), and value x gelu(gate).
+// With x = |g| / sqrt 2 <= 4:  t = erfc(x) = 2^P(x), P a degree-11 fit of log2 erfc on [0, 4]
+// (|P - log2 erfc| < 4e-8, so t is good to a few 1e-6 RELATIVE down to erfc(4) = 1.5e-8), and
+// 1 + erf(g / sqrt 2) = t for g < 0, 2 - t otherwise: no cancellation in the negative tail, no
+// branch, one v_exp_f32.  Evaluated in fp32 the gate is within 4e-7 (one ulp at its largest)
+// of the exact gelu, like the textbook formula on a correctly rounded erff.
+__device__ __forceinline__ float gelu_value(float g) {
+  const float ax = __builtin_fabsf(g) * 0.70710678118654752f;
+  const float x = __builtin_fminf(ax, 4.0f);
+  float p = 1.133601089e-07f;
+  p = __builtin_fmaf(p, x, -2.984485036e-06f);
+  p = __builtin_fmaf(p, x, 3.493388431e-05f);
+  p = __builtin_fmaf(p, x, -2.373710740e-04f);
+  p = __builtin_fmaf(p, x, 1.004358870e-03f);
+  p = __builtin_fmaf(p, x, -2.405994106e-03f);
+  p = __builtin_fmaf(p, x, 7.954029570e-05f);
+  p = __builtin_fmaf(p, x, 2.782256342e-02f);
+  p = __builtin_fmaf(p, x, -1.483802944e-01f);
+  p = __builtin_fmaf(p, x, -9.184222221e-01f);
+  p = __builtin_fmaf(p, x, -1.627909303e+00f);
+  p = __builtin_fmaf(p, x, 3.292588246e-08f);
+  const float t = ax > 4.0f ? 0.f : __builtin_amdgcn_exp2f(p);   // beyond: erfc < 1.6e-8, taken as 0
+  return 0.5f * g * (g < 0.f ? t : 2.f - t);
+}
+__device__ __forceinline__ float gated_value(float v, float g) { return v * gelu_value(g); }
+
 struct GroupParams {
   int M, N, K;
   int64_t lda, ldb, ldc;
@@ -314,9 +340,10 @@ struct GroupParams {
   size_t workspace_bytes;
   int k_splits;             // LDS-tiled kernels: work item = (split, problem, tile); 0 or 1 = no split
   const int32_t* tensor_exps;  // fp8: {e_A, e_B} of problem i at [2i], [2i + 1]; NULL = all zero
-  // Gated epilogue (prepared-weight kernels): the N columns of B alternate 32 "value" and 32
-  // "gate" columns; C has N/2 columns, C[m][32 j + l] = (h[m][64 j + l] + bias[32 j + l]) *
-  // gelu(h[m][64 j + 32 + l] + bias[N/2 + 32 j + l]) with h = A x B.
+  // Gated epilogue: C has N/2 columns, C[m][32 j + l] = (v + bias[32 j + l]) * gelu(g + bias[N/2 + 32 j + l])
+  // with v and g the entries of A x B in row m whose columns of B are, for a prepared operand (which
+  // alternates 32 "value" and 32 "gate" columns), 64 j + l and 64 j + 32 + l, and for a raw operand
+  // (value columns in the first half, gate columns in the second) 32 j + l and N/2 + 32 j + l.
   int glu;
   // fp8-rate kernel only: the left operand's scale exponent is found inside the launch (two kernels:
   // per-workgroup maxima, then the operand split reduces them) and written, with *b_exp_src, to

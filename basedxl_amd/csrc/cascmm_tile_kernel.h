@@ -168,30 +168,7 @@ struct TileGemm {
   // the gated epilogue needs prepared B (columns in any order at no cost) and a consumer wave that
   // owns whole value / gate pairs of 32-column blocks
   static constexpr bool kGluCapable = BPRE && TL::BNQ == 0 && TL::NTL % 2 == 0;
-  // value x gelu(gate), gelu(g) = 0.5 g (1 + erf(g / sqrt 2)) = 0.5 g erfc(-g / sqrt 2).
-  // With x = |g| / sqrt 2 <= 4:  t = erfc(x) = 2^P(x), P a degree-11 fit of log2 erfc on [0, 4]
-  // (|P - log2 erfc| < 4e-8, so t is good to a few 1e-6 RELATIVE down to erfc(4) = 1.5e-8), and
-  // 1 + erf(g / sqrt 2) = t for g < 0, 2 - t otherwise: no cancellation in the negative tail, no
-  // branch, one v_exp_f32.  Evaluated in fp32 the gate is within 4e-7 (one ulp at its largest)
-  // of the exact gelu, like the textbook formula on a correctly rounded erff.
-  static __device__ __forceinline__ float gated(float v, float g) {
-    const float ax = __builtin_fabsf(g) * 0.70710678118654752f;
-    const float x = __builtin_fminf(ax, 4.0f);
-    float p = 1.133601089e-07f;
-    p = __builtin_fmaf(p, x, -2.984485036e-06f);
-    p = __builtin_fmaf(p, x, 3.493388431e-05f);
-    p = __builtin_fmaf(p, x, -2.373710740e-04f);
-    p = __builtin_fmaf(p, x, 1.004358870e-03f);
-    p = __builtin_fmaf(p, x, -2.405994106e-03f);
-    p = __builtin_fmaf(p, x, 7.954029570e-05f);
-    p = __builtin_fmaf(p, x, 2.782256342e-02f);
-    p = __builtin_fmaf(p, x, -1.483802944e-01f);
-    p = __builtin_fmaf(p, x, -9.184222221e-01f);
-    p = __builtin_fmaf(p, x, -1.627909303e+00f);
-    p = __builtin_fmaf(p, x, 3.292588246e-08f);
-    const float t = ax > 4.0f ? 0.f : __builtin_amdgcn_exp2f(p);   // beyond: erfc < 1.6e-8, taken as 0
-    return v * (0.5f * g * (g < 0.f ? t : 2.f - t));
-  }
+  static __device__ __forceinline__ float gated(float v, float g) { return gated_value(v, g); }
   static constexpr int QN = TL::QN;
   static constexpr int QW = TL::BNQ > 0 ? TL::BNQ / QN : 1;   // blocks per row of the permuted part
   static constexpr int SW = TL::BNS > 0 ? TL::BNS : 1;       // columns of the unpermuted part

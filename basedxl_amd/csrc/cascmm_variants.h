@@ -49,7 +49,7 @@ struct VariantDesc {
   bool grouped;  // one launch may run several same-shape problems and several tiles per workgroup
   int (*launch)(const GroupParams&, hipStream_t);
   bool bpre = false;  // takes the right operand already split (cascmm_prepare_weight)
-  bool glu = false;   // has the gated epilogue (a consumer wave owns whole value / gate block pairs)
+  bool glu = false;   // has the gated epilogue
 };
 
 template <class TL, int IODT, int FMT, int TERMS, bool FULL, bool FAST, bool BPRE = false>
@@ -187,15 +187,10 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
 }
 
 // the large-tile kernel (BPRE = 1: right operand prepared)
-template <int BPRE>
-int launch_w512(const GroupParams& p, hipStream_t stream) {
+template <int BPRE, int GLU>
+int launch_w512_kernel(const GroupParams& p, hipStream_t stream) {
   typedef W512 T;
-  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_w512_kernel<BPRE>; return CASCMM_OK; }
-  if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
-  if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
-  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
-    return CASCMM_ERR_TOO_LARGE;
-  auto kfn = cascmm_w512_kernel<BPRE>;
+  auto kfn = cascmm_w512_kernel<BPRE, GLU>;
   static bool lds_set[kMaxDevices] = {false};
   const int d = device_index();
   if (d < 0) return CASCMM_ERR_LAUNCH;
@@ -207,6 +202,18 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n);
   if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
   return CASCMM_OK;
+}
+
+template <int BPRE>
+int launch_w512(const GroupParams& p, hipStream_t stream) {
+  typedef W512 T;
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_w512_kernel<BPRE, 0>; return CASCMM_OK; }
+  if (p.count != 1 || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
+  if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
+  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
+    return CASCMM_ERR_TOO_LARGE;
+  // (the gated store is an instantiation of its own)
+  return p.glu ? launch_w512_kernel<BPRE, 1>(p, stream) : launch_w512_kernel<BPRE, 0>(p, stream);
 }
 
 // skinny problems, K split over the waves of a workgroup
@@ -349,7 +356,7 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
 
 #define CASCMM_W512_VARIANT(NAME, BPRE)                                                                             \
   {NAME, KIND_W512, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, W512::BM, W512::BN, 32, W512::NT, W512::LDS_BYTES, true, \
-   false, &launch_w512<BPRE>, BPRE != 0}
+   false, &launch_w512<BPRE>, BPRE != 0, true}
 
 // eight producer waves, every B column loaded singly (all producer threads share A and B evenly)
 #define CASCMM_TILE_VARIANT_PS(NAME, BM, BN, BK, WM, WN, WK, DEPTH, NP, IODT, FMT, TERMS, FULL, FAST)          \

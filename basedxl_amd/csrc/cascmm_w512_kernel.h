@@ -58,13 +58,17 @@ __device__ __forceinline__ f32x16 w512_mfma_a(u32x4 a, u32x4 b, f32x16 c) {
 // Host-checked: M % 256 == 0, N % 320 == 0, K % 32 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
 // aligned, M * lda * 4 and K * ldb * 4 below 2 GiB, C rows addressable with 32-bit byte offsets
 // inside a tile.
+// GLU = 1: the gated store (C has N / 2 columns, see GroupParams); a raw operand's gate columns are
+// fetched from N / 2 further right, so that both kinds of operand fill the same accumulator blocks.
+// (An instantiation of its own: the plain kernel stays as it is, without the scratch bytes this epilogue's
+// register allocation asks for.)
 // BPRE = 1: the right operand comes already split (cascmm_prepare_weight: 16-byte slots of 8 k of one
 // column of one term, [term][K/8][N], below 2 GiB).  A stage then holds the same 20 KB of B as slots
 // [term][k group][320], copied by the same twenty 1 KB loads; a lane reads its two operands with two
 // 16-byte reads instead of eight 4-byte ones, and the split of B, 55 % of the kernel's VALU work,
 // is gone.  Same terms, same order of products: the results equal the raw kernel's bit for bit.
 // (a template, so that only the translation unit that lists the variant compiles it)
-template <int BPRE>
+template <int BPRE, int GLU = 0>
 __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_w512_kernel(const GroupParams p) {
   typedef W512 T;
   extern __shared__ __attribute__((aligned(1024))) unsigned char w512_smem[];
@@ -105,7 +109,11 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
       const int k = f / T::BN, pos = f % T::BN;
       int n = pos - 32 * ((k >> 3) & 1);
       n = n < 0 ? n + T::BN : n;
-      b_voff[j] = k * ldb_bytes + (n0 + n) * 4;
+      int col = n0 + n;
+      // gated store: the tile's ten column blocks are value 0, gate 0, value 1, ... of output columns
+      // n0 / 2 + 32 j + l; the raw operand keeps its gate columns N / 2 further right
+      if (GLU) col = ((n >> 5) & 1) * (p.N >> 1) + (n0 >> 1) + 32 * (n >> 6) + (n & 31);
+      b_voff[j] = k * ldb_bytes + col * 4;
     }
   }
   const int b_step = BPRE ? 2 * p.N * 16 : T::BK * ldb_bytes;   // bytes of B per stage
@@ -276,10 +284,54 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   asm volatile("s_nop 7\n s_nop 7\n s_nop 7" ::: "memory");
 
   // ---- epilogue: of every block a lane holds column l31, rows 8 q + 4 g + e -----------------------
-  float* C = (float*)p.C[0] + (int64_t)(m0 + wm0) * p.ldc + n0 + wn0;
   const float* bias = (const float*)p.bias[0];
-  const i32x4 rc = make_rsrc(C, 0x7FFFFFFF);
   const int ldc_bytes = (int)p.ldc * 4;
+  if constexpr (GLU != 0) {
+    // Gated store: C[m][n0 / 2 + 32 j + l] = (value j + bias) x gelu(gate j + bias), j = 0 .. 4.  The
+    // left wave of a row pair holds value 0, gate 0, value 1, gate 1, value 2, the right one gate 2,
+    // value 3, gate 3, value 4, gate 4: pair 2 is the only one that spans two waves; the right wave
+    // evaluates its gate (which evens out the two waves' arithmetic) and hands gelu(gate), same lanes and
+    // registers, over through the LDS the main loop has given up.
+    const int half = p.N >> 1, c0 = n0 >> 1;
+    float* xbuf = (float*)smem + (wave >> 1) * (T::MT * 16 * 64);   // 16 KB per row pair of waves
+    __builtin_amdgcn_s_barrier();                                    // every wave has read its last fragments
+    if (wave & 1) {
+      const float bg = bias ? bias[half + c0 + 64 + l31] : 0.f;
+#pragma unroll
+      for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) xbuf[(mi * 16 + r) * 64 + lane] = gelu_value(acc[mi][0][r] + bg);
+    }
+    __syncthreads();
+    float* C = (float*)p.C[0] + (int64_t)(m0 + wm0) * p.ldc + c0;
+    const i32x4 rc = make_rsrc(C, 0x7FFFFFFF);
+    auto out_pair = [&](int pair, int vb, int gb, bool gate_in_lds) {
+      const float bv = bias ? bias[c0 + 32 * pair + l31] : 0.f;
+      const float bg = (bias && !gate_in_lds) ? bias[half + c0 + 32 * pair + l31] : 0.f;
+      const int voff = g * 4 * ldc_bytes + (pair * 32 + l31) * 4;
+#pragma unroll
+      for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * q + e;
+            const float gl = gate_in_lds ? xbuf[(mi * 16 + r) * 64 + lane] : gelu_value(acc[mi][gb][r] + bg);
+            llvm_raw_buffer_store_f32((acc[mi][vb][r] + bv) * gl, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+          }
+    };
+    if ((wave & 1) == 0) {
+      out_pair(0, 0, 1, false);
+      out_pair(1, 2, 3, false);
+      out_pair(2, 4, 0, true);
+    } else {
+      out_pair(3, 1, 2, false);
+      out_pair(4, 3, 4, false);
+    }
+    return;
+  }
+  float* C = (float*)p.C[0] + (int64_t)(m0 + wm0) * p.ldc + n0 + wn0;
+  const i32x4 rc = make_rsrc(C, 0x7FFFFFFF);
 #pragma unroll
   for (int ni = 0; ni < T::NTL; ++ni) {
     const float bv = bias ? bias[n0 + wn0 + ni * 32 + l31] : 0.f;

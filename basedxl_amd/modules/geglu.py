@@ -14,19 +14,22 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from ..cascaded_lowp_matmul import PreparedWeight, cascaded_lowp_matmul, default_cascade
+from ..cascaded_lowp_matmul import PreparedWeight, cascaded_lowp_matmul, cascaded_lowp_matmul_glu, default_cascade, gated_variant
 
 
 class BasedXLLowPGEGLU(nn.Module):
     """Wraps the ``proj`` Linear ([in] -> [2 * inner]) of a GEGLU block; ``forward(x)`` returns
     ``value * gelu(gate)`` ([..., inner]), gelu in its exact (erf) form.
 
-    The fused kernel takes fp32 activations (any cascade) or fp16 / bf16 activations (as one term of
-    their own format) on the GPU with ``in % 64 == 0`` and ``inner % 32 == 0``; anything else runs the cascade GEMM on the raw weight followed by torch's gate (the same
-    arithmetic in three kernels)."""
+    The fused kernels take fp32 activations (any cascade) or fp16 / bf16 activations (as one term of
+    their own format) on the GPU with ``in % 64 == 0`` and ``inner % 32 == 0`` and read a prepared
+    (pre-split, column-interleaved) copy of the weight, made on first use.  ``prepared=False`` keeps
+    no such copy: the large-tile kernel applies the gate on the raw weight where it takes the problem
+    (fp32, two bf16 terms, rows % 256 == 0, inner % 160 == 0).  Anything else runs the cascade GEMM on the
+    raw weight followed by torch's gate (the same arithmetic in three kernels)."""
 
     def __init__(self, proj: nn.Linear, *, lowp: Optional[str] = None, terms: Optional[int] = None,
-                 products: str = "tri"):
+                 products: str = "tri", prepared: Optional[bool] = None):
         super().__init__()
         if proj.out_features % 2 != 0:
             raise ValueError("a gated projection has an even number of output features")
@@ -35,6 +38,7 @@ class BasedXLLowPGEGLU(nn.Module):
         self.bias = proj.bias.detach().clone() if proj.bias is not None else None
         d_lowp, d_terms = default_cascade(self.weight.dtype)
         self.lowp, self.terms, self.products = d_lowp if lowp is None else lowp, d_terms if terms is None else terms, products
+        self.prepared = True if prepared is None else bool(prepared)
         self._prepared: Optional[PreparedWeight] = None
 
     def _fusable(self, x: torch.Tensor) -> bool:
@@ -45,7 +49,7 @@ class BasedXLLowPGEGLU(nn.Module):
 
     def prepare(self) -> None:
         """Prepare the gated weight now (needs the weight on the GPU); otherwise on the first eager call."""
-        if self.weight.is_cuda and self.in_features % 64 == 0 and self.inner % 32 == 0 and (
+        if self.prepared and self.weight.is_cuda and self.in_features % 64 == 0 and self.inner % 32 == 0 and (
                 self._prepared is None or self._prepared.device != self.weight.device):
             self._prepared = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms, glu=True)
 
@@ -59,7 +63,10 @@ class BasedXLLowPGEGLU(nn.Module):
             h = cascade_linear(x, self.weight, None, self.bias, self.lowp, self.terms, self.products, False, None)
             value, gate = h.chunk(2, dim=-1)
             return value * F.gelu(gate)
-        if self._fusable(x):
+        if not self.prepared and x.is_cuda and x.dtype == self.weight.dtype and gated_variant(
+                x, self.weight, lowp=self.lowp, terms=self.terms, products=self.products) >= 0:
+            return cascaded_lowp_matmul_glu(x, self.weight, bias=self.bias, lowp=self.lowp, terms=self.terms, products=self.products)
+        if self.prepared and self._fusable(x):
             if self._prepared is None or self._prepared.device != self.weight.device:
                 self._prepared = PreparedWeight(self.weight, lowp=self.lowp, terms=self.terms, glu=True)
             x2 = x.reshape(-1, self.in_features)

@@ -27,7 +27,7 @@ def patch_unet(model: nn.Module, cfg: BasedXLConfig) -> nn.Module:
     if cfg.fuse_kv:
         fuse_kv_projections(model, cache_cross=cfg.cache_cross_kv, fuse_q=cfg.fuse_qkv, **lin_kw)
     if cfg.fuse_geglu:
-        fuse_geglu_layers(model, **kw)
+        fuse_geglu_layers(model, **lin_kw)
     patch_linear_layers(model, **lin_kw)
     if cfg.route_pointwise_convs:
         patch_pointwise_convs(model, **kw)

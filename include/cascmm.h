@@ -182,6 +182,20 @@ int cascmm_gemm_prepared_glu(int count, const void* const* A, const void* const*
                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldc,
                              int dtype, int fmt, int terms, int products,
                              const int32_t* tensor_exps, void* stream, int variant);
+/* The same gated product on the RAW weight W [K, N] (row-major, ldb; value columns in the first half,
+ * gate columns in the second, as the module holds it): no prepared copy of the weight is needed.  Only
+ * the large-tile kernel of the two-term bf16 cascade has this store (fp32 tensors, M % 256 == 0,
+ * N % 320 == 0, K % 32 == 0, rows 16-byte aligned): cascmm_select_variant_glu returns its index, or
+ * CASCMM_ERR_BAD_FORMAT when it does not take the problem or when the library's cost estimates put the
+ * best plain kernel plus a separate gate pass ahead (few tiles on many CUs); the caller then runs
+ * cascmm_gemm and applies the gate itself.  cascmm_gemm_glu launches it wherever it takes the problem
+ * (variant < 0: automatic).  `bias` as above.  Same place in the reference
+ * as above. */
+int cascmm_select_variant_glu(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                              int dtype, int fmt, int terms, int products);
+int cascmm_gemm_glu(const void* A, const void* B, void* C, const void* bias,
+                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                    int dtype, int fmt, int terms, int products, void* stream, int variant);
 
 /* Bytes of device workspace cascmm_gemm can use for this problem (0 for most shapes).
  * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,

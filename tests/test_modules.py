@@ -216,6 +216,75 @@ def test_gated_kernels_integer_exact_value_and_gate_pairing(gpu_device):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_large_tile_kernel_gated_store_raw_and_prepared_weight(gpu_device, with_bias):
+    """The 256 x 320 kernel's gated store, on the raw weight (gate columns fetched from the second half)
+    and on the prepared one (columns interleaved): small-integer operands make h exact, so both must
+    give value * gelu(gate) of the integer product up to the erf evaluation, and the same bits as each
+    other; 2 x 3 tiles, so every wave's pairs and the pair that crosses two waves land in two row tiles."""
+    from basedxl_amd import PreparedWeight, _lib, cascaded_lowp_matmul
+    from basedxl_amd.cascaded_lowp_matmul import cascaded_lowp_matmul_glu, gated_variant
+
+    g = torch.Generator().manual_seed(43)
+    M, K, inner = 512, 128, 480
+    a = torch.randint(-3, 4, (M, K), generator=g).float()
+    w = torch.randint(-2, 3, (K, 2 * inner), generator=g).float()
+    bias = torch.randint(-2, 3, (2 * inner,), generator=g).float()
+    h = (a.long() @ w.long() + (bias.long() if with_bias else 0)).double()
+    want = h[:, :inner] * torch.nn.functional.gelu(h[:, inner:])
+    ad, wd, bd = a.to("cuda:0"), w.to("cuda:0"), bias.to("cuda:0") if with_bias else None
+    names = _lib.variant_names()
+    # (the selection: the kernel where it fills the chip, the plain product plus a gate pass where it does not)
+    big_a, big_w = torch.empty(2048, 1280, device="cuda:0"), torch.empty(1280, 10240, device="cuda:0")
+    assert names[gated_variant(big_a, big_w)] == "t256x320x32_w512_bf16x2_tri"
+    assert gated_variant(big_a[:1024], big_w) < 0 and gated_variant(ad, wd) < 0
+    out = torch.full((M, inner + 8), -7.0, device="cuda:0")
+    y = cascaded_lowp_matmul_glu(ad, wd, bias=bd, out=out[:, :inner])
+    assert bool((out[:, inner:] == -7.0).all())                        # nothing written past the row
+    torch.testing.assert_close(y.cpu().double(), want, rtol=1e-5, atol=2e-5)
+    pw = PreparedWeight(wd, lowp="bf16", terms=2, glu=True)
+    y2 = cascaded_lowp_matmul(ad, pw, bias=bd, variant=names.index("t256x320x32_w512_bf16x2_tri_bpre"))
+    assert torch.equal(y2, y)
+    # problems the kernel does not take are reported, not launched
+    assert gated_variant(ad[:200], wd) < 0 and gated_variant(ad, wd[:, :704].contiguous()) < 0
+    assert gated_variant(ad, wd, lowp="fp16", terms=3) < 0
+    with pytest.raises(RuntimeError):
+        cascaded_lowp_matmul_glu(ad[:200], wd)
+
+
+@pytest.mark.gpu
+def test_geglu_module_on_the_raw_weight_at_the_feed_forward_shape(gpu_device):
+    """`prepared=False`: no second copy of the weight; the 32x32-stage feed-forward projection
+    (2048 x 1280 x 10240) runs the gate in the large-tile kernel's store.  Against the oracle's gated
+    projection (1.25x bound) and against the plain product followed by torch's gate."""
+    from basedxl_amd import BasedXLLowPGEGLU, BasedXLLowPLinear
+
+    torch.manual_seed(44)
+    M, K, inner = 2048, 1280, 5120
+    proj = torch.nn.Linear(K, 2 * inner).to("cuda:0")
+    with torch.no_grad():
+        proj.weight.mul_(0.02 * K ** 0.5)
+    x = torch.randn(2, M // 2, K, device="cuda:0")
+    mod = BasedXLLowPGEGLU(proj, prepared=False)
+    y = mod(x)
+    assert y.shape == (2, M // 2, inner) and mod._prepared is None
+    h = BasedXLLowPLinear(proj, prepared=False)(x)
+    unfused = h[..., :inner] * torch.nn.functional.gelu(h[..., inner:])
+    torch.testing.assert_close(y, unfused, rtol=2e-5, atol=2e-5)
+    rows = torch.arange(0, M, 8)                                       # a row sample keeps the fp64 product short
+    x2, wt, b = x.cpu().reshape(-1, K)[rows], proj.weight.detach().cpu().T.contiguous(), proj.bias.detach().cpu()
+    want = oc.gated_projection_ref(x2, wt, b)
+    h64 = oc.fp64_matmul(x2, wt) + b.double()
+    exp = h64[:, :inner] * oc.gelu_erf(h64[:, inner:])
+    got, ref = oc.error_metrics(y.cpu().reshape(-1, inner)[rows], exp), oc.error_metrics(want, exp)
+    assert got["rel_fro"] <= 1.25 * ref["rel_fro"] and got["max_abs"] <= 1.25 * ref["max_abs"], (got, ref)
+    # a shape the kernel does not take: the plain product and torch's gate, still without a prepared copy
+    y3 = mod(x[:, :100])
+    torch.testing.assert_close(y3, unfused[:, :100], rtol=2e-5, atol=2e-5)
+    assert mod._prepared is None
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("M,K,inner", [(4096, 640, 2560), (1024, 1280, 5120), (77, 640, 2560)])
 def test_geglu_module_matches_oracle_and_unfused_path(gpu_device, M, K, inner):
     from basedxl_amd import BasedXLLowPGEGLU, BasedXLLowPLinear
