@@ -253,14 +253,15 @@ def test_large_tile_kernel_gated_store_raw_and_prepared_weight(gpu_device, with_
 
 
 @pytest.mark.gpu
-def test_geglu_module_on_the_raw_weight_at_the_feed_forward_shape(gpu_device):
-    """`prepared=False`: no second copy of the weight; the 32x32-stage feed-forward projection
-    (2048 x 1280 x 10240) runs the gate in the large-tile kernel's store.  Against the oracle's gated
-    projection (1.25x bound) and against the plain product followed by torch's gate."""
+@pytest.mark.parametrize("M,K,inner", [(2048, 1280, 5120), (8192, 640, 2560)])
+def test_geglu_module_on_the_raw_weight_at_the_feed_forward_shape(gpu_device, M, K, inner):
+    """`prepared=False`: no second copy of the weight; the feed-forward projections of the 32x32 and
+    64x64 stages at full latent (2048 x 1280 x 10240: one tile per CU; 8192 x 640 x 5120: two) run the
+    gate in the large-tile kernel's store.  Against the oracle's gated projection (1.25x bound) and
+    against the plain product followed by torch's gate."""
     from basedxl_amd import BasedXLLowPGEGLU, BasedXLLowPLinear
 
     torch.manual_seed(44)
-    M, K, inner = 2048, 1280, 5120
     proj = torch.nn.Linear(K, 2 * inner).to("cuda:0")
     with torch.no_grad():
         proj.weight.mul_(0.02 * K ** 0.5)
