@@ -50,6 +50,8 @@ SIGNATURES = {
     "cascmm_variant_count": (c_int, []),
     "cascmm_variant_name": (c_char_p, [c_int]),
     "cascmm_variant_kernel": (c_char_p, [c_int]),
+    "cascmm_probe_mfma": (c_int, [c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "cascmm_probe_stream": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p, c_size_t, c_void_p]),
     "cascmm_tensor_exp": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
     "cascmm_tensor_exps": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "cascmm_gemm_fp8_autoscale": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p] + [c_int64] * 6 + [c_int, c_int]

@@ -157,6 +157,47 @@ def _graph_time_us(fn, reps, replays=5, spin_s=0.2):
     return e0.elapsed_time(e1) * 1e3 / (replays * reps)
 
 
+def measured_peaks(dev):
+    """What this GPU sustains where the published peaks assume the boost clock: a register-only loop of
+    bf16 MFMAs on every SIMD, one streaming read and one copy of 1 GiB (the library's probe kernels,
+    events around five launches each after the clocks are up)."""
+    import torch
+    from basedxl_amd import _lib
+
+    l = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(launch, n=5, spin_s=0.2):
+        t_end = time.perf_counter() + spin_s
+        while time.perf_counter() < t_end:
+            launch()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n          # seconds per launch
+
+    wgs, iters = 2 * 256, 8000                          # two workgroups of four waves per CU
+    out = torch.empty(wgs * 256, device=dev)
+    t = timed(lambda: _lib.check(l.cascmm_probe_mfma(wgs, iters, out.data_ptr(), out.numel() * 4, stream), "cascmm_probe_mfma"))
+    mfma = wgs * 4 * iters * 4 * 2.0 * 32 * 32 * 16 / t * 1e-12
+    n = 1 << 30
+    src = torch.empty(n // 4, device=dev).normal_()
+    dst = torch.empty_like(src)
+    g = 8 * 256
+    sums = torch.empty(g * 256, device=dev)
+    t_r = timed(lambda: _lib.check(l.cascmm_probe_stream(src.data_ptr(), None, n, g, sums.data_ptr(), sums.numel() * 4, stream),
+                                   "cascmm_probe_stream"))
+    t_c = timed(lambda: _lib.check(l.cascmm_probe_stream(src.data_ptr(), dst.data_ptr(), n, g, None, 0, stream), "cascmm_probe_stream"))
+    del src, dst
+    return {"mfma_bf16_tflops": round(mfma, 1), "hbm_read_gbs": round(n / t_r * 1e-9, 1), "hbm_copy_gbs": round(2 * n / t_c * 1e-9, 1),
+            "how": "register-only loop of v_mfma_f32_32x32x16_bf16, 8 waves per CU; 1 GiB streamed once (read) / copied (read + write bytes); "
+                   "events around 5 launches after 0.2 s of the same launches"}
+
+
 KV_TRAFFIC_BYTES = {1280: 21034047.0, 640: 18076444.0}   # HBM-side bytes per launch from rocprofv3 counters (see profiles/), when measured
 
 
@@ -628,6 +669,12 @@ def main():
         del sets, a_dev, w_dev
         torch.cuda.empty_cache()
         result["other_workloads"] = {"kv": bench_kv(dev), "unet": bench_unet(dev), "eager_launch": bench_eager_launch(dev)}
+    if args.workload == "ffn" and not args.no_graph:
+        # the published peak beside what the board holds: `peak` and `frac` stay the published ones
+        torch.cuda.empty_cache()
+        mp = measured_peaks(dev)
+        result["roofline"]["measured_peaks"] = mp
+        result["roofline"]["frac_of_measured_mfma"] = round(dom["mfma_tflops"] / mp["mfma_bf16_tflops"], 4)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cpu_in, launches)
     print(json.dumps(result))

@@ -261,6 +261,18 @@ int cascmm_gemm_fp8_autoscale(const void* A, const void* B, int b_prepared, void
 int cascmm_split_terms(const void* x, float* out, int64_t n, int dtype, int fmt, int terms,
                        int tensor_exp, void* stream);
 
+/* Measurement hooks (no counterpart in the reference, whose self-benchmark only times its kernel,
+ * basedxl/triton/cascaded_lowp_matmul.py:204-242): what the GPU at hand sustains on the two resources a
+ * roofline prices the cascade against.
+ * cascmm_probe_mfma: `workgroups` x 4 waves each issue `iters` x 4 independent v_mfma_f32_32x32x16_bf16
+ * on registers only (131072 flop per wave and iteration); out: workgroups x 256 floats of device memory.
+ * cascmm_probe_stream: one pass over `bytes` (a multiple of 16) of device memory at src with
+ * `workgroups` x 256 threads, 16 bytes per thread and step: copied to dst, or, with dst NULL, only read
+ * (sums: workgroups x 256 floats).  Timing is the caller's (events on `stream`). */
+int cascmm_probe_mfma(int workgroups, int iters, float* out, size_t out_bytes, void* stream);
+int cascmm_probe_stream(const void* src, void* dst, size_t bytes, int workgroups, float* sums, size_t sums_bytes,
+                        void* stream);
+
 /* Consistency of the library's own tables (no counterpart in the reference): the number of entries of
  * the measured-cost table that do not name exactly one compiled kernel variant, plus the number of
  * variant names that occur twice; 0 for a sound build.  (A cost entry whose kernel was renamed would

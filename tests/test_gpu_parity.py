@@ -600,6 +600,28 @@ def test_dump_ptx_writes_the_listing_of_the_kernel_that_ran(gpu_device, tmp_path
         assert "no listing" not in text and "v_mfma_f32_32x32x16_bf16" in text and "s_endpgm" in text
 
 
+def test_measurement_probes_run_and_check_their_arguments(gpu_device):
+    """The register-only MFMA loop and the streaming kernels behind the bench's measured peaks: the
+    copy copies, the read leaves the sum of what it read, bad arguments are refused."""
+    from basedxl_amd import _lib
+    l = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    out = torch.zeros(8 * 256, device="cuda:0")
+    assert l.cascmm_probe_mfma(8, 10, out.data_ptr(), out.numel() * 4, stream) == 0
+    assert l.cascmm_probe_mfma(8, 10, out.data_ptr(), 16, stream) != 0 and l.cascmm_probe_mfma(0, 10, out.data_ptr(), 1 << 20, stream) != 0
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and float(out.abs().max()) > 0
+    src = torch.randint(-8, 9, (1 << 18,), device="cuda:0").float()          # 1 MiB of small integers: the sum is exact
+    dst = torch.zeros_like(src)
+    sums = torch.zeros(4 * 256, device="cuda:0")
+    assert l.cascmm_probe_stream(src.data_ptr(), dst.data_ptr(), src.numel() * 4, 4, None, 0, stream) == 0
+    assert l.cascmm_probe_stream(src.data_ptr(), None, src.numel() * 4, 4, sums.data_ptr(), sums.numel() * 4, stream) == 0
+    assert l.cascmm_probe_stream(src.data_ptr(), None, src.numel() * 4, 4, sums.data_ptr(), 16, stream) != 0
+    assert l.cascmm_probe_stream(src.data_ptr(), dst.data_ptr(), 24, 4, None, 0, stream) != 0
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src) and float(sums.sum()) == float(src.sum())
+
+
 def test_out_argument_strided_input_and_bias(gpu_device):
     g = torch.Generator().manual_seed(12)
     big = _gpu(torch.randn(64, 200, generator=g))
