@@ -209,7 +209,7 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
   typedef W512 T;
   if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_w512_kernel<BPRE, 0>; return CASCMM_OK; }
   if (p.count != 1 || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
-  if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
+  if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0 || p.K < 32) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
   // (the gated store is an instantiation of its own)

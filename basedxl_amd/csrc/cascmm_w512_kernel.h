@@ -284,6 +284,9 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   asm volatile("s_nop 7\n s_nop 7\n s_nop 7" ::: "memory");
 
   // ---- epilogue: of every block a lane holds column l31, rows 8 q + 4 g + e -----------------------
+  // (the lane number is taken afresh: a register kept alive through the main loop for it would be spilled)
+  const int elane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  const int el31 = elane & 31, eg = elane >> 5;
   const float* bias = (const float*)p.bias[0];
   const int ldc_bytes = (int)p.ldc * 4;
   if constexpr (GLU != 0) {
@@ -296,19 +299,19 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
     float* xbuf = (float*)smem + (wave >> 1) * (T::MT * 16 * 64);   // 16 KB per row pair of waves
     __builtin_amdgcn_s_barrier();                                    // every wave has read its last fragments
     if (wave & 1) {
-      const float bg = bias ? bias[half + c0 + 64 + l31] : 0.f;
+      const float bg = bias ? bias[half + c0 + 64 + el31] : 0.f;
 #pragma unroll
       for (int mi = 0; mi < T::MT; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) xbuf[(mi * 16 + r) * 64 + lane] = gelu_value(acc[mi][0][r] + bg);
+        for (int r = 0; r < 16; ++r) xbuf[(mi * 16 + r) * 64 + elane] = gelu_value(acc[mi][0][r] + bg);
     }
     __syncthreads();
     float* C = (float*)p.C[0] + (int64_t)(m0 + wm0) * p.ldc + c0;
     const i32x4 rc = make_rsrc(C, 0x7FFFFFFF);
     auto out_pair = [&](int pair, int vb, int gb, bool gate_in_lds) {
-      const float bv = bias ? bias[c0 + 32 * pair + l31] : 0.f;
-      const float bg = (bias && !gate_in_lds) ? bias[half + c0 + 32 * pair + l31] : 0.f;
-      const int voff = g * 4 * ldc_bytes + (pair * 32 + l31) * 4;
+      const float bv = bias ? bias[c0 + 32 * pair + el31] : 0.f;
+      const float bg = (bias && !gate_in_lds) ? bias[half + c0 + 32 * pair + el31] : 0.f;
+      const int voff = eg * 4 * ldc_bytes + (pair * 32 + el31) * 4;
 #pragma unroll
       for (int mi = 0; mi < T::MT; ++mi)
 #pragma unroll
@@ -316,7 +319,7 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int r = 4 * q + e;
-            const float gl = gate_in_lds ? xbuf[(mi * 16 + r) * 64 + lane] : gelu_value(acc[mi][gb][r] + bg);
+            const float gl = gate_in_lds ? xbuf[(mi * 16 + r) * 64 + elane] : gelu_value(acc[mi][gb][r] + bg);
             llvm_raw_buffer_store_f32((acc[mi][vb][r] + bv) * gl, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
           }
     };
@@ -334,8 +337,8 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   const i32x4 rc = make_rsrc(C, 0x7FFFFFFF);
 #pragma unroll
   for (int ni = 0; ni < T::NTL; ++ni) {
-    const float bv = bias ? bias[n0 + wn0 + ni * 32 + l31] : 0.f;
-    const int voff = g * 4 * ldc_bytes + (ni * 32 + l31) * 4;
+    const float bv = bias ? bias[n0 + wn0 + ni * 32 + el31] : 0.f;
+    const int voff = eg * 4 * ldc_bytes + (ni * 32 + el31) * 4;
 #pragma unroll
     for (int mi = 0; mi < T::MT; ++mi)
 #pragma unroll
