@@ -142,12 +142,6 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   }
 
   f32x16 acc[T::MT][T::NTL];
-#pragma unroll
-  for (int mi = 0; mi < T::MT; ++mi)
-#pragma unroll
-    for (int ni = 0; ni < T::NTL; ++ni)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
 
   // ---- software pipeline ---------------------------------------------------------------------
   // Blocks are numbered t = stage * 5 + ni.  While the 12 MFMAs of block t issue, the raw B values of
@@ -185,6 +179,25 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   for (int s = 0; s < T::NS - 1; ++s)
 #pragma unroll
     for (int j = 0; j < T::LOADS; ++j) issue1(s, j);
+  // the accumulators are cleared while the first loads are in flight: not before them, which would hold
+  // the loads back, and not after the barrier, where the first MFMA would wait for it
+  W512_FENCE();
+#pragma unroll
+  for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
+  // (an empty statement that "uses" every block makes the zeros real here; left alone the compiler creates them
+  // right before the first MFMAs)
+#pragma unroll
+  for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni) {
+      if (ni < 4) asm volatile("" : "+a"(acc[mi][ni]));
+      else asm volatile("" : "+v"(acc[mi][ni]));
+    }
+  W512_FENCE();
   __builtin_amdgcn_s_waitcnt(0x0F70 | (18 & 0xF) | ((18 >> 4) << 14));   // vmcnt(18): stage 0 has landed
   __builtin_amdgcn_s_barrier();
   {
