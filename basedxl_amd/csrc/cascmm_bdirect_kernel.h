@@ -324,6 +324,21 @@ static __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* 
   const int64_t stride = total / 4;
   f32x4 s = src[0];
   int k = 1;
+  // two to four splits (what the LDS-tiled kernels use): every load in flight before the first addition;
+  // the general loop below waits for each load of its tail in turn.  Same order of additions.
+  if (k_splits == 4) {
+    const f32x4 v1 = __builtin_nontemporal_load(src + stride), v2 = __builtin_nontemporal_load(src + 2 * stride),
+                v3 = __builtin_nontemporal_load(src + 3 * stride);
+    s += v1;
+    s += v2;
+    s += v3;
+    k = 4;
+  } else if (k_splits == 3) {
+    const f32x4 v1 = __builtin_nontemporal_load(src + stride), v2 = __builtin_nontemporal_load(src + 2 * stride);
+    s += v1;
+    s += v2;
+    k = 3;
+  }
   for (; k + 8 <= k_splits; k += 8) {
     f32x4 v[8];
 #pragma unroll
