@@ -69,10 +69,14 @@ def _listing(src: str) -> str:
     newest = max(os.path.getmtime(os.path.join(CSRC, f)) for f in os.listdir(CSRC) if f.endswith((".hip", ".h")))
     if not os.path.exists(out) or os.path.getmtime(out) < newest:
         os.makedirs(OBJ, exist_ok=True)
-        cmd = [HIPCC, *FLAGS, "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", out]
+        tmp = f"{out}.{os.getpid()}.tmp"      # (another process may be making the same listing: rename a finished file into place)
+        cmd = [HIPCC, *FLAGS, "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", tmp]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
+            if os.path.exists(tmp):
+                os.remove(tmp)
             raise RuntimeError(f"hipcc -S failed on {src}:\n{r.stderr[-2000:]}")
+        os.replace(tmp, out)
     return out
 
 
