@@ -31,6 +31,7 @@ SIGNATURES = {
     "cascmm_gemm": (c_int, _GEMM_ARGS),
     "cascmm_gemm_variant": (c_int, _GEMM_ARGS + [c_int]),
     "cascmm_gemm_noalloc": (c_int, _GEMM_ARGS[:15] + [c_void_p]),
+    "cascmm_init": (c_int, []),
     "cascmm_gemm_grouped": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p] + _GEMM_ARGS[4:] + [c_int]),
     "cascmm_prepared_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
     "cascmm_prepare_weight": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p,

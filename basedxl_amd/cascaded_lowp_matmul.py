@@ -30,15 +30,34 @@ _workspaces: Dict[Tuple[int, object], torch.Tensor] = {}
 _MIN_WORKSPACE = 1 << 20
 
 
+#: capture buffers that a larger one has replaced.  A device graph recorded earlier has the old
+#: buffer's address baked into its launches and writes its partial results there on every replay, so
+#: the memory must stay this package's for as long as the process lives (buffers double in size, which
+#: bounds what is kept to the size of the current one).
+_retired_capture_buffers: list = []
+
+
+def _grow_capture_workspace(index: int, dev: torch.device, nbytes: int) -> torch.Tensor:
+    key = (index, "capture")
+    old = _workspaces.get(key)
+    if old is not None:
+        _retired_capture_buffers.append(old)
+        nbytes = max(nbytes, 2 * old.numel())
+    ws = _workspaces[key] = torch.empty(max(nbytes, _MIN_WORKSPACE), dtype=torch.uint8, device=dev)
+    return ws
+
+
 def reserve_workspace(nbytes: int, device=None) -> None:
     """Make sure the workspace that launches recorded into a device graph use holds ``nbytes``, so
     that a capture allocates nothing.  Every eager launch does this for its own need, so a capture
-    that follows the usual eager warm-up of the same calls finds its workspace already there."""
+    that follows the usual eager warm-up of the same calls finds its workspace already there.  A
+    buffer that has to grow is replaced, never freed: graphs recorded against it keep replaying into
+    memory that nothing else can own."""
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), "capture")
-    ws = _workspaces.get(key)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    ws = _workspaces.get((index, "capture"))
     if ws is None or ws.numel() < nbytes:
-        _workspaces[key] = torch.empty(max(nbytes, _MIN_WORKSPACE), dtype=torch.uint8, device=dev)
+        _grow_capture_workspace(index, dev, nbytes)
 
 
 def _workspace(device: torch.device, stream: int, nbytes: int) -> Optional[torch.Tensor]:
@@ -52,7 +71,7 @@ def _workspace(device: torch.device, stream: int, nbytes: int) -> Optional[torch
         if ws is None or ws.numel() < nbytes:
             # no eager warm-up came first: the buffer comes from the graph's own pool (an
             # allocation inside the capture, but no fill: nothing is recorded for it)
-            ws = _workspaces[(index, "capture")] = torch.empty(max(nbytes, _MIN_WORKSPACE), dtype=torch.uint8, device=device)
+            ws = _grow_capture_workspace(index, device, nbytes)
         return ws
     reserve_workspace(nbytes, device)
     key = (index, stream)

@@ -99,7 +99,9 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
                                f8k64_slot_bytes(q.M, q.K) > INT32_MAX || f8k64_slot_bytes(q.N, q.K) > INT32_MAX))
     return false;
   if (v.bpre && v.kind != KIND_F8K64 && prepared_as_k16_slots(q.K, q.fmt, q.terms, q.glu)) return false;   // other layout
-  if (v.kind == KIND_W512 && (q.M % v.BM != 0 || q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX)) return false;
+  if (v.kind == KIND_W512 && (q.M % v.BM != 0 || q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX ||
+                              (!q.bpre && q.K * q.ldb * 4 > INT32_MAX) || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
+    return false;
   if (v.kind == KIND_WAVEK && (q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX || q.K == 0)) return false;
   if (q.glu && !v.glu) return false;
   return true;
@@ -283,7 +285,9 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
 struct SelectKey {
   int64_t M, N, K;
   size_t ws_bytes;
-  int dtype, fmt, terms, products, count, flags;   // flags: fast | bpre << 1 | glu << 2
+  // flags: fast | bpre << 1 | glu << 2, and what variant_matches reads of the leading dimensions (the
+  // 32-bit addressing limits of some kernels): M lda, K ldb and 1024 ldc beyond 2^31 bytes << 3, 4, 5
+  int dtype, fmt, terms, products, count, flags;
   bool operator==(const SelectKey& o) const {
     return M == o.M && N == o.N && K == o.K && ws_bytes == o.ws_bytes && dtype == o.dtype && fmt == o.fmt &&
            terms == o.terms && products == o.products && count == o.count && flags == o.flags;
@@ -303,12 +307,19 @@ struct SelectHit { int variant, splits; };
 
 static int select_variant_uncached(const Problem& q, bool fast, int count, size_t ws_bytes, int* splits_out);
 
+// a x b x c > 2^31 - 1, for any non-negative 64-bit factors (the product itself may not fit 64 bits)
+static bool beyond_i32(int64_t a, int64_t b, int64_t c) {
+  int64_t ab = 0, abc = 0;
+  return __builtin_mul_overflow(a, b, &ab) || __builtin_mul_overflow(ab, c, &abc) || abc > INT32_MAX;
+}
+
 static int select_variant(const Problem& q, bool fast, int count, size_t ws_bytes = (size_t)-1,
                           int* splits_out = nullptr) {
   static std::mutex mu;
   static std::unordered_map<SelectKey, SelectHit, SelectKeyHash> memo;
   const SelectKey key{q.M, q.N, q.K, ws_bytes, q.dtype, q.fmt, q.terms, q.products, count,
-                      (fast ? 1 : 0) | (q.bpre ? 2 : 0) | (q.glu ? 4 : 0)};
+                      (fast ? 1 : 0) | (q.bpre ? 2 : 0) | (q.glu ? 4 : 0) | (beyond_i32(q.M, q.lda, 4) ? 8 : 0) |
+                          (beyond_i32(q.K, q.ldb, 4) ? 16 : 0) | (beyond_i32(q.ldc, 1024, 1) ? 32 : 0)};
   {
     std::lock_guard<std::mutex> lock(mu);
     auto it = memo.find(key);
@@ -654,6 +665,11 @@ static int noalloc_scratch(void** out) {
 }
 
 extern "C" {
+
+int cascmm_init(void) {
+  void* p = nullptr;
+  return noalloc_scratch(&p);
+}
 
 int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias, int64_t M, int64_t N, int64_t K,
                         int64_t lda, int64_t ldb, int64_t ldc, int dtype, int fmt, int terms, int products,

@@ -1,5 +1,6 @@
 // Host-side table of compiled kernel variants and the launcher template that fills it.
 #pragma once
+#include <atomic>
 #include <cstring>
 #include <mutex>
 
@@ -28,15 +29,28 @@ inline int device_index() {
   return d;
 }
 inline int device_cus() {
-  static int cus[kMaxDevices] = {0};
+  static std::atomic<int> cus[kMaxDevices];   // (zero-initialised; every thread that finds 0 stores the same answer)
   const int d = device_index();
   if (d < 0) return kNumCUs;
-  if (cus[d] == 0) {
-    int n = 0;
+  int n = cus[d].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, d) != hipSuccess || n <= 0) n = kNumCUs;
-    cus[d] = n;   // (a benign race: every thread stores the same value)
+    cus[d].store(n, std::memory_order_relaxed);
   }
-  return cus[d];
+  return n;
+}
+
+// More than 64 KB of dynamic LDS must be asked for once per kernel and device.  `done` is the kernel's
+// own per-device record (zero-initialised atomics: host threads may launch at once; the attribute call
+// is idempotent, so two threads that both find the flag clear both make it and both succeed).
+typedef std::atomic<bool> LdsFlags[kMaxDevices];
+inline bool ensure_lds(const void* kfn, int lds_bytes, LdsFlags& done) {
+  const int d = device_index();
+  if (d < 0) return false;
+  if (done[d].load(std::memory_order_acquire)) return true;
+  if (hipFuncSetAttribute(kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) return false;
+  done[d].store(true, std::memory_order_release);
+  return true;
 }
 
 struct VariantDesc {
@@ -59,25 +73,18 @@ int launch_tile(const GroupParams& p, hipStream_t stream) {
   constexpr int lds = LdsLayout<TL, Lowp<FMT>::planes(TERMS)>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
-    // more than 64 KB of LDS must be asked for once per device (the attribute is per device)
-    static bool lds_set[kMaxDevices] = {false};
-    const int d = device_index();
-    if (d < 0) return CASCMM_ERR_LAUNCH;
-    if (!lds_set[d]) {
-      if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-        return CASCMM_ERR_LAUNCH;
-      lds_set[d] = true;
-    }
+    static LdsFlags lds_set;
+    if (!ensure_lds((const void*)kfn, lds, lds_set)) return CASCMM_ERR_LAUNCH;
   }
   // persistent grid: at most as many workgroups as can be resident at once on this device
-  static int occupancy[kMaxDevices] = {0};
+  static std::atomic<int> occupancy[kMaxDevices];
   const int dev = device_index();
   if (dev < 0) return CASCMM_ERR_LAUNCH;
-  int per_cu = occupancy[dev];
+  int per_cu = occupancy[dev].load(std::memory_order_relaxed);
   if (per_cu == 0) {
     int n = 0;
     per_cu = (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)kfn, TL::NT, lds) == hipSuccess && n > 0) ? n : 1;
-    occupancy[dev] = per_cu;
+    occupancy[dev].store(per_cu, std::memory_order_relaxed);
   }
   const int splits = p.k_splits > 1 ? p.k_splits : 1;
   if (splits > 1) {
@@ -164,15 +171,8 @@ int launch_bdirect(const GroupParams& gp, hipStream_t stream) {
   constexpr int lds = LdsLayoutA<TL, TERMS>::kBytes;
   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
   if (lds > 64 * 1024) {
-    // more than 64 KB of LDS must be asked for once per device (the attribute is per device)
-    static bool lds_set[kMaxDevices] = {false};
-    const int d = device_index();
-    if (d < 0) return CASCMM_ERR_LAUNCH;
-    if (!lds_set[d]) {
-      if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-        return CASCMM_ERR_LAUNCH;
-      lds_set[d] = true;
-    }
+    static LdsFlags lds_set;
+    if (!ensure_lds((const void*)kfn, lds, lds_set)) return CASCMM_ERR_LAUNCH;
   }
   const unsigned grid = (unsigned)p.tiles_m * (unsigned)p.tiles_n * (unsigned)p.k_splits;
   if (launch_kernel(kfn, dim3(grid), dim3(TL::NT), lds, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
@@ -191,14 +191,8 @@ template <int BPRE, int GLU>
 int launch_w512_kernel(const GroupParams& p, hipStream_t stream) {
   typedef W512 T;
   auto kfn = cascmm_w512_kernel<BPRE, GLU>;
-  static bool lds_set[kMaxDevices] = {false};
-  const int d = device_index();
-  if (d < 0) return CASCMM_ERR_LAUNCH;
-  if (!lds_set[d]) {
-    if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
-      return CASCMM_ERR_LAUNCH;
-    lds_set[d] = true;
-  }
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
   const unsigned grid = (unsigned)(p.tiles_m * p.tiles_n);
   if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) != hipSuccess) return CASCMM_ERR_LAUNCH;
   return CASCMM_OK;
@@ -225,14 +219,8 @@ int launch_wavek(const GroupParams& p, hipStream_t stream) {
   if (p.N % T::BN != 0 || p.K % T::BK != 0) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
   auto kfn = cascmm_wavek_kernel<NB>;
-  static bool lds_set[kMaxDevices] = {false};
-  const int d = device_index();
-  if (d < 0) return CASCMM_ERR_LAUNCH;
-  if (!lds_set[d]) {
-    if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
-      return CASCMM_ERR_LAUNCH;
-    lds_set[d] = true;
-  }
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
   GroupParams q = p;
   q.tiles_m = (p.M + T::BM - 1) / T::BM;
   q.tiles_n = p.N / T::BN;
@@ -284,14 +272,8 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
   if (f8k64_slot_bytes(p.M, p.K) > 0x7FFFFFFF || f8k64_slot_bytes(p.N, p.K) > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
   auto kfn = cascmm_f8k64_kernel<MT>;
-  static bool lds_set[kMaxDevices] = {false};
-  const int d = device_index();
-  if (d < 0) return CASCMM_ERR_LAUNCH;
-  if (!lds_set[d]) {
-    if (hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES) != hipSuccess)
-      return CASCMM_ERR_LAUNCH;
-    lds_set[d] = true;
-  }
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
   u32x4* a_slots = (u32x4*)p.workspace;
   const u32x4* b_slots = (const u32x4*)p.B[0];
   char* ws_next = (char*)p.workspace + f8k64_up(f8k64_slot_bytes(p.M, p.K));

@@ -57,6 +57,9 @@ class Attention(nn.Module):
     Linear; after :func:`fuse_kv_projections` the key and value come from one ``to_kv`` module, or
     (self-attention, ``fuse_q``) query, key and value from one ``to_qkv`` module."""
 
+    #: this forward knows ``to_kv`` / ``to_qkv``: the mark :func:`fuse_kv_projections` looks for
+    consumes_fused_projections = True
+
     def __init__(self, query_dim: int, cross_dim: Optional[int], heads: int):
         super().__init__()
         self.heads = heads
@@ -308,8 +311,12 @@ def synthetic_inputs(model: SDXLUNetSkeleton, *, batch: int = 2, latent: int = 1
 # patchers beyond the reference's Linear walk, and the record of what a forward pass routes
 # ---------------------------------------------------------------------------------------------
 def fuse_kv_projections(model: nn.Module, *, cache_cross: bool = False, fuse_q: bool = False, **cascade_kwargs) -> nn.Module:
-    """Every attention module with ``to_k`` / ``to_v`` Linear children gets one ``to_kv``
-    (:class:`BasedXLFusedKV`) instead, as basedxl/modules/attn.py:16-39 does; with ``cache_cross``
+    """Every attention module with ``to_k`` / ``to_v`` Linear children WHOSE FORWARD IS KNOWN TO READ
+    THE FUSED MODULES (class attribute ``consumes_fused_projections``, as :class:`Attention` here has)
+    gets one ``to_kv`` (:class:`BasedXLFusedKV`) instead, as basedxl/modules/attn.py:16-39 does by
+    wrapping the attention module in one of its own.  Any other attention module (a diffusers
+    ``Attention``, whose processor calls ``attn.to_k`` / ``attn.to_v``) keeps its three Linear children
+    for the plain walk of patch_linear_layers: removing them would break its forward.  With ``cache_cross``
     the cross-attention modules (``is_cross``) keep their result like attn.py:57,74-78.  With
     ``fuse_q`` the self-attention modules (not ``is_cross``: query, key and value read the same tokens)
     get one ``to_qkv`` (:class:`BasedXLFusedQKV`) for all three.  Call it BEFORE patch_linear_layers
@@ -317,6 +324,8 @@ def fuse_kv_projections(model: nn.Module, *, cache_cross: bool = False, fuse_q: 
     for module in list(model.modules()):
         to_q, to_k, to_v = getattr(module, "to_q", None), getattr(module, "to_k", None), getattr(module, "to_v", None)
         if not (isinstance(to_k, nn.Linear) and isinstance(to_v, nn.Linear)):
+            continue
+        if not getattr(module, "consumes_fused_projections", False):
             continue
         is_cross = bool(getattr(module, "is_cross", False))
         if (fuse_q and not is_cross and hasattr(module, "is_cross") and isinstance(to_q, nn.Linear)

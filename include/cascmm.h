@@ -105,8 +105,15 @@ int cascmm_gemm_variant(const void* A, const void* B, void* C, const void* bias,
  * partial results than that returns CASCMM_ERR_SCRATCH_LIMIT (nothing is launched).  All calls on one GPU share the buffer: calls that may overlap in time on
  * one GPU (different streams, or graphs replayed concurrently) race on it and must be ordered by the
  * caller.  Nothing in the buffer needs initialisation between calls.
+ * The device address of the buffer is looked up once per GPU, on the first call there or by cascmm_init;
+ * a caller that records its first call on a GPU into a graph calls cascmm_init() before the capture
+ * (with that GPU current), so that the lookup is not part of it.
  */
 #define CASCMM_NOALLOC_SCRATCH_BYTES (8u << 20)
+/* Optional set-up for the current GPU (no counterpart in the reference): resolves what the library
+ * otherwise resolves on first use there -- today the address of cascmm_gemm_noalloc's built-in buffer.
+ * Allocates nothing, launches nothing; CASCMM_ERR_LAUNCH when no GPU is current. */
+int cascmm_init(void);
 int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
                         int64_t M, int64_t N, int64_t K,
                         int64_t lda, int64_t ldb, int64_t ldc,

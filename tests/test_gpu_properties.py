@@ -240,6 +240,52 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
             assert torch.equal(a, b), (rep, i)
 
 
+def test_a_captured_graph_keeps_its_workspace_when_a_later_call_needs_a_larger_one(gpu_device):
+    """A graph has the address of the K-split workspace baked into its launches.  An eager call with a
+    larger problem makes the package replace that buffer; the old one must stay the package's, or the
+    caching allocator hands it to the next tensor and the graph's replays write partial results into
+    it.  Capture a small K-split GEMM, run a larger one eagerly, allocate tensors of the old buffer's
+    size class, replay: the replay equals the eager result and none of the new tensors was touched."""
+    from basedxl_amd.cascaded_lowp_matmul import _retired_capture_buffers, _workspaces
+
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(9)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+    # start from a capture buffer of exactly this problem's need, so that the next problem must grow it
+    x1, w1 = rn(154, 2048), rn(2048, 640) * 0.02          # skinny: K split with partial results in the workspace
+    need1 = _lib.lib().cascmm_workspace_bytes(154, 640, 2048, _lib.DT_F32, _lib.FMT_BF16, 2, _lib.PROD_TRI)
+    assert need1 > 0
+    saved = dict(_workspaces)
+    _workspaces.clear()
+    try:
+        want1 = cascaded_lowp_matmul(x1, w1)              # eager warm-up sizes the capture buffer
+        torch.cuda.synchronize()
+        old = _workspaces[(0, "capture")]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out1 = cascaded_lowp_matmul(x1, w1)
+        x2, w2 = rn(1024, 5120), rn(5120, 1280) * 0.02    # needs 4 x 1024 x 1280 x 4 bytes: far more
+        cascaded_lowp_matmul(x2, w2)
+        torch.cuda.synchronize()
+        new = _workspaces[(0, "capture")]
+        assert new.data_ptr() != old.data_ptr() and new.numel() > old.numel()
+        old_ptr, old_bytes = old.data_ptr(), old.numel()
+        del old
+        # tensors of the old buffer's size: the allocator would reuse a freed block of that size at once
+        canaries = [torch.full((old_bytes,), 0x5A, dtype=torch.uint8, device=dev) for _ in range(4)]
+        assert all(c.data_ptr() != old_ptr for c in canaries)
+        for rep in range(2):
+            out1.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out1, want1), rep
+            assert all(bool((c == 0x5A).all()) for c in canaries)
+    finally:
+        _workspaces.clear()
+        _workspaces.update(saved)
+    assert _retired_capture_buffers
+
+
 def test_operands_beyond_two_gib_are_addressed_correctly(gpu_device):
     """The fast kernels address rows through 32-bit offsets from a per-tile buffer descriptor, the
     bounds-checked ones through 64-bit pointers: a left operand and a result of 2.3 GB each (row offsets

@@ -70,6 +70,43 @@ def test_fused_kv_weight_is_the_concatenation():
         BasedXLFusedKV(to_k, torch.nn.Linear(12, 4))
 
 
+class _ForeignAttention(torch.nn.Module):
+    """An attention module of somebody else's (like diffusers'): its forward reads to_q / to_k / to_v."""
+
+    def __init__(self):
+        super().__init__()
+        self.to_q = torch.nn.Linear(8, 8, bias=False)
+        self.to_k = torch.nn.Linear(8, 8, bias=False)
+        self.to_v = torch.nn.Linear(8, 8, bias=False)
+
+    def forward(self, x):
+        return self.to_q(x) + self.to_k(x) + self.to_v(x)
+
+
+def test_fusion_leaves_attention_modules_it_does_not_know_alone():
+    """The key / value fusion replaces children that only the skeleton's own forward knows how to use;
+    a foreign attention module must come out of patch_unet with to_q / to_k / to_v still there (routed
+    one by one, as basedxl/unet.py:81-87 does) and a forward that still runs."""
+    from basedxl_amd.unet import patch_unet
+    from basedxl_amd.utils import BasedXLConfig
+    from basedxl_amd.unet_skeleton import Attention, fuse_kv_projections
+
+    model = torch.nn.ModuleDict({"foreign": _ForeignAttention(), "own_self": Attention(8, None, 2),
+                                 "own_cross": Attention(8, 12, 2)})
+    want = model["foreign"](torch.ones(3, 8))
+    fuse_kv_projections(model, fuse_q=True)
+    f = model["foreign"]
+    assert all(isinstance(getattr(f, n), torch.nn.Linear) for n in ("to_q", "to_k", "to_v"))
+    assert not hasattr(f, "to_kv") and not hasattr(f, "to_qkv")
+    assert torch.equal(f(torch.ones(3, 8)), want)                       # its forward still finds its children
+    assert hasattr(model["own_self"], "to_qkv") and not hasattr(model["own_self"], "to_k")
+    assert hasattr(model["own_cross"], "to_kv") and hasattr(model["own_cross"], "to_q")
+    # the install hook routes the foreign module's three projections through the plain Linear walk
+    model2 = torch.nn.ModuleDict({"foreign": _ForeignAttention()})
+    patch_unet(model2, BasedXLConfig(fp16_acc_matmul=True))
+    assert all(isinstance(getattr(model2["foreign"], n), BasedXLLowPLinear) for n in ("to_q", "to_k", "to_v"))
+
+
 # ---------------------------------------------------------------------------------- GPU
 
 

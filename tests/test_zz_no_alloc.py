@@ -39,16 +39,53 @@ def test_noalloc_entry_equals_the_workspace_entry_on_consecutive_calls(gpu_devic
         st = _call(l, l.cascmm_gemm, a, b, want, bias, lambda s: (ws.data_ptr(), ws.numel(), s))
         assert st == 0, l.cascmm_strerror(st)
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+        # the driver's own count of free device memory sees any allocation, the library's included
+        # (torch's counters only see torch's); the look-up of the buffer's address comes first, as a
+        # caller that records its first call into a graph would do it
+        assert l.cascmm_init() == 0
+        before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
         st = _call(l, l.cascmm_gemm_noalloc, a, b, got, bias, lambda s: (s,))
         assert st == 0, l.cascmm_strerror(st)
         torch.cuda.synchronize()
-        assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
+        assert (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == before
         assert torch.equal(got, want)
         exp = oc.fp64_matmul(a_cpu, b_cpu) + bias.cpu().double()
         ek = oc.error_metrics(got.cpu(), exp)
         eo = oc.error_metrics(oc.cascade_matmul_ref(a_cpu, b_cpu) + bias.cpu(), exp)
         assert ek["rel_fro"] <= 1.25 * eo["rel_fro"] and ek["max_abs"] <= 1.25 * eo["max_abs"]
+
+
+def test_noalloc_entry_records_into_a_graph_and_replays(gpu_device):
+    """What the entry point is for: a call under stream capture.  The capture records the library's
+    kernels and nothing else (no allocation: free device memory is the same before and after), and
+    every replay, with fresh operand values and eager work in between, equals the eager cascmm_gemm."""
+    l = _lib.lib()
+    M, K, N = 154, 2048, 640
+    g = torch.Generator(device="cuda:0").manual_seed(4)
+    a = torch.randn(M, K, device=gpu_device, generator=g)
+    b = torch.randn(K, N, device=gpu_device, generator=g) * 0.02
+    got = torch.empty(M, N, device=gpu_device)
+    want = torch.empty(M, N, device=gpu_device)
+    need = l.cascmm_workspace_bytes(M, N, K, _lib.DT_F32, _lib.FMT_BF16, 2, _lib.PROD_TRI)
+    assert 0 < need <= SCRATCH_BYTES
+    ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+    assert l.cascmm_init() == 0                      # the address look-up stays outside the capture
+    assert _call(l, l.cascmm_gemm_noalloc, a, b, got, None, lambda s: (s,)) == 0     # eager warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    free_before = torch.cuda.mem_get_info()[0]
+    with torch.cuda.graph(graph):
+        st = _call(l, l.cascmm_gemm_noalloc, a, b, got, None, lambda s: (s,))
+    assert st == 0, l.cascmm_strerror(st)
+    assert torch.cuda.mem_get_info()[0] == free_before
+    for rep in range(3):
+        a.copy_(torch.randn(M, K, device=gpu_device, generator=g) * (1.0 + rep))
+        got.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert _call(l, l.cascmm_gemm, a, b, want, None, lambda s: (ws.data_ptr(), ws.numel(), s)) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
 
 
 def test_noalloc_entry_refuses_what_exceeds_its_scratch_and_runs_what_needs_none(gpu_device):
