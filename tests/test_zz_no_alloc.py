@@ -57,7 +57,8 @@ def test_noalloc_entry_equals_the_workspace_entry_on_consecutive_calls(gpu_devic
 
 def test_noalloc_entry_records_into_a_graph_and_replays(gpu_device):
     """What the entry point is for: a call under stream capture.  The capture records the library's
-    kernels and nothing else (no allocation: free device memory is the same before and after), and
+    kernels (that the call itself allocates nothing is checked on the eager calls above: the graph
+    object and its memory pool are the caller's and do take device memory), and
     every replay, with fresh operand values and eager work in between, equals the eager cascmm_gemm."""
     l = _lib.lib()
     M, K, N = 154, 2048, 640
@@ -73,11 +74,9 @@ def test_noalloc_entry_records_into_a_graph_and_replays(gpu_device):
     assert _call(l, l.cascmm_gemm_noalloc, a, b, got, None, lambda s: (s,)) == 0     # eager warm-up
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    free_before = torch.cuda.mem_get_info()[0]
     with torch.cuda.graph(graph):
         st = _call(l, l.cascmm_gemm_noalloc, a, b, got, None, lambda s: (s,))
     assert st == 0, l.cascmm_strerror(st)
-    assert torch.cuda.mem_get_info()[0] == free_before
     for rep in range(3):
         a.copy_(torch.randn(M, K, device=gpu_device, generator=g) * (1.0 + rep))
         got.fill_(float("nan"))
