@@ -45,6 +45,13 @@ SIGNATURES = {
     "cascmm_select_variant_prepared": (c_int, [c_int] + [c_int64] * 5 + [c_int] * 4),
     "cascmm_select_variant_glu": (c_int, [c_int64] * 6 + [c_int] * 4),
     "cascmm_gemm_glu": (c_int, [c_void_p] * 4 + [c_int64] * 6 + [c_int] * 4 + [c_void_p, c_int]),
+    "cascmm_left_slots_bytes": (c_size_t, [c_int64, c_int64]),
+    "cascmm_prepare_left": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "cascmm_prepare_weight_chained": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "cascmm_gemm_glu_chained": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                        c_int64, c_void_p]),
+    "cascmm_chained_supported": (c_int, [c_int64, c_int64, c_int64]),
+    "cascmm_gemm_chained": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "cascmm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int]),
     "cascmm_select_variant": (c_int, [c_int64] * 6 + [c_int] * 4),
     "cascmm_select_variant_grouped": (c_int, [c_int] + [c_int64] * 6 + [c_int] * 4),

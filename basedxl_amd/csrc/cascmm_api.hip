@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "cascmm_variants.h"
+#include "cascmm_slotk_kernel.h"
 
 namespace cascmm {
 
@@ -28,6 +29,8 @@ static const std::vector<VariantDesc>& table() {
     v.insert(v.end(), p, p + n);
     p = variants_bpre(&n);
     v.insert(v.end(), p, p + n);
+    p = variants_chain(&n);
+    v.insert(v.end(), p, p + n);
     return v;
   }();
   return t;
@@ -47,6 +50,7 @@ struct Problem {
   int dtype, fmt, terms, products;
   bool bpre = false;  // B is a prepared (already split) weight buffer
   bool glu = false;   // gated epilogue: B prepared by cascmm_prepare_weight_glu, C has N / 2 columns
+  bool glu_slots = false;   // ... written as the left operand slots of the next GEMM (large-tile kernel only)
 };
 
 // Three fp8 terms with K a multiple of 64 are prepared for the fp8-rate kernel: [term][K/16][N] slots
@@ -103,7 +107,10 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
                               (!q.bpre && q.K * q.ldb * 4 > INT32_MAX) || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
     return false;
   if (v.kind == KIND_WAVEK && (q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX || q.K == 0)) return false;
+  if (v.kind == KIND_SLOTK && (q.K < 64 || q.N % 32 != 0 || q.M * q.lda * 4 > INT32_MAX || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
+    return false;
   if (q.glu && !v.glu) return false;
+  if (q.glu_slots && v.kind != KIND_W512) return false;
   return true;
 }
 
@@ -147,6 +154,9 @@ static const TunedCost kTuned[] = {
     {"t64x256x32_w1x4x1_d3_bf16x2_tri_bpre", 1.250, 5.89, 0.80, 0.50},
     {"t256x160x32_w4x1x1_d2_bf16x2_tri_bpre", 2.837, 12.00, 0.60, 0.50},
     {"t256x320x32_w512_bf16x2_tri_bpre", 5.50, 16.0, 1.00, 1.00},
+    // K split over the waves: a round of 256 tiles costs 0.012 us per k + 8 us, and rounds do not overlap
+    // (2048 x {1280, 5120} x 1280: 23.3 / 69.3 us; 8192 x 640 x 640, two rounds: 31.9 us; 1024 x 1280 x 1280: 19.1 us)
+    {"k64x160x16_wk4_bf16x2_tri_bpre", 0.767, 8.0, 0.65, 0.95},
 };
 
 constexpr int kMaxTileSplits = 4;
@@ -235,7 +245,7 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     // columns: measured about a quarter slower (32768 x 640 x 320 on the 128-wide tile)
     const double edge = (q.N % v.BN != 0 || q.M % v.BM != 0) ? 1.25 : 1.0;
     double best = edge * rounds * ((double)q.K / 64.0 * t.step64_us + t.fixed_us);
-    if (count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0 && !q.glu) {
+    if (v.kind == KIND_TILE && count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0 && !q.glu) {
       const int64_t ksteps = (q.K + v.BK - 1) / v.BK;
       for (int sp = 2; sp <= kMaxTileSplits; ++sp) {
         if (ksteps % sp != 0 || ksteps / sp < 4 || tiles * sp > kNumCUs) continue;
@@ -318,7 +328,7 @@ static int select_variant(const Problem& q, bool fast, int count, size_t ws_byte
   static std::mutex mu;
   static std::unordered_map<SelectKey, SelectHit, SelectKeyHash> memo;
   const SelectKey key{q.M, q.N, q.K, ws_bytes, q.dtype, q.fmt, q.terms, q.products, count,
-                      (fast ? 1 : 0) | (q.bpre ? 2 : 0) | (q.glu ? 4 : 0) | (beyond_i32(q.M, q.lda, 4) ? 8 : 0) |
+                      (fast ? 1 : 0) | (q.bpre ? 2 : 0) | (q.glu ? 4 : 0) | (q.glu_slots ? 64 : 0) | (beyond_i32(q.M, q.lda, 4) ? 8 : 0) |
                           (beyond_i32(q.K, q.ldb, 4) ? 16 : 0) | (beyond_i32(q.ldc, 1024, 1) ? 32 : 0)};
   {
     std::lock_guard<std::mutex> lock(mu);
@@ -449,8 +459,9 @@ static int launch_split(const void* x, float* out, int64_t n, int terms, int ten
 // out[(plane * K/8 + kg) * N + n].
 template <int IODT, int FMT, int TERMS>
 __global__ __launch_bounds__(256) void prepare_weight_kernel(const void* B, int K, int N, int64_t ldb,
-                                                            const int32_t* tensor_exp, u32x4* out, int glu) {
+                                                            const int32_t* tensor_exp, u32x4* out, int flags) {
   typedef typename IoType<IODT>::T T;
+  const int glu = flags & 1, chained = flags & 2;
   const int kgs = (K + 7) / 8;
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (int64_t)kgs * N) return;
@@ -461,7 +472,9 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(const void* B, int 
   float r[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const int k = kg * 8 + e;
+    // chained: the k order of the left operand's slots as the gated store writes them (see
+    // cascmm_prepare_left): positions 0..3 are k = 16 t + 4 g + 0..3 and 4..7 the same + 8, kg = 2 t + g
+    const int k = chained ? 16 * (kg >> 1) + 8 * (e >> 2) + 4 * (kg & 1) + (e & 3) : kg * 8 + e;
     r[e] = k < K ? IoType<IODT>::load((const T*)B + (int64_t)k * ldb + src) : 0.f;
   }
   constexpr int PL = Lowp<FMT>::planes(TERMS);
@@ -630,7 +643,7 @@ static int gemm_impl(int count, const void* const* A, const void* const* B, void
   p.workspace_bytes = workspace_bytes;
   p.k_splits = v.kind == KIND_TILE ? splits : 1;
   p.tensor_exps = q.fmt == CASCMM_FMT_FP8 ? tensor_exps : nullptr;
-  p.glu = q.glu ? 1 : 0;
+  p.glu = q.glu_slots ? 2 : (q.glu ? 1 : 0);
   p.exps_dyn = exps_dyn;
   p.b_exp_src = b_exp_src;
   for (int i = 0; i < count; ++i) {
@@ -1033,6 +1046,76 @@ int cascmm_selftest(void) {
   for (size_t i = 0; i < t.size(); ++i)
     for (size_t j = i + 1; j < t.size(); ++j) bad += strcmp(t[i].name, t[j].name) == 0 ? 1 : 0;
   return bad;
+}
+
+// ---- chained feed-forward: both operands as slots -------------------------------------------------
+size_t cascmm_left_slots_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || K % 16 != 0) return 0;
+  int64_t mk = 0, bytes = 0;
+  if (__builtin_mul_overflow(M, K, &mk) || __builtin_mul_overflow(mk, (int64_t)4, &bytes)) return 0;
+  return (size_t)bytes;
+}
+
+int cascmm_prepare_left(const void* A, int64_t M, int64_t K, int64_t lda, void* out, size_t out_bytes, void* stream) {
+  if (M < 0 || K < 0 || lda < K || K % 16 != 0) return CASCMM_ERR_BAD_SHAPE;
+  if (M > INT32_MAX || K > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (M == 0 || K == 0) return CASCMM_OK;
+  if (!A || !out) return CASCMM_ERR_NULL_POINTER;
+  if (!aligned_to(A, 16) || !aligned_to(out, 16) || lda % 4 != 0) return CASCMM_ERR_ALIGNMENT;
+  const size_t need = cascmm_left_slots_bytes(M, K);
+  if (need == 0 || need > (size_t)INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (out_bytes < need) return CASCMM_ERR_WORKSPACE;
+  return launch_prepare_left((const float*)A, (int)M, (int)K, lda, out, (hipStream_t)stream);
+}
+
+int cascmm_prepare_weight_chained(const void* B, int64_t K, int64_t N, int64_t ldb, void* out, size_t out_bytes, void* stream) {
+  if (K < 0 || N < 0 || ldb < N || K % 16 != 0) return CASCMM_ERR_BAD_SHAPE;
+  if (K > INT32_MAX || N > INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (K == 0 || N == 0) return CASCMM_OK;
+  if (!B || !out) return CASCMM_ERR_NULL_POINTER;
+  if (!aligned_to(out, 16)) return CASCMM_ERR_ALIGNMENT;
+  if (out_bytes < (size_t)prepared_bytes(K, N, CASCMM_FMT_BF16, 2)) return CASCMM_ERR_WORKSPACE;
+  return launch_prepare<CASCMM_DT_F32, CASCMM_FMT_BF16>(B, (int)K, (int)N, ldb, 2, nullptr, (u32x4*)out, (hipStream_t)stream, 2);
+}
+
+int cascmm_gemm_glu_chained(const void* A, const void* B, int b_prepared, void* out_slots, size_t out_bytes, const void* bias,
+                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* stream) {
+  if (N % 64 != 0) return CASCMM_ERR_BAD_SHAPE;
+  Problem q{M, N, K, lda, b_prepared ? N : ldb, N / 2, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, CASCMM_PROD_TRI};
+  q.bpre = b_prepared != 0;
+  q.glu = true;
+  q.glu_slots = true;
+  const int st = check_problem(q);
+  if (st != CASCMM_OK) return st;
+  if (M == 0 || N == 0) return CASCMM_OK;
+  if (!out_slots) return CASCMM_ERR_NULL_POINTER;
+  if (!aligned_to(out_slots, 16)) return CASCMM_ERR_ALIGNMENT;
+  const size_t need = cascmm_left_slots_bytes(M, N / 2);
+  if (need == 0 || need > (size_t)INT32_MAX) return CASCMM_ERR_TOO_LARGE;
+  if (out_bytes < need) return CASCMM_ERR_WORKSPACE;
+  return gemm_impl(1, &A, &B, &out_slots, bias ? &bias : nullptr, q, nullptr, nullptr, 0, (hipStream_t)stream, -1);
+}
+
+int cascmm_chained_supported(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K < 64 || K % 16 != 0 || N % 32 != 0) return 0;
+  if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
+  if (beyond_i32(M, K, 4) || beyond_i32(N, K, 4)) return 0;   // both slot buffers below 2 GiB
+  return 1;
+}
+
+int cascmm_gemm_chained(const void* Aslots, const void* Bslots, void* C, const void* bias, int64_t M, int64_t N, int64_t K,
+                        int64_t ldc, void* stream) {
+  if (M < 0 || N < 0 || K < 0 || ldc < N) return CASCMM_ERR_BAD_SHAPE;
+  if (M == 0 || N == 0) return CASCMM_OK;
+  if (!cascmm_chained_supported(M, N, K)) return CASCMM_ERR_BAD_FORMAT;
+  if (!Aslots || !Bslots || !C) return CASCMM_ERR_NULL_POINTER;
+  if (!aligned_to(Aslots, 16) || !aligned_to(Bslots, 16) || !aligned_to(C, 4) || !aligned_to(bias, 4)) return CASCMM_ERR_ALIGNMENT;
+  if (beyond_i32(ldc, SlotK::BM, 4)) return CASCMM_ERR_TOO_LARGE;
+  SlotKParams q;
+  memset(&q, 0, sizeof(q));
+  q.a = Aslots; q.b_slots = Bslots; q.C = (float*)C; q.bias = (const float*)bias;
+  q.M = (int)M; q.N = (int)N; q.K = (int)K; q.ldc = ldc;
+  return launch_slotk(q, 0, (hipStream_t)stream);
 }
 
 int cascmm_version(void) { return CASCMM_VERSION; }

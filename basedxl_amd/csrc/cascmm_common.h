@@ -344,6 +344,8 @@ struct GroupParams {
   // with v and g the entries of A x B in row m whose columns of B are, for a prepared operand (which
   // alternates 32 "value" and 32 "gate" columns), 64 j + l and 64 j + 32 + l, and for a raw operand
   // (value columns in the first half, gate columns in the second) 32 j + l and N/2 + 32 j + l.
+  // glu == 2 (large-tile kernel only): the gated result leaves as the left operand slots of the next GEMM,
+  // two bf16 terms, [term][(N / 2) / 8][M] x 16 bytes at C (see cascmm_prepare_left for the order of k)
   int glu;
   // fp8-rate kernel only: the left operand's scale exponent is found inside the launch (two kernels:
   // per-workgroup maxima, then the operand split reduces them) and written, with *b_exp_src, to

@@ -1,0 +1,83 @@
+// Instantiations and launchers of the chained feed-forward path: the GEMM whose operands are both
+// operand slots, and the pass that writes a left operand as slots (the gated store of the first GEMM
+// writes the same layout directly; this pass is its stand-alone counterpart).
+#include "cascmm_variants.h"
+#include "cascmm_slotk_kernel.h"
+
+namespace cascmm {
+
+// Thread (row, k group) reads its 8 values of A (two 16-byte pieces: positions 0..3 of the slot are
+// k = 16 t + 4 g + 0..3, positions 4..7 the same + 8, for k group 2 t + g), splits them and writes the
+// two terms' slots.  Four consecutive threads cover 32 consecutive k of one row (128 bytes read);
+// a wave writes 256-byte runs of 16 consecutive rows.
+__global__ __launch_bounds__(256) void prepare_left_kernel(const float* A, int M, int K, int64_t lda, u32x4* out) {
+  const int kgroups = K >> 3;
+  const int kg = blockIdx.y * 4 + (threadIdx.x & 3);
+  const int m = blockIdx.x * 64 + (threadIdx.x >> 2);
+  if (m >= M || kg >= kgroups) return;
+  const float* src = A + (int64_t)m * lda + 16 * (kg >> 1) + 4 * (kg & 1);
+  const f32x4 x0 = *(const f32x4*)src, x1 = *(const f32x4*)(src + 8);
+  float r[8] = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+  u32x4 t[2];
+  split8<CASCMM_FMT_BF16, 2>(r, t);
+  out[(int64_t)kg * M + m] = t[0];
+  out[((int64_t)kgroups + kg) * M + m] = t[1];
+}
+
+int launch_prepare_left(const float* A, int M, int K, int64_t lda, void* out, hipStream_t stream) {
+  const dim3 grid((unsigned)((M + 63) / 64), (unsigned)(((K >> 3) + 3) / 4));
+  return launch_kernel(prepare_left_kernel, grid, dim3(256), 0, stream, A, M, K, lda, (u32x4*)out) == hipSuccess ? CASCMM_OK
+                                                                                                                 : CASCMM_ERR_LAUNCH;
+}
+
+const void* slotk_kernel_handle(int araw) { return araw ? (const void*)cascmm_slotk_kernel<1> : (const void*)cascmm_slotk_kernel<0>; }
+
+template <int ARAW>
+static int launch_slotk_t(const SlotKParams& q, hipStream_t stream) {
+  typedef SlotK T;
+  auto kfn = cascmm_slotk_kernel<ARAW>;
+  if (const char* e = getenv("SLOTK_ABL")) {
+    if (e[0] == '1') kfn = cascmm_slotk_kernel<ARAW, 1>;
+    if (e[0] == '2') kfn = cascmm_slotk_kernel<ARAW, 2>;
+    (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+  }
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
+  SlotKParams p = q;
+  p.tiles_m = (q.M + T::BM - 1) / T::BM;
+  p.tiles_n = (q.N + T::BN - 1) / T::BN;
+  const int64_t grid = (int64_t)p.tiles_m * p.tiles_n;
+  if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  return launch_kernel(kfn, dim3((unsigned)grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) == hipSuccess ? CASCMM_OK
+                                                                                                              : CASCMM_ERR_LAUNCH;
+}
+
+int launch_slotk(const SlotKParams& q, int araw, hipStream_t stream) {
+  return araw ? launch_slotk_t<1>(q, stream) : launch_slotk_t<0>(q, stream);
+}
+
+// the variant-table face of the kernel: raw fp32 left operand, prepared right operand
+static int launch_slotk_variant(const GroupParams& p, hipStream_t stream) {
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_slotk_kernel<1>; return CASCMM_OK; }
+  if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
+  if (p.K % SlotK::BK != 0 || p.K < 64 || p.N % 32 != 0) return CASCMM_ERR_BAD_VARIANT;
+  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.N * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(SlotK::BM * 4) > 0x7FFFFFFF)
+    return CASCMM_ERR_TOO_LARGE;
+  SlotKParams q;
+  memset(&q, 0, sizeof(q));
+  q.a = p.A[0]; q.b_slots = p.B[0]; q.C = (float*)p.C[0]; q.bias = (const float*)p.bias[0];
+  q.M = p.M; q.N = p.N; q.K = p.K; q.lda = p.lda; q.ldc = p.ldc;
+  return launch_slotk_t<1>(q, stream);
+}
+
+static const VariantDesc kChainTable[] = {
+    {"k64x160x16_wk4_bf16x2_tri_bpre", KIND_SLOTK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, SlotK::BM, SlotK::BN, SlotK::BK, SlotK::NT,
+     SlotK::LDS_BYTES, true, false, &launch_slotk_variant, true, false},
+};
+
+const VariantDesc* variants_chain(int* n) {
+  *n = (int)(sizeof(kChainTable) / sizeof(kChainTable[0]));
+  return kChainTable;
+}
+
+}  // namespace cascmm

@@ -1,0 +1,299 @@
+// Two-term bf16 cascade on a prepared right operand with K split over the waves of a workgroup
+// (gfx950): the kernel of the mid-size Linear layers and of the second GEMM of a feed-forward block.
+//
+// The right operand comes as MFMA operand slots (cascmm_prepare_weight: 16 bytes = 8 k of one column
+// of one term, [term][K/8][N]): a lane's operand is one 16-byte load and 32 consecutive lanes read 512
+// contiguous bytes, so B needs no transposition through LDS.  One workgroup computes a 64 x 160 tile of
+// C; its four waves split K: wave w takes the 16-k stages w, w + 4, w + 8, ... and owns the whole tile
+// (ten 32 x 32 accumulator blocks) over them.  Nothing is shared between waves until the end, so every
+// wave streams its own operands, B straight into registers four stages deep, and the main loop has no
+// barrier.  A 2048 x 1280 result is 256 tiles, one per CU, whatever K is: no partial results through
+// memory, no second kernel.  At the end the four partial tiles meet in LDS: every wave owns two or three
+// of the ten blocks, receives the other waves' partial sums of them and adds the four in wave order
+// (deterministic), then stores its blocks with the bias.
+//
+// The left operand comes in one of two forms:
+//   ARAW = 0: operand slots as well, [term][K/8][M] (written by the gated store of the preceding GEMM
+//     or by cascmm_prepare_left): loaded like B, straight into registers; no LDS access and no VALU
+//     work in the loop.  The order of k inside a 16-k stage is whatever the two slot buffers agree on.
+//   ARAW = 1: raw fp32 rows.  A stage's 64 rows x 64 bytes go to a private LDS ring of the wave without
+//     passing registers (four `buffer_load ... lds` of 1 KB: four consecutive lanes fetch the four
+//     16-byte chunks of a row, rotated by row / 4 so that fragment reads spread over all banks), six
+//     stages ahead; the fragments of the next stage are read and split in registers between the MFMAs
+//     of the current one.
+//
+// What bounds it: a workgroup pulls (64 + 160) x 4 bytes per k through its CU's vector memory path,
+// which for 256 CUs is 84 % of what the eight L2s can deliver while the MFMAs of that k take as long.
+#pragma once
+#include <type_traits>
+
+#include "cascmm_wavek_kernel.h"
+
+namespace cascmm {
+
+struct SlotK {
+  static constexpr int BM = 64, BN = 160, BK = 16, NW = 4, NT = 256, D = 4, GROUP_M = 8;
+  static constexpr int MT = 2, NTL = 5, BLOCKS = MT * NTL;
+  static constexpr int BLOCK_BYTES = 16 * 64 * 4;                  // one wave's 32 x 32 partial block
+  static constexpr int RED_BYTES = BLOCKS * 3 * BLOCK_BYTES;       // 120 KB: every block from its three non-owners
+  static constexpr int RA = 8, A_STAGE = BM * BK * 4;              // raw A: ring of 8 stages of 4 KB per wave
+  static constexpr int RING = RA * A_STAGE;
+  static constexpr int LDS_BYTES = NW * RING > RED_BYTES ? NW * RING : RED_BYTES;   // 128 KB
+};
+
+struct SlotKParams {
+  const void* a;         // ARAW = 0: slots [2][K/8][M] x 16 bytes; ARAW = 1: fp32 [M][lda]
+  const void* b_slots;   // [2][K/8][N] x 16 bytes
+  float* C;
+  const float* bias;
+  int M, N, K;
+  int64_t lda, ldc;
+  int tiles_m, tiles_n;
+};
+
+// Host-checked: K % 16 == 0, K >= 64, N % 32 == 0, the slot buffers 16-byte aligned and below 2 GiB,
+// raw A 16-byte aligned with lda % 4 == 0 and M * lda * 4 below 2 GiB, C rows addressable with 32-bit
+// byte offsets inside a tile.
+template <int ARAW, int ABL = 0>
+__global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_slotk_kernel(const SlotKParams p) {
+  typedef SlotK T;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char slotk_smem[];
+  const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Tile order: every XCD (its own L2; workgroup ids are dealt to the XCDs round-robin) gets one
+  // contiguous range of tile ids, and ids walk GROUP_M tile rows down before moving one tile to the right:
+  // a tile's B slots are 2.5 times its A slots, so the block of tiles that share an L2 is taller than wide.
+  int tm, tn;
+  {
+    const int total = p.tiles_m * p.tiles_n, per = total >> 3;
+    int id = blockIdx.x;
+    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
+    const int group = T::GROUP_M * p.tiles_n;
+    const int gi = id / group, first = gi * T::GROUP_M;
+    const int rows = (p.tiles_m - first) < T::GROUP_M ? (p.tiles_m - first) : T::GROUP_M;
+    const int in = id - gi * group;
+    tm = first + in % rows;
+    tn = in / rows;
+  }
+  const int m0 = tm * T::BM, n0 = tn * T::BN;
+  const int kgroups = p.K >> 3;
+  const int ksteps = p.K >> 4;
+  const int n_own = (ksteps - wave + T::NW - 1) / T::NW;   // >= 1 (K >= 64)
+  // Own stage i is stage wave + 4 i of the problem.  The loop below runs in trips of D stages and has no
+  // branch inside a trip (a branch costs the compiler its count of the loads in flight, and it then waits
+  // for all of them).  A wave whose number of stages is not a multiple of D runs up to D - 1 stages past
+  // its last one: their slot loads point beyond the end of the buffers and return zeros, whose products
+  // add nothing (raw A: the last stage again, times the zero slots of B).
+  auto step_of = [&](int i) { return wave + T::NW * (i < n_own ? i : n_own - 1); };
+
+  // ---- right operand: lane (l31, g) reads k group 2 step + g, column block ni 512 bytes further ----
+  const i32x4 rb = make_rsrc(p.b_slots, (int64_t)2 * kgroups * p.N * 16);
+  const int vb = (g * p.N + n0 + l31) * 16;
+  const int b_term = kgroups * p.N * 16;   // from term 0 to term 1
+  const int b_step = 2 * p.N * 16;         // from one 16-k stage to the next
+  u32x4 Br[T::D][T::NTL][2];               // [ring buffer][column block][term]
+  const int b_end = 2 * b_term;            // the buffer's size: every offset from there on is outside
+  auto issue_b = [&](int i, int buf, int ni) {
+    const int base = i < n_own ? (wave + T::NW * i) * b_step : b_end;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      Br[buf][ni][t] = __builtin_bit_cast(u32x4, llvm_raw_buffer_load_v4f32(rb, vb + ni * 512, base + t * b_term, 0));
+  };
+
+  // ---- left operand as slots ------------------------------------------------------------------------
+  const i32x4 ra = make_rsrc(p.a, ARAW ? (int64_t)16 : (int64_t)2 * kgroups * p.M * 16);
+  const int va = (g * p.M + m0 + l31) * 16;
+  const int a_term = kgroups * p.M * 16, a_step = 2 * p.M * 16;
+  u32x4 Ar[ARAW ? 2 : T::D][T::MT][2];     // slots: [ring buffer][row block][term]; raw: [stage parity] after the split
+  auto issue_a1 = [&](int i, int buf, int mi, int t) {
+    const int base = i < n_own ? (wave + T::NW * i) * a_step : 2 * a_term;
+    Ar[buf][mi][t] = __builtin_bit_cast(u32x4, llvm_raw_buffer_load_v4f32(ra, va + mi * 512, base + t * a_term, 0));
+  };
+
+  // ---- left operand raw -----------------------------------------------------------------------------
+  // rows past M read as zero: the buffer ends with row M - 1
+  const int64_t a_bytes = ((int64_t)(p.M - 1) * p.lda + p.K) * 4;
+  const __amdgpu_buffer_rsrc_t rar =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, ARAW ? (int)(a_bytes > 0x7FFFFFFF ? 0x7FFFFFFF : a_bytes) : 0, 0x00020000);
+  unsigned char* ring = slotk_smem + wave * T::RING;
+  // load j of a stage: rows 16 j + lane / 4, LDS position 4 row + pos holds chunk (pos - row / 4) mod 4
+  const int dma_voff = (int)(((int64_t)(m0 + (lane >> 2)) * p.lda + (((lane & 3) - (lane >> 4)) & 3) * 4) * 4);
+  const int dma_rows16 = (int)p.lda * 64;   // bytes from one load's rows to the next one's
+  auto dma_a = [&](int i, int j) {
+    wavek_load_lds(rar, ring + (i & (T::RA - 1)) * T::A_STAGE + j * 1024, dma_voff, step_of(i) * (T::BK * 4) + j * dma_rows16);
+  };
+  // fragment of lane (l31, g), row block mi: row 32 mi + l31, chunks 2 g and 2 g + 1 at their rotated places
+  const int a_frag0 = l31 * 64 + ((2 * g + (l31 >> 2)) & 3) * 16;
+  const int a_frag1 = l31 * 64 + ((2 * g + 1 + (l31 >> 2)) & 3) * 16;
+  f32x4 X[T::MT][2];   // raw fragments of the next stage on their way to the split
+  auto read_a = [&](int i, int mi) {
+    const unsigned char* st = ring + (i & (T::RA - 1)) * T::A_STAGE + mi * 2048;
+    X[mi][0] = *(const f32x4*)(st + a_frag0);
+    X[mi][1] = *(const f32x4*)(st + a_frag1);
+  };
+  auto split_a = [&](int buf, int mi) {
+    float r[8] = {X[mi][0][0], X[mi][0][1], X[mi][0][2], X[mi][0][3], X[mi][1][0], X[mi][1][1], X[mi][1][2], X[mi][1][3]};
+    u32x4 t[2];
+    split8<CASCMM_FMT_BF16, 2>(r, t);
+    Ar[buf][mi][0] = t[0];
+    Ar[buf][mi][1] = t[1];
+  };
+
+  // ---- prologue ---------------------------------------------------------------------------------------
+  // B: stages 0 .. D - 2 whole, of stage D - 1 the column blocks 0 .. 3 (its last column block is loaded
+  // during stage 0, like that of every later stage: see the loop).  A as slots: stages 0 .. D - 2.
+  // A raw: stage 0 first, so that its fragments can be read while everything else is still in flight,
+  // then stages 1 .. RA - 3.
+  f32x16 acc[T::MT][T::NTL];
+  if (ARAW) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma_a(0, j);
+    __builtin_amdgcn_sched_barrier(0);   // (the wait below counts on these four being the oldest)
+  }
+#pragma unroll
+  for (int d = 0; d < T::D; ++d) {
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni)
+      if (d < T::D - 1 || ni < T::NTL - 1) issue_b(d, d, ni);
+    if (!ARAW && d < T::D - 1) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) issue_a1(d, d, x >> 1, x & 1);
+    }
+  }
+  constexpr int AHEAD = T::RA - 2;   // raw A: stage i + AHEAD is requested during stage i
+  if (ARAW) {
+#pragma unroll
+    for (int d = 1; d < AHEAD; ++d)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dma_a(d, j);
+  }
+#pragma unroll
+  for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
+  if (ARAW) {
+    // everything requested after stage 0's four loads may still be in flight
+    constexpr int LATER = (T::D - 1) * 2 * T::NTL + 2 * (T::NTL - 1) + 4 * (AHEAD - 1);   // 58
+    static_assert(LATER <= 63, "the wait counter has six bits");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (LATER & 0xF) | ((LATER >> 4) << 14));
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi);
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi) split_a(0, mi);
+  }
+
+  auto mfma = [&](u32x4 a, u32x4 b, f32x16 c) -> f32x16 {
+    if (ABL == 1) { asm volatile("" ::"v"(a), "v"(b)); return c; }
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  };
+  // Stage i multiplies B from ring buffer i % D.  Its six MFMAs of column block ni are interleaved with
+  // loads into registers that are free by then: the two slots of column block ni - 1 of stage i + D
+  // (same buffer; ni = 0: the last column block of the previous buffer's next stage) and, A as slots,
+  // one of the four row slots of the previous buffer's next stage, i + D - 1.  A raw: one of the four
+  // loads of stage i + AHEAD into the ring (its place was last read during stage i - 3), and the
+  // fragments of stage i + 1, which landed long ago (requested 70 loads back, and no more than 63 can be
+  // outstanding; the wait the compiler puts in front of the stage's first MFMA for B is stricter still).
+  for (int i0 = 0; i0 < n_own; i0 += T::D) {
+#pragma unroll
+    for (int u = 0; u < T::D; ++u) {
+      const int i = i0 + u;
+      constexpr int P = T::D - 1;               // (u + P) % D: the previous stage's buffer
+      const int ab = ARAW ? (u & 1) : u;        // where this stage's A operands are
+#pragma unroll
+      for (int ni = 0; ni < T::NTL; ++ni) {
+        // products lo.hi, hi.lo, hi.hi: smallest first, consecutive MFMAs on different accumulators
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][1], Br[u][ni][0], acc[mi][ni]);
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], Br[u][ni][1], acc[mi][ni]);
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], Br[u][ni][0], acc[mi][ni]);
+        if (ABL != 2) {
+          if (ni == 0) issue_b(i + P, (u + P) % T::D, T::NTL - 1);
+          else issue_b(i + T::D, u, ni - 1);
+          if (ni < 4) {
+            if (ARAW) dma_a(i + AHEAD, ni);
+            else issue_a1(i + P, (u + P) % T::D, ni >> 1, ni & 1);
+          }
+        }
+        if (ARAW) {
+          if (ni < T::MT) read_a(i + 1, ni);
+          if (ni >= 1 && ni <= T::MT) split_a(ab ^ 1, ni - 1);
+        }
+        // two MFMAs, one load, three times (the last block has two loads)
+#pragma unroll
+        for (int x = 0; x < (ni < 4 ? 3 : 2); ++x) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        if (ni == 4) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- the four partial tiles meet in LDS ---------------------------------------------------------
+  // block b = mi * 5 + ni is owned by wave b % 4; a non-owner w puts its partial block at
+  // [b][(w - owner - 1) mod 4], 16 bytes per lane and register quad
+  if (ARAW) {
+    // the area overlaps the rings: every load into them has landed and every wave has read its last fragments
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  }
+  auto reduce_and_store = [&](auto owner_tag) {
+    constexpr int W = decltype(owner_tag)::value;
+#pragma unroll
+    for (int b = 0; b < T::BLOCKS; ++b) {
+      if (b % T::NW == W) continue;
+      const int slot = ((W - b % T::NW - 1) & 3);
+      unsigned char* dst = slotk_smem + (b * 3 + slot) * T::BLOCK_BYTES + lane * 16;
+      const f32x16& v = acc[b / T::NTL][b % T::NTL];
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) *(f32x4*)(dst + r4 * 1024) = (f32x4){v[4 * r4], v[4 * r4 + 1], v[4 * r4 + 2], v[4 * r4 + 3]};
+    }
+    __syncthreads();
+    const int ldc_bytes = (int)p.ldc * 4;
+    // rows past M fall beyond the end of the buffer and are dropped
+    const i32x4 rc = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, ((int64_t)(p.M - 1 - m0) * p.ldc + (p.N - n0)) * 4);
+#pragma unroll
+    for (int b = W; b < T::BLOCKS; b += T::NW) {
+      const int mi = b / T::NTL, ni = b % T::NTL;
+      if (n0 + ni * 32 >= p.N) continue;
+      f32x16 sum;
+      // partial sums in wave order 0, 1, 2, 3: the own one at its place
+#pragma unroll
+      for (int w = 0; w < T::NW; ++w) {
+        f32x16 part;
+        if (w == W) {
+          part = acc[mi][ni];
+        } else {
+          const unsigned char* src = slotk_smem + (b * 3 + ((w - W - 1) & 3)) * T::BLOCK_BYTES + lane * 16;
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const f32x4 x = *(const f32x4*)(src + r4 * 1024);
+            part[4 * r4] = x[0]; part[4 * r4 + 1] = x[1]; part[4 * r4 + 2] = x[2]; part[4 * r4 + 3] = x[3];
+          }
+        }
+        if (w == 0) sum = part;
+        else
+#pragma unroll
+          for (int e = 0; e < 16; ++e) sum[e] += part[e];
+      }
+      const float bv = p.bias ? p.bias[n0 + ni * 32 + l31] : 0.f;
+      const int voff = (g * 4 * ldc_bytes) + (ni * 32 + l31) * 4;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          llvm_raw_buffer_store_f32(sum[4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+    }
+  };
+  if (wave == 0) reduce_and_store(std::integral_constant<int, 0>{});
+  else if (wave == 1) reduce_and_store(std::integral_constant<int, 1>{});
+  else if (wave == 2) reduce_and_store(std::integral_constant<int, 2>{});
+  else reduce_and_store(std::integral_constant<int, 3>{});
+}
+
+}  // namespace cascmm

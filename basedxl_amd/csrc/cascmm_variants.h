@@ -14,7 +14,8 @@ namespace cascmm {
 // KIND_W512: the large-tile kernel (whole 256 x 320 tiles only, one problem per launch)
 // KIND_F8K64: three fp8 terms on the fp8-rate MFMA; splits its operands into the workspace first
 // KIND_WAVEK: skinny problems in one launch, K split over the waves of a workgroup (no workspace)
-enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3, KIND_WAVEK = 4 };
+// KIND_SLOTK: prepared right operand, K split over the waves of a workgroup (64 x 160 tiles, one problem per launch)
+enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3, KIND_WAVEK = 4, KIND_SLOTK = 5 };
 constexpr int kNumCUs = 256;  // MI355X: what the cost model's constants were measured on
 constexpr int kMaxDevices = 64;
 
@@ -206,7 +207,8 @@ int launch_w512(const GroupParams& p, hipStream_t stream) {
   if (p.M % T::BM != 0 || p.N % T::BN != 0 || p.K % 32 != 0 || p.K < 32) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
-  // (the gated store is an instantiation of its own)
+  // (the gated stores are instantiations of their own; glu == 2: the result leaves as operand slots)
+  if (p.glu == 2) return launch_w512_kernel<BPRE, 2>(p, stream);
   return p.glu ? launch_w512_kernel<BPRE, 1>(p, stream) : launch_w512_kernel<BPRE, 0>(p, stream);
 }
 
@@ -373,11 +375,18 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
    LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true, false,                               \
    &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL, true>}
 
+// the chained feed-forward path (cascmm_inst_chain.hip)
+struct SlotKParams;
+int launch_slotk(const SlotKParams& q, int araw, hipStream_t stream);
+int launch_prepare_left(const float* A, int M, int K, int64_t lda, void* out, hipStream_t stream);
+const void* slotk_kernel_handle(int araw);
+
 // each instantiation unit exports its slice of the table
 const VariantDesc* variants_bf16(int* n);
 const VariantDesc* variants_fp16(int* n);
 const VariantDesc* variants_fp8(int* n);
 const VariantDesc* variants_io16(int* n);
 const VariantDesc* variants_bpre(int* n);
+const VariantDesc* variants_chain(int* n);
 
 }  // namespace cascmm

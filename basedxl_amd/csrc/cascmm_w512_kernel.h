@@ -62,6 +62,13 @@ __device__ __forceinline__ f32x16 w512_mfma_a(u32x4 a, u32x4 b, f32x16 c) {
 // fetched from N / 2 further right, so that both kinds of operand fill the same accumulator blocks.
 // (An instantiation of its own: the plain kernel stays as it is, without the scratch bytes this epilogue's
 // register allocation asks for.)
+// GLU = 2: the gated store writes its result as the LEFT OPERAND SLOTS of the next GEMM (two bf16 terms,
+// [term][(N / 2) / 8][M] x 16 bytes at C) instead of fp32.  The MFMAs then take their operands the other
+// way round, which leaves every accumulator block transposed in the registers: a lane holds one row of C
+// and four consecutive columns per register quad, i.e. half a slot per quad -- the slot of k group
+// 2 t + g holds columns 16 t + 4 g + 0..3 and 16 t + 8 + 4 g + 0..3 -- and 32 consecutive lanes write 32
+// consecutive slots, 512 contiguous bytes.  (cascmm_prepare_weight_chained gives the next GEMM's weight
+// the same order of k.)
 // BPRE = 1: the right operand comes already split (cascmm_prepare_weight: 16-byte slots of 8 k of one
 // column of one term, [term][K/8][N], below 2 GiB).  A stage then holds the same 20 KB of B as slots
 // [term][k group][320], copied by the same twenty 1 KB loads; a lane reads its two operands with two
@@ -249,8 +256,13 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
           const int prod = idx >> 2, mi = idx & 3;
           const u32x4 a = prod == 0 ? Al[mi] : Ah[mi];
           const u32x4 b = prod == 1 ? L[cur] : H[cur];
-          if (ni < 4) acc[mi][ni] = w512_mfma_a(a, b, acc[mi][ni]);
-          else w512_mfma_v(a, b, acc[mi][ni]);
+          if (GLU == 2) {   // operands swapped: the block comes out transposed
+            if (ni < 4) acc[mi][ni] = w512_mfma_a(b, a, acc[mi][ni]);
+            else w512_mfma_v(b, a, acc[mi][ni]);
+          } else {
+            if (ni < 4) acc[mi][ni] = w512_mfma_a(a, b, acc[mi][ni]);
+            else w512_mfma_v(a, b, acc[mi][ni]);
+          }
         };
         auto dl = [&](int k) {   // two load slots per block: 10 per stage, 9 used
           const int slot = ni * 2 + k;
@@ -302,7 +314,71 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   const int el31 = elane & 31, eg = elane >> 5;
   const float* bias = (const float*)p.bias[0];
   const int ldc_bytes = (int)p.ldc * 4;
-  if constexpr (GLU != 0) {
+  if constexpr (GLU == 2) {
+    // Gated store as operand slots.  Blocks are transposed: of block (mi, ni) a lane holds row 32 mi + l31
+    // and columns 8 q + 4 g + e in register 4 q + e.  Pairs of blocks as below (value j, gate j); the gate
+    // of pair 2 crosses from the right wave to the left one through LDS, same lanes and registers.
+    const int half = p.N >> 1, c0 = n0 >> 1;
+    const int kgroups = half >> 3;                                  // k groups of the next GEMM
+    float* xbuf = (float*)smem + (wave >> 1) * (T::MT * 16 * 64);
+    __builtin_amdgcn_s_barrier();
+    auto bias_at = [&](int col) { return bias ? bias[col] : 0.f; };
+    if (wave & 1) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float bg = bias_at(half + c0 + 64 + 8 * (r >> 2) + 4 * eg + (r & 3));
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) xbuf[(mi * 16 + r) * 64 + elane] = gelu_value(acc[mi][0][r] + bg);
+      }
+    }
+    __syncthreads();
+    // 4 M K2 bytes of slots, below 2 GiB (host-checked)
+    const i32x4 rc = make_rsrc(p.C[0], (int64_t)2 * kgroups * p.M * 16);
+    const int voff = (eg * p.M + m0 + wm0 + el31) * 16;             // + mi * 512
+    const int term1 = kgroups * p.M * 16;
+    auto out_pair = [&](int pair, int vb, int gb, bool gate_in_lds) {
+      const int col0 = c0 + 32 * pair;                              // first output column of the pair
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {                              // k groups 4 (col0 / 32) + 2 s2 + g
+        float bv[8], bgt[8];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          const int col = col0 + 16 * s2 + 8 * (x >> 2) + 4 * eg + (x & 3);
+          bv[x] = bias_at(col);
+          bgt[x] = gate_in_lds ? 0.f : bias_at(half + col);
+        }
+        const int soff = ((col0 >> 3) + 2 * s2) * p.M * 16;
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) {
+          float r8[8];
+#pragma unroll
+          for (int x = 0; x < 8; ++x) {
+            const int r = 8 * s2 + x;                               // register 4 q + e with q = 2 s2 + x / 4
+            const float gl = gate_in_lds ? xbuf[(mi * 16 + r) * 64 + elane] : gelu_value(acc[mi][gb][r] + bgt[x]);
+            r8[x] = (acc[mi][vb][r] + bv[x]) * gl;
+            // the slots are the split of this product ROUNDED to fp32, as a separate pass over the fp32
+            // result would split it: keep the compiler from folding the multiplication into the split's
+            // subtraction (a fused multiply-subtract would take the residual of the unrounded product)
+            asm volatile("" : "+v"(r8[x]));
+          }
+          u32x4 t[2];
+          split8<CASCMM_FMT_BF16, 2>(r8, t);
+          llvm_raw_buffer_store_v4f32(__builtin_bit_cast(f32x4, t[0]), rc, voff + mi * 512, soff, 0);
+          llvm_raw_buffer_store_v4f32(__builtin_bit_cast(f32x4, t[1]), rc, voff + mi * 512, soff + term1, 0);
+        }
+      }
+    };
+    if ((wave & 1) == 0) {
+      out_pair(0, 0, 1, false);
+      out_pair(1, 2, 3, false);
+      out_pair(2, 4, 0, true);
+    } else {
+      out_pair(3, 1, 2, false);
+      out_pair(4, 3, 4, false);
+    }
+    return;
+  }
+  if constexpr (GLU == 1) {
     // Gated store: C[m][n0 / 2 + 32 j + l] = (value j + bias) x gelu(gate j + bias), j = 0 .. 4.  The
     // left wave of a row pair holds value 0, gate 0, value 1, gate 1, value 2, the right one gate 2,
     // value 3, gate 3, value 4, gate 4: pair 2 is the only one that spans two waves; the right wave

@@ -204,6 +204,42 @@ int cascmm_gemm_glu(const void* A, const void* B, void* C, const void* bias,
                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                     int dtype, int fmt, int terms, int products, void* stream, int variant);
 
+/*
+ * Chained feed-forward: the second GEMM with BOTH operands already split.  The reference runs the two
+ * Linear layers of a feed-forward block as two independent calls of its operator
+ * (basedxl/modules/lowp_linear.py:15-20 on `ff.net.0.proj` and on `ff.net.2`, installed at
+ * basedxl/unet.py:81-87); the result of the first is written as fp32, read back, cast again.  Here the
+ * first GEMM's gated store can write its result as the operand slots of the second (two bf16 terms,
+ * fp32 tensors), and the second multiplies slots by slots:
+ *   left slots  [2 terms][K/8][M] x 16 bytes, K % 16 == 0.  Slot (term, kg, m) holds, with kg = 2 t + g,
+ *               A[m][16 t + 4 g + 0..3] at positions 0..3 and A[m][16 t + 8 + 4 g + 0..3] at 4..7 (the
+ *               order in which the gated store holds its results in registers);
+ *   weight      cascmm_prepare_weight_chained: the layout of cascmm_prepare_weight for two bf16 terms
+ *               with the same order of k inside every group of 16 (cascmm_prepared_bytes(K, N, bf16, 2)).
+ * cascmm_prepare_left writes the left slots of any fp32 A [M, K] (lda % 4 == 0, 16-byte aligned) in a
+ * pass of its own -- what the gated store does on the fly; cascmm_left_slots_bytes gives the size
+ * (4 M K).  cascmm_gemm_chained computes C = A . B (+ bias) from the two slot buffers in one launch for
+ * any M, N % 32 == 0, K % 16 == 0, K >= 64, slot buffers below 2 GiB (cascmm_chained_supported says
+ * whether a shape is taken); K is split over the waves of a workgroup, so no workspace is needed.
+ * Same terms, same three products as cascmm_gemm with two bf16 terms; the order of summation over k
+ * differs (four interleaved partial sums), as it does between any two kernel tiles.
+ * cascmm_gemm_glu_chained is the first GEMM of such a block: cascmm_gemm_glu (b_prepared == 0: raw weight
+ * W [K, N], ldb) or cascmm_gemm_prepared_glu (b_prepared != 0: B written by cascmm_prepare_weight_glu)
+ * whose gated result y [M, N / 2] leaves as left slots at out_slots (cascmm_left_slots_bytes(M, N / 2)
+ * bytes) instead of fp32.  Only the large-tile kernel has this store (M % 256 == 0, N % 320 == 0,
+ * K % 32 == 0, rows of A 16-byte aligned; CASCMM_ERR_BAD_FORMAT otherwise).  The slots hold exactly the
+ * split of the fp32 values cascmm_gemm_glu would have written.
+ */
+size_t cascmm_left_slots_bytes(int64_t M, int64_t K);
+int cascmm_gemm_glu_chained(const void* A, const void* B, int b_prepared, void* out_slots, size_t out_bytes,
+                            const void* bias, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, void* stream);
+int cascmm_prepare_left(const void* A, int64_t M, int64_t K, int64_t lda, void* out, size_t out_bytes, void* stream);
+int cascmm_prepare_weight_chained(const void* B, int64_t K, int64_t N, int64_t ldb, void* out, size_t out_bytes,
+                                  void* stream);
+int cascmm_chained_supported(int64_t M, int64_t N, int64_t K);
+int cascmm_gemm_chained(const void* Aslots, const void* Bslots, void* C, const void* bias,
+                        int64_t M, int64_t N, int64_t K, int64_t ldc, void* stream);
+
 /* Bytes of device workspace cascmm_gemm can use for this problem (0 for most shapes).
  * Counterpart of nothing in the reference (its small-M shapes fall back to torch.matmul,
  * cascaded_lowp_matmul.py:155-156); the caller allocates, as it allocates `out` (:161). */
