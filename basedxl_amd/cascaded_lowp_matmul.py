@@ -551,6 +551,162 @@ def cascaded_lowp_matmul_glu(a: torch.Tensor, b: torch.Tensor, *, bias: Optional
     return out.reshape(*batch_dims, inner)
 
 
+class LeftSlots:
+    """A left operand ``a`` ([..., K] fp32) already split into the two bf16 terms of the default cascade
+    and kept as MFMA operand slots, ``[2 terms][K / 8][M] x 16 bytes``: what the gated store of a
+    feed-forward block's first GEMM writes for the second one (:func:`cascaded_lowp_matmul_glu_chained`),
+    or what :meth:`from_tensor` makes of any fp32 tensor in a pass of its own."""
+
+    def __init__(self, slots: torch.Tensor, batch_shape, K: int):
+        self.slots, self.batch_shape, self.K = slots, tuple(batch_shape), int(K)
+        self.M = 1
+        for d in self.batch_shape:
+            self.M *= int(d)
+        self.device = slots.device
+
+    @classmethod
+    def empty(cls, batch_shape, K: int, device) -> "LeftSlots":
+        M = 1
+        for d in batch_shape:
+            M *= int(d)
+        nbytes = _lib.lib().cascmm_left_slots_bytes(M, K)
+        if nbytes == 0:
+            raise ValueError(f"left operand slots need K % 16 == 0 and M, K > 0 (got M = {M}, K = {K})")
+        return cls(torch.empty(nbytes, dtype=torch.uint8, device=device), batch_shape, K)
+
+    @classmethod
+    def from_tensor(cls, a: torch.Tensor) -> "LeftSlots":
+        _check_device_tensor(a, "a")
+        if a.dtype != torch.float32:
+            raise TypeError("left operand slots are made from fp32 tensors")
+        K = a.shape[-1]
+        a2 = a.reshape(-1, K)
+        if a2.stride(-1) != 1 or a2.data_ptr() % 16 != 0 or (a2.shape[0] > 1 and a2.stride(0) % 4 != 0):
+            a2 = a2.contiguous()
+        out = cls.empty(a.shape[:-1], K, a.device)
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        _lib.check(_lib.lib().cascmm_prepare_left(a2.data_ptr(), a2.shape[0], K, a2.stride(0) if a2.shape[0] > 1 else K,
+                                                  out.slots.data_ptr(), out.slots.numel(), stream), "cascmm_prepare_left")
+        return out
+
+    def terms(self) -> torch.Tensor:
+        """The two terms as fp32 ``[2, ..., K]`` in the natural order of k (torch arithmetic: for tests
+        and inspection, not a fast path)."""
+        M, K = self.M, self.K
+        t = self.slots.view(torch.bfloat16).view(2, K // 8, M, 8).float()
+        kg = torch.arange(K // 8, device=self.device).view(-1, 1)
+        pos = torch.arange(8, device=self.device).view(1, -1)
+        k = (16 * (kg >> 1) + 8 * (pos >> 2) + 4 * (kg & 1) + (pos & 3)).flatten()
+        out = torch.empty(2, M, K, device=self.device)
+        out[:, :, k] = t.permute(0, 2, 1, 3).reshape(2, M, K)
+        return out.reshape(2, *self.batch_shape, K)
+
+    def to_dense(self) -> torch.Tensor:
+        """hi + lo as fp32 ``[..., K]`` (the fp32 value rounded to 16 significant bits)."""
+        t = self.terms()
+        return t[0] + t[1]
+
+
+class ChainedWeight:
+    """The ``[K, N]`` fp32 weight of a feed-forward block's second Linear, split once into two bf16 terms
+    in the order of k in which :class:`LeftSlots` holds its operand (counterpart of the one-time
+    transpose at basedxl/modules/lowp_linear.py:12)."""
+
+    def __init__(self, w: torch.Tensor):
+        _check_device_tensor(w, "w")
+        if w.dim() != 2 or w.dtype != torch.float32:
+            raise ValueError("ChainedWeight needs a 2-D fp32 tensor")
+        self.K, self.N = int(w.shape[0]), int(w.shape[1])
+        if self.K % 16 != 0:
+            raise ValueError("ChainedWeight needs K % 16 == 0")
+        self.device = w.device
+        w2 = _rows(w)
+        l = _lib.lib()
+        self.slots = torch.empty(max(l.cascmm_prepared_bytes(self.K, self.N, _lib.FMT_BF16, 2), 16), dtype=torch.uint8, device=w.device)
+        stream = torch.cuda.current_stream(w.device).cuda_stream
+        _lib.check(l.cascmm_prepare_weight_chained(w2.data_ptr(), self.K, self.N, w2.stride(0) if self.K > 1 else max(self.N, 1),
+                                                   self.slots.data_ptr(), self.slots.numel(), stream), "cascmm_prepare_weight_chained")
+
+
+def chained_supported(M: int, N: int, K: int) -> bool:
+    """Whether :func:`cascaded_lowp_matmul_chained` takes the shape (``[M, K]`` slots times ``[K, N]``)."""
+    return bool(_lib.lib().cascmm_chained_supported(M, N, K))
+
+
+def cascaded_lowp_matmul_chained(a: LeftSlots, w: ChainedWeight, *, bias: Optional[torch.Tensor] = None,
+                                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``a @ w (+ bias)`` with BOTH operands already split (two bf16 terms, products hi.hi + hi.lo + lo.hi,
+    fp32 accumulation): the second GEMM of a feed-forward block, one launch, no workspace."""
+    if not isinstance(a, LeftSlots) or not isinstance(w, ChainedWeight):
+        raise TypeError("cascaded_lowp_matmul_chained takes LeftSlots and a ChainedWeight")
+    assert a.K == w.K, "Incompatible dimensions"
+    if a.device != w.device:
+        raise ValueError("operands are on different devices")
+    M, K, N = a.M, a.K, w.N
+    if out is None:
+        out = torch.empty((M, N), device=a.device, dtype=torch.float32)
+    else:
+        _check_device_tensor(out, "out")
+        if out.dtype != torch.float32 or out.numel() != M * N:
+            raise ValueError(f"out must hold {M * N} fp32 elements")
+    out2 = out if out.dim() == 2 and out.shape == (M, N) else out.view(M, N)
+    if N > 1 and out2.stride(1) != 1:
+        raise ValueError("out must have unit stride along N")
+    if bias is not None:
+        bias = _check_bias(bias, out2, N)
+    stream = torch.cuda.current_stream(a.device).cuda_stream
+    _lib.check(_lib.lib().cascmm_gemm_chained(a.slots.data_ptr(), w.slots.data_ptr(), out2.data_ptr(),
+                                              None if bias is None else bias.data_ptr(), M, N, K,
+                                              out2.stride(0) if M > 1 else max(N, 1), stream), "cascmm_gemm_chained")
+    return out.reshape(*a.batch_shape, N)
+
+
+def glu_chained_supported(a: torch.Tensor, N: int) -> bool:
+    """Whether :func:`cascaded_lowp_matmul_glu_chained` takes ``a`` ([..., K]) times a ``[K, N]`` gated
+    weight: the large-tile kernel's shapes (rows % 256, N % 320, K % 32 all zero), fp32 on the GPU."""
+    K = a.shape[-1]
+    M = a.numel() // K if K else 0
+    return bool(a.is_cuda and a.dtype == torch.float32 and M > 0 and M % 256 == 0 and N % 320 == 0 and K % 32 == 0
+                and K >= 32 and chained_supported(M, 32, N // 2) and 4 * M * (N // 2) < 2 ** 31)
+
+
+def cascaded_lowp_matmul_glu_chained(a: torch.Tensor, w, *, bias: Optional[torch.Tensor] = None,
+                                     out: Optional[LeftSlots] = None) -> LeftSlots:
+    """``h = a @ w + bias; value, gate = h.chunk(2, -1); value * gelu(gate)`` like
+    :func:`cascaded_lowp_matmul_glu`, with the result written as the :class:`LeftSlots` of the next GEMM
+    instead of fp32: ``h`` and the fp32 result never reach memory, and the next GEMM has nothing to split.
+    ``w``: the raw ``[K, 2 * inner]`` fp32 weight or a ``PreparedWeight(..., glu=True)`` of it (two bf16
+    terms).  Raises CascmmError where :func:`glu_chained_supported` is false."""
+    _check_device_tensor(a, "a")
+    prepared = isinstance(w, PreparedWeight)
+    if prepared:
+        if not w.glu or (w.lowp, w.terms) != ("bf16", 2):
+            raise ValueError("the prepared weight must be a gated one of two bf16 terms")
+        K, N, wptr = w.K, w.N, w.slots.data_ptr()
+    else:
+        _check_device_tensor(w, "w")
+        assert w.is_contiguous(), "Matrix B must be contiguous"
+        K, N, wptr = w.shape[-2], w.shape[-1], w.data_ptr()
+    assert a.shape[-1] == K, "Incompatible dimensions"
+    if a.dtype != torch.float32:
+        raise TypeError("the chained gated product takes fp32 tensors")
+    bias = _check_bias(bias, a, N)
+    batch_dims = a.shape[:-1]
+    M = batch_dims.numel()
+    a2 = _rows(a.reshape(M, K))
+    if a2.data_ptr() % 16 != 0 or (M > 1 and a2.stride(0) % 4 != 0):
+        a2 = a2.contiguous()
+    if out is None:
+        out = LeftSlots.empty(batch_dims, N // 2, a.device)
+    elif out.M != M or out.K != N // 2:
+        raise ValueError("out holds slots of another shape")
+    stream = torch.cuda.current_stream(a.device).cuda_stream
+    _lib.check(_lib.lib().cascmm_gemm_glu_chained(a2.data_ptr(), wptr, 1 if prepared else 0, out.slots.data_ptr(), out.slots.numel(),
+                                                  None if bias is None else bias.data_ptr(), M, N, K,
+                                                  a2.stride(0) if M > 1 else max(K, 1), N, stream), "cascmm_gemm_glu_chained")
+    return out
+
+
 def kernel_listing(variant: int) -> str:
     """What `dump_ptx=True` writes: the variant's name, its kernel's symbol and the kernel's gfx950
     assembly (compiled from the library's sources on first use; without a compiler the two header

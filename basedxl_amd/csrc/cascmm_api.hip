@@ -107,7 +107,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
                               (!q.bpre && q.K * q.ldb * 4 > INT32_MAX) || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
     return false;
   if (v.kind == KIND_WAVEK && (q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX || q.K == 0)) return false;
-  if (v.kind == KIND_SLOTK && (q.K < 64 || q.N % 32 != 0 || q.M * q.lda * 4 > INT32_MAX || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
+  if (v.kind == KIND_SLOTK && (q.K < 64 || q.M * q.lda * 4 > INT32_MAX || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
     return false;
   if (q.glu && !v.glu) return false;
   if (q.glu_slots && v.kind != KIND_W512) return false;
@@ -1097,7 +1097,7 @@ int cascmm_gemm_glu_chained(const void* A, const void* B, int b_prepared, void* 
 }
 
 int cascmm_chained_supported(int64_t M, int64_t N, int64_t K) {
-  if (M <= 0 || N <= 0 || K < 64 || K % 16 != 0 || N % 32 != 0) return 0;
+  if (M <= 0 || N <= 0 || K < 64 || K % 16 != 0) return 0;
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
   if (beyond_i32(M, K, 4) || beyond_i32(N, K, 4)) return 0;   // both slot buffers below 2 GiB
   return 1;

@@ -51,7 +51,7 @@ struct SlotKParams {
   int tiles_m, tiles_n;
 };
 
-// Host-checked: K % 16 == 0, K >= 64, N % 32 == 0, the slot buffers 16-byte aligned and below 2 GiB,
+// Host-checked: K % 16 == 0, K >= 64, the slot buffers 16-byte aligned and below 2 GiB,
 // raw A 16-byte aligned with lda % 4 == 0 and M * lda * 4 below 2 GiB, C rows addressable with 32-bit
 // byte offsets inside a tile.
 template <int ARAW, int ABL = 0>
@@ -256,7 +256,8 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     __syncthreads();
     const int ldc_bytes = (int)p.ldc * 4;
     // rows past M fall beyond the end of the buffer and are dropped
-    const i32x4 rc = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, ((int64_t)(p.M - 1 - m0) * p.ldc + (p.N - n0)) * 4);
+    const int64_t c_bytes = ((int64_t)(p.M - 1 - m0) * p.ldc + (p.N - n0)) * 4;
+    const i32x4 rc = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, c_bytes);
 #pragma unroll
     for (int b = W; b < T::BLOCKS; b += T::NW) {
       const int mi = b / T::NTL, ni = b % T::NTL;
@@ -281,8 +282,10 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #pragma unroll
           for (int e = 0; e < 16; ++e) sum[e] += part[e];
       }
-      const float bv = p.bias ? p.bias[n0 + ni * 32 + l31] : 0.f;
-      const int voff = (g * 4 * ldc_bytes) + (ni * 32 + l31) * 4;
+      // columns past N (a ragged last tile; their slots were some other column's) are sent beyond the end too
+      const bool inside = n0 + ni * 32 + l31 < p.N;
+      const float bv = (p.bias && inside) ? p.bias[n0 + ni * 32 + l31] : 0.f;
+      const int voff = inside ? (g * 4 * ldc_bytes) + (ni * 32 + l31) * 4 : (int)(c_bytes > 0x7FFFFFFF ? 0x7FFFFFFF : c_bytes);
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll

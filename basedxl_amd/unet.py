@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch.nn as nn
 
-from .modules import patch_linear_layers, patch_pointwise_convs
+from .modules import chain_feed_forward_layers, patch_linear_layers, patch_pointwise_convs
 from .unet_skeleton import fuse_geglu_layers, fuse_kv_projections
 from .utils import BasedXLConfig
 
@@ -26,6 +26,8 @@ def patch_unet(model: nn.Module, cfg: BasedXLConfig) -> nn.Module:
     lin_kw = dict(kw, prepared=cfg.prepared)
     if cfg.fuse_kv:
         fuse_kv_projections(model, cache_cross=cfg.cache_cross_kv, fuse_q=cfg.fuse_qkv, **lin_kw)
+    if cfg.chain_ffn:
+        chain_feed_forward_layers(model, **lin_kw)
     if cfg.fuse_geglu:
         fuse_geglu_layers(model, **lin_kw)
     patch_linear_layers(model, **lin_kw)

@@ -33,6 +33,9 @@ class BasedXLConfig:
     fuse_qkv: bool = True
     #: GEGLU gate applied in the store of the projection GEMM (weights kept split)
     fuse_geglu: bool = False
+    #: the two Linear layers of every feed-forward block as a chain: the gated store of the first GEMM
+    #: writes the operand slots of the second (fp32, two bf16 terms; other layers fall back by themselves)
+    chain_ffn: bool = False
     #: keep the weights of the Linear layers split (None: the module's default for its dtype)
     prepared: Optional[bool] = None
 
