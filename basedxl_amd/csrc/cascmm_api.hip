@@ -107,7 +107,7 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
                               (!q.bpre && q.K * q.ldb * 4 > INT32_MAX) || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
     return false;
   if (v.kind == KIND_WAVEK && (q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX || q.K == 0)) return false;
-  if (v.kind == KIND_SLOTK && (q.K < 64 || q.M * q.lda * 4 > INT32_MAX || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
+  if (v.kind == KIND_SLOTK && (q.K < 16 || q.glu || q.M * q.lda * 4 > INT32_MAX || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
     return false;
   if (q.glu && !v.glu) return false;
   if (q.glu_slots && v.kind != KIND_W512) return false;
@@ -157,6 +157,7 @@ static const TunedCost kTuned[] = {
     // K split over the waves: a round of 256 tiles costs 0.012 us per k + 8 us, and rounds do not overlap
     // (2048 x {1280, 5120} x 1280: 23.3 / 69.3 us; 8192 x 640 x 640, two rounds: 31.9 us; 1024 x 1280 x 1280: 19.1 us)
     {"k64x160x16_wk4_bf16x2_tri_bpre", 0.767, 8.0, 0.65, 0.95},
+    {"k64x160x16_wk4_bf16x2_tri", 0.80, 8.5, 0.65, 0.95},
 };
 
 constexpr int kMaxTileSplits = 4;
@@ -1097,7 +1098,7 @@ int cascmm_gemm_glu_chained(const void* A, const void* B, int b_prepared, void* 
 }
 
 int cascmm_chained_supported(int64_t M, int64_t N, int64_t K) {
-  if (M <= 0 || N <= 0 || K < 64 || K % 16 != 0) return 0;
+  if (M <= 0 || N <= 0 || K < 16 || K % 16 != 0) return 0;
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return 0;
   if (beyond_i32(M, K, 4) || beyond_i32(N, K, 4)) return 0;   // both slot buffers below 2 GiB
   return 1;

@@ -60,7 +60,7 @@ int launch_slotk(const SlotKParams& q, int araw, hipStream_t stream) {
 static int launch_slotk_variant(const GroupParams& p, hipStream_t stream) {
   if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_slotk_kernel<1>; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
-  if (p.K % SlotK::BK != 0 || p.K < 64) return CASCMM_ERR_BAD_VARIANT;
+  if (p.K % SlotK::BK != 0 || p.K < SlotK::BK) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.N * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(SlotK::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
   SlotKParams q;
@@ -70,7 +70,38 @@ static int launch_slotk_variant(const GroupParams& p, hipStream_t stream) {
   return launch_slotk_t<1>(q, stream);
 }
 
+// both operands raw fp32
+static int launch_rawk_variant(const GroupParams& p, hipStream_t stream) {
+  typedef SlotK T;
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_rawk_kernel<0>; return CASCMM_OK; }
+  if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
+  if (p.K % T::BK != 0 || p.K < T::BK || p.N % 4 != 0) return CASCMM_ERR_BAD_VARIANT;
+  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
+    return CASCMM_ERR_TOO_LARGE;
+  auto kfn = cascmm_rawk_kernel<0>;
+  if (const char* e = getenv("SLOTK_ABL")) {
+    if (e[0] == '1') kfn = cascmm_rawk_kernel<1>;
+    if (e[0] == '2') kfn = cascmm_rawk_kernel<2>;
+    (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
+  }
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
+  SlotKParams q;
+  memset(&q, 0, sizeof(q));
+  q.a = p.A[0]; q.b_slots = p.B[0]; q.C = (float*)p.C[0]; q.bias = (const float*)p.bias[0];
+  q.M = p.M; q.N = p.N; q.K = p.K; q.lda = p.lda; q.ldb = p.ldb; q.ldc = p.ldc;
+  q.tiles_m = (p.M + T::BM - 1) / T::BM;
+  q.tiles_n = (p.N + T::BN - 1) / T::BN;
+  const int64_t grid = (int64_t)q.tiles_m * q.tiles_n;
+  if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  const int c_vec = p.ldc % 4 == 0 && (uintptr_t)p.C[0] % 16 == 0;
+  return launch_kernel(kfn, dim3((unsigned)grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q, c_vec) == hipSuccess ? CASCMM_OK
+                                                                                                                     : CASCMM_ERR_LAUNCH;
+}
+
 static const VariantDesc kChainTable[] = {
+    {"k64x160x16_wk4_bf16x2_tri", KIND_SLOTK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, SlotK::BM, SlotK::BN, SlotK::BK, SlotK::NT,
+     SlotK::LDS_BYTES, true, false, &launch_rawk_variant, false, false},
     {"k64x160x16_wk4_bf16x2_tri_bpre", KIND_SLOTK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, SlotK::BM, SlotK::BN, SlotK::BK, SlotK::NT,
      SlotK::LDS_BYTES, true, false, &launch_slotk_variant, true, false},
 };

@@ -47,11 +47,11 @@ struct SlotKParams {
   float* C;
   const float* bias;
   int M, N, K;
-  int64_t lda, ldc;
+  int64_t lda, ldb, ldc;   // ldb: cascmm_rawk_kernel only (raw B)
   int tiles_m, tiles_n;
 };
 
-// Host-checked: K % 16 == 0, K >= 64, the slot buffers 16-byte aligned and below 2 GiB,
+// Host-checked: K % 16 == 0, K >= 16, the slot buffers 16-byte aligned and below 2 GiB,
 // raw A 16-byte aligned with lda % 4 == 0 and M * lda * 4 below 2 GiB, C rows addressable with 32-bit
 // byte offsets inside a tile.
 template <int ARAW, int ABL = 0>
@@ -78,13 +78,13 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int kgroups = p.K >> 3;
   const int ksteps = p.K >> 4;
-  const int n_own = (ksteps - wave + T::NW - 1) / T::NW;   // >= 1 (K >= 64)
+  const int n_own = (ksteps - wave + T::NW - 1) / T::NW;   // 0 for the last waves of a very short K: they add zeros
   // Own stage i is stage wave + 4 i of the problem.  The loop below runs in trips of D stages and has no
   // branch inside a trip (a branch costs the compiler its count of the loads in flight, and it then waits
   // for all of them).  A wave whose number of stages is not a multiple of D runs up to D - 1 stages past
   // its last one: their slot loads point beyond the end of the buffers and return zeros, whose products
   // add nothing (raw A: the last stage again, times the zero slots of B).
-  auto step_of = [&](int i) { return wave + T::NW * (i < n_own ? i : n_own - 1); };
+  auto step_of = [&](int i) { return wave + T::NW * (i < n_own ? i : (n_own > 0 ? n_own - 1 : 0)); };
 
   // ---- right operand: lane (l31, g) reads k group 2 step + g, column block ni 512 bytes further ----
   const i32x4 rb = make_rsrc(p.b_slots, (int64_t)2 * kgroups * p.N * 16);
@@ -142,16 +142,22 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // ---- prologue ---------------------------------------------------------------------------------------
   // B: stages 0 .. D - 2 whole, of stage D - 1 the column blocks 0 .. 3 (its last column block is loaded
   // during stage 0, like that of every later stage: see the loop).  A as slots: stages 0 .. D - 2.
-  // A raw: stage 0 first, so that its fragments can be read while everything else is still in flight,
-  // then stages 1 .. RA - 3.
+  // A raw: stages 0 .. AHEAD - 1 FIRST, then stage 0 of B, then the rest: the wait below names exactly the
+  // rest, so everything the first AHEAD - 1 stages read from LDS has landed when the loop starts (later
+  // stages: see the wait at the top of a stage).
+  constexpr int AHEAD = T::RA - 2;   // raw A: stage i + AHEAD is requested during stage i
   f32x16 acc[T::MT][T::NTL];
   if (ARAW) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dma_a(0, j);
-    __builtin_amdgcn_sched_barrier(0);   // (the wait below counts on these four being the oldest)
+    for (int d = 0; d < AHEAD; ++d)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dma_a(d, j);
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni) issue_b(0, 0, ni);
+    __builtin_amdgcn_sched_barrier(0);   // (the wait below counts on everything above being older than everything below)
   }
 #pragma unroll
-  for (int d = 0; d < T::D; ++d) {
+  for (int d = ARAW ? 1 : 0; d < T::D; ++d) {
 #pragma unroll
     for (int ni = 0; ni < T::NTL; ++ni)
       if (d < T::D - 1 || ni < T::NTL - 1) issue_b(d, d, ni);
@@ -160,13 +166,6 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       for (int x = 0; x < 4; ++x) issue_a1(d, d, x >> 1, x & 1);
     }
   }
-  constexpr int AHEAD = T::RA - 2;   // raw A: stage i + AHEAD is requested during stage i
-  if (ARAW) {
-#pragma unroll
-    for (int d = 1; d < AHEAD; ++d)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) dma_a(d, j);
-  }
 #pragma unroll
   for (int mi = 0; mi < T::MT; ++mi)
 #pragma unroll
@@ -174,9 +173,8 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
   if (ARAW) {
-    // everything requested after stage 0's four loads may still be in flight
-    constexpr int LATER = (T::D - 1) * 2 * T::NTL + 2 * (T::NTL - 1) + 4 * (AHEAD - 1);   // 58
-    static_assert(LATER <= 63, "the wait counter has six bits");
+    constexpr int LATER = (T::D - 2) * 2 * T::NTL + 2 * (T::NTL - 1);   // 28: B of stages 1 .. D - 1
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (LATER & 0xF) | ((LATER >> 4) << 14));
 #pragma unroll
     for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi);
@@ -193,12 +191,19 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // (same buffer; ni = 0: the last column block of the previous buffer's next stage) and, A as slots,
   // one of the four row slots of the previous buffer's next stage, i + D - 1.  A raw: one of the four
   // loads of stage i + AHEAD into the ring (its place was last read during stage i - 3), and the
-  // fragments of stage i + 1, which landed long ago (requested 70 loads back, and no more than 63 can be
-  // outstanding; the wait the compiler puts in front of the stage's first MFMA for B is stricter still).
+  // fragments of stage i + 1.  Those were requested during stage i + 1 - AHEAD; a stage issues 14 loads and
+  // nothing moves across a stage's end, so once at most 14 (AHEAD - 2) loads are outstanding at the top of
+  // stage i they have landed (the wait is explicit: the compiler does not connect a load into LDS with the
+  // read of that LDS address).
   for (int i0 = 0; i0 < n_own; i0 += T::D) {
 #pragma unroll
     for (int u = 0; u < T::D; ++u) {
       const int i = i0 + u;
+      if (ARAW) {
+        constexpr int YOUNGER = 14 * (AHEAD - 2);   // 56
+        static_assert(YOUNGER <= 63, "the wait counter has six bits");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14));
+      }
       constexpr int P = T::D - 1;               // (u + P) % D: the previous stage's buffer
       const int ab = ARAW ? (u & 1) : u;        // where this stage's A operands are
 #pragma unroll
@@ -292,6 +297,268 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         for (int e = 0; e < 4; ++e)
           llvm_raw_buffer_store_f32(sum[4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
     }
+  };
+  if (wave == 0) reduce_and_store(std::integral_constant<int, 0>{});
+  else if (wave == 1) reduce_and_store(std::integral_constant<int, 1>{});
+  else if (wave == 2) reduce_and_store(std::integral_constant<int, 2>{});
+  else reduce_and_store(std::integral_constant<int, 3>{});
+}
+
+
+// ---------------------------------------------------------------------------------------------------
+// The same design with BOTH operands raw fp32 (the operator's plain call: nothing prepared).
+//
+// A as in the kernel above (ARAW = 1).  B [K][N] row-major needs no LDS either: the 32 columns of an
+// MFMA block may be any 32 columns of the tile as long as the store knows which, so a lane takes FOUR
+// ADJACENT columns as its column of blocks 0 .. 3 (block j of lane l31 is column 4 l31 + j of the tile's
+// first 128) and column 128 + l31 as its column of block 4.  Its eight k of a stage are then eight 16-byte
+// loads (32 lanes: 512 contiguous bytes of one row of B) plus eight 4-byte loads, straight into registers,
+// four stages deep like the slots above; component j of the eight loads is the lane's operand of block
+// j, split in registers right before its MFMAs (one block ahead).  The store writes the four adjacent
+// columns of a row as 16 bytes.
+// At the end every wave owns one register quad (eight rows) of all ten blocks instead of whole blocks:
+// the same LDS traffic, and the 16-byte stores stay possible.
+// ---------------------------------------------------------------------------------------------------
+struct RawK {
+  static constexpr int D = 4, AHEAD = 5;   // B ring in registers; raw A requested this many stages ahead
+};
+
+// Host-checked: fp32 operands, K % 16 == 0, K >= 16, N % 4 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
+// aligned, M * lda * 4 and K * ldb * 4 below 2 GiB, C rows addressable with 32-bit byte offsets inside a
+// tile.  c_vec: ldc % 4 == 0 and C 16-byte aligned (16-byte stores).
+template <int ABL = 0>
+__global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_rawk_kernel(const SlotKParams p, int c_vec) {
+  typedef SlotK T;
+  constexpr int D = RawK::D, AHEAD = RawK::AHEAD;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char slotk_smem[];
+  const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int tm, tn;
+  {
+    const int total = p.tiles_m * p.tiles_n, per = total >> 3;
+    int id = blockIdx.x;
+    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
+    const int group = T::GROUP_M * p.tiles_n;
+    const int gi = id / group, first = gi * T::GROUP_M;
+    const int rows = (p.tiles_m - first) < T::GROUP_M ? (p.tiles_m - first) : T::GROUP_M;
+    const int in = id - gi * group;
+    tm = first + in % rows;
+    tn = in / rows;
+  }
+  const int m0 = tm * T::BM, n0 = tn * T::BN;
+  const int ksteps = p.K >> 4;
+  const int n_own = (ksteps - wave + T::NW - 1) / T::NW;   // 0 for the last waves of a very short K: they add zeros
+  const int ldb_bytes = (int)p.ldb * 4;
+
+  // ---- B: rows 8 g .. 8 g + 7 of a stage; beyond the last stage the loads point past the end of the
+  // buffer and return zeros (see the kernel above) ----
+  const int64_t b_bytes64 = ((int64_t)(p.K - 1) * p.ldb + p.N) * 4;
+  const int b_bytes = (int)(b_bytes64 > 0x7FFFFFFF ? 0x7FFFFFFF : b_bytes64);
+  const i32x4 rb = make_rsrc(p.b_slots, b_bytes);
+  const int vbq = 8 * g * ldb_bytes + (n0 + 4 * l31) * 4;
+  const int vbs = 8 * g * ldb_bytes + (n0 + 128 + l31) * 4;
+  f32x4 Bq[D][8];   // [ring buffer][k]: columns 4 l31 .. 4 l31 + 3
+  float Bs[D][8];   // column 128 + l31
+  auto b_base = [&](int i) { return i < n_own ? (wave + T::NW * i) * (T::BK * ldb_bytes) : b_bytes; };
+  auto issue_bq = [&](int i, int buf, int e) { Bq[buf][e] = llvm_raw_buffer_load_v4f32(rb, vbq, b_base(i) + e * ldb_bytes, 0); };
+  auto issue_bs = [&](int i, int buf, int e) { Bs[buf][e] = llvm_raw_buffer_load_f32(rb, vbs, b_base(i) + e * ldb_bytes, 0); };
+  u32x4 H[2], L[2];   // the split operand of the current / next block
+  auto split_b = [&](int buf, int ni, int dst) {
+    float r[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = ni < 4 ? Bq[buf][e][ni] : Bs[buf][e];
+    u32x4 t[2];
+    split8<CASCMM_FMT_BF16, 2>(r, t);
+    H[dst] = t[0];
+    L[dst] = t[1];
+  };
+
+  // ---- A: as in cascmm_slotk_kernel<1> ----
+  const int64_t a_bytes = ((int64_t)(p.M - 1) * p.lda + p.K) * 4;
+  const __amdgpu_buffer_rsrc_t rar =
+      __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)(a_bytes > 0x7FFFFFFF ? 0x7FFFFFFF : a_bytes), 0x00020000);
+  unsigned char* ring = slotk_smem + wave * T::RING;
+  const int dma_voff = (int)(((int64_t)(m0 + (lane >> 2)) * p.lda + (((lane & 3) - (lane >> 4)) & 3) * 4) * 4);
+  const int dma_rows16 = (int)p.lda * 64;
+  auto dma_a = [&](int i, int j) {
+    const int step = wave + T::NW * (i < n_own ? i : (n_own > 0 ? n_own - 1 : 0));
+    wavek_load_lds(rar, ring + (i & (T::RA - 1)) * T::A_STAGE + j * 1024, dma_voff, step * (T::BK * 4) + j * dma_rows16);
+  };
+  const int a_frag0 = l31 * 64 + ((2 * g + (l31 >> 2)) & 3) * 16;
+  const int a_frag1 = l31 * 64 + ((2 * g + 1 + (l31 >> 2)) & 3) * 16;
+  f32x4 X[T::MT][2];
+  u32x4 Ar[2][T::MT][2];   // [stage parity][row block][term]
+  auto read_a = [&](int i, int mi) {
+    const unsigned char* st = ring + (i & (T::RA - 1)) * T::A_STAGE + mi * 2048;
+    X[mi][0] = *(const f32x4*)(st + a_frag0);
+    X[mi][1] = *(const f32x4*)(st + a_frag1);
+  };
+  auto split_a = [&](int buf, int mi) {
+    float r[8] = {X[mi][0][0], X[mi][0][1], X[mi][0][2], X[mi][0][3], X[mi][1][0], X[mi][1][1], X[mi][1][2], X[mi][1][3]};
+    u32x4 t[2];
+    split8<CASCMM_FMT_BF16, 2>(r, t);
+    Ar[buf][mi][0] = t[0];
+    Ar[buf][mi][1] = t[1];
+  };
+
+  // ---- prologue: raw A of stages 0 .. AHEAD - 1 and stage 0 of B first (36 loads), then the rest of B
+  // (40 loads: the wait below names exactly those) ----
+  f32x16 acc[T::MT][T::NTL];
+#pragma unroll
+  for (int d = 0; d < AHEAD; ++d)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma_a(d, j);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) issue_bq(0, 0, e);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) issue_bs(0, 0, e);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int d = 1; d < D; ++d)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) issue_bq(d, d, e);
+#pragma unroll
+  for (int d = 1; d < D - 1; ++d)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) issue_bs(d, d, e);
+#pragma unroll
+  for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < T::NTL; ++ni)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[mi][ni][e] = 0.f;
+  {
+    constexpr int LATER = 8 * (D - 1) + 8 * (D - 2);   // 40
+    static_assert(LATER <= 63, "the wait counter has six bits");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (LATER & 0xF) | ((LATER >> 4) << 14));
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi);
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi) split_a(0, mi);
+    split_b(0, 0, 0);
+  }
+
+  auto mfma = [&](u32x4 a, u32x4 b, f32x16 c) -> f32x16 {
+    if (ABL == 1) { asm volatile("" ::"v"(a), "v"(b)); return c; }
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  };
+  // Stage i, ring buffer u = i % D.  During column block ni: the MFMAs of the block; the split of the next
+  // block (ni = 4: block 0 of the next stage); loads into registers that are free by then -- ni = 0 .. 2:
+  // the single column of the PREVIOUS buffer's next stage (its last reader was the split during the
+  // previous stage's block 3), ni = 3, 4: the four adjacent columns of this buffer's next stage (last read
+  // by the split during block 2); ni = 0 .. 3: one load of raw A into the LDS ring; ni = 0, 1: the A
+  // fragments of the next stage, split during ni = 1, 2.  Those fragments were requested during stage
+  // i + 1 - AHEAD; a stage issues 20 loads and nothing moves across a stage's end, so once at most
+  // 20 (AHEAD - 2) = 60 loads are outstanding at the top of stage i they have landed.
+  for (int i0 = 0; i0 < n_own; i0 += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int i = i0 + u;
+      {
+        constexpr int YOUNGER = 20 * (AHEAD - 2);
+        static_assert(YOUNGER <= 63, "the wait counter has six bits");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14));
+      }
+      constexpr int P = D - 1;
+      const int ab = u & 1;
+#pragma unroll
+      for (int ni = 0; ni < T::NTL; ++ni) {
+        const int cur = (u * T::NTL + ni) & 1;
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][1], H[cur], acc[mi][ni]);
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], L[cur], acc[mi][ni]);
+#pragma unroll
+        for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], H[cur], acc[mi][ni]);
+        if (ni < T::NTL - 1) split_b(u, ni + 1, cur ^ 1);
+        else split_b((u + 1) % D, 0, cur ^ 1);
+        if (ABL != 2) {
+          if (ni < 3) {
+#pragma unroll
+            for (int e = 3 * ni; e < (ni == 2 ? 8 : 3 * ni + 3); ++e) issue_bs(i + P, (u + P) % D, e);
+          } else {
+#pragma unroll
+            for (int e = 4 * (ni - 3); e < 4 * (ni - 3) + 4; ++e) issue_bq(i + D, u, e);
+          }
+          if (ni < 4) dma_a(i + AHEAD, ni);
+        }
+        if (ni < T::MT) read_a(i + 1, ni);
+        if (ni >= 1 && ni <= T::MT) split_a(ab ^ 1, ni - 1);
+        // loads of this block: 4, 4, 3, 5, 4 -- one behind each of the first MFMAs
+        constexpr int kLoads[5] = {4, 4, 3, 5, 4};
+#pragma unroll
+        for (int x = 0; x < 6; ++x) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (x < kLoads[ni]) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // ---- the four partial tiles meet in LDS: wave W owns register quad W (rows 8 W + 4 g + e) of all ten
+  // blocks; a non-owner w puts its quad q of block b at [q][(w - q - 1) mod 4][b], 16 bytes per lane ----
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  __syncthreads();
+  auto reduce_and_store = [&](auto owner_tag) {
+    constexpr int W = decltype(owner_tag)::value;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (q == W) continue;
+      const int slot = (W - q - 1) & 3;
+#pragma unroll
+      for (int b = 0; b < T::BLOCKS; ++b) {
+        const f32x16& v = acc[b / T::NTL][b % T::NTL];
+        *(f32x4*)(slotk_smem + ((q * 3 + slot) * T::BLOCKS + b) * 1024 + lane * 16) = (f32x4){v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+      }
+    }
+    __syncthreads();
+    f32x4 sum[T::MT][T::NTL];
+#pragma unroll
+    for (int b = 0; b < T::BLOCKS; ++b) {
+      const f32x16& v = acc[b / T::NTL][b % T::NTL];
+      f32x4 s4;
+      // partial sums in wave order 0, 1, 2, 3: the own one at its place
+#pragma unroll
+      for (int w = 0; w < T::NW; ++w) {
+        const f32x4 part = w == W ? (f32x4){v[4 * W], v[4 * W + 1], v[4 * W + 2], v[4 * W + 3]}
+                                  : *(const f32x4*)(slotk_smem + ((W * 3 + ((w - W - 1) & 3)) * T::BLOCKS + b) * 1024 + lane * 16);
+        if (w == 0) s4 = part;
+        else s4 += part;
+      }
+      sum[b / T::NTL][b % T::NTL] = s4;
+    }
+    const int ldc_bytes = (int)p.ldc * 4;
+    const int64_t c_bytes64 = ((int64_t)(p.M - 1 - m0) * p.ldc + (p.N - n0)) * 4;   // rows past M fall beyond the end: dropped
+    const int c_bytes = (int)(c_bytes64 > 0x7FFFFFFF ? 0x7FFFFFFF : c_bytes64);
+    const i32x4 rc = make_rsrc(p.C + (int64_t)m0 * p.ldc + n0, c_bytes);
+    // columns past N (a ragged last tile) are sent beyond the end as well
+    const int colq = 4 * l31, cols = 128 + l31;
+    const bool inq = n0 + colq < p.N, ins = n0 + cols < p.N;   // (N % 4 == 0: four adjacent columns are inside together)
+    f32x4 bq = {0.f, 0.f, 0.f, 0.f};
+    float bs = 0.f;
+    if (p.bias && inq) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bq[j] = p.bias[n0 + colq + j];
+    }
+    if (p.bias && ins) bs = p.bias[n0 + cols];
+    const int voq = inq ? (g * 4 * ldc_bytes) + colq * 4 : c_bytes;
+    const int vos = ins ? (g * 4 * ldc_bytes) + cols * 4 : c_bytes;
+#pragma unroll
+    for (int mi = 0; mi < T::MT; ++mi)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int soff = (mi * 32 + W * 8 + e) * ldc_bytes;
+        const f32x4 v4 = {sum[mi][0][e] + bq[0], sum[mi][1][e] + bq[1], sum[mi][2][e] + bq[2], sum[mi][3][e] + bq[3]};
+        if (c_vec) {
+          llvm_raw_buffer_store_v4f32(v4, rc, voq, soff, 0);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) llvm_raw_buffer_store_f32(v4[j], rc, inq ? voq + 4 * j : c_bytes, soff, 0);
+        }
+        llvm_raw_buffer_store_f32(sum[mi][4][e] + bs, rc, vos, soff, 0);
+      }
   };
   if (wave == 0) reduce_and_store(std::integral_constant<int, 0>{});
   else if (wave == 1) reduce_and_store(std::integral_constant<int, 1>{});

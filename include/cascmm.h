@@ -219,7 +219,7 @@ int cascmm_gemm_glu(const void* A, const void* B, void* C, const void* bias,
  * cascmm_prepare_left writes the left slots of any fp32 A [M, K] (lda % 4 == 0, 16-byte aligned) in a
  * pass of its own -- what the gated store does on the fly; cascmm_left_slots_bytes gives the size
  * (4 M K).  cascmm_gemm_chained computes C = A . B (+ bias) from the two slot buffers in one launch for
- * any M and N, K % 16 == 0, K >= 64, slot buffers below 2 GiB (cascmm_chained_supported says
+ * any M and N, K % 16 == 0, slot buffers below 2 GiB (cascmm_chained_supported says
  * whether a shape is taken); K is split over the waves of a workgroup, so no workspace is needed.
  * Same terms, same three products as cascmm_gemm with two bf16 terms; the order of summation over k
  * differs (four interleaved partial sums), as it does between any two kernel tiles.
