@@ -157,7 +157,8 @@ static const TunedCost kTuned[] = {
     // K split over the waves: a round of 256 tiles costs 0.012 us per k + 8 us, and rounds do not overlap
     // (2048 x {1280, 5120} x 1280: 23.3 / 69.3 us; 8192 x 640 x 640, two rounds: 31.9 us; 1024 x 1280 x 1280: 19.1 us)
     {"k64x160x16_wk4_bf16x2_tri_bpre", 0.767, 8.0, 0.65, 0.95},
-    {"k64x160x16_wk4_bf16x2_tri", 0.80, 8.5, 0.65, 0.95},
+    // ... both operands raw (2048 x {1280, 5120} x 1280: 24.0 / 77.2 us; 8192 x 2560 x 640, two rounds: 79.3 us)
+    {"k64x160x16_wk4_bf16x2_tri", 0.887, 6.3, 0.65, 0.95},
 };
 
 constexpr int kMaxTileSplits = 4;
@@ -245,7 +246,9 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     // tiles that hang over the edge of C take the bounds-checked epilogue and load clamped
     // columns: measured about a quarter slower (32768 x 640 x 320 on the 128-wide tile)
     const double edge = (q.N % v.BN != 0 || q.M % v.BM != 0) ? 1.25 : 1.0;
-    double best = edge * rounds * ((double)q.K / 64.0 * t.step64_us + t.fixed_us);
+    // (the kernels that split K over their waves run whole trips of four stages per wave: K in steps of 256)
+    const double k_run = v.kind == KIND_SLOTK ? (double)((q.K + 255) / 256 * 256) : (double)q.K;
+    double best = edge * rounds * (k_run / 64.0 * t.step64_us + t.fixed_us);
     if (v.kind == KIND_TILE && count == 1 && q.dtype == CASCMM_DT_F32 && q.N % 4 == 0 && full == 0 && !q.glu) {
       const int64_t ksteps = (q.K + v.BK - 1) / v.BK;
       for (int sp = 2; sp <= kMaxTileSplits; ++sp) {

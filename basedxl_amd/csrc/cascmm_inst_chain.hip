@@ -30,6 +30,11 @@ int launch_prepare_left(const float* A, int M, int K, int64_t lda, void* out, hi
                                                                                                                  : CASCMM_ERR_LAUNCH;
 }
 
+static int slotk_group_m() {
+  if (const char* e = getenv("SLOTK_GROUP_M")) return atoi(e) > 0 ? atoi(e) : SlotK::GROUP_M;
+  return SlotK::GROUP_M;
+}
+
 const void* slotk_kernel_handle(int araw) { return araw ? (const void*)cascmm_slotk_kernel<1> : (const void*)cascmm_slotk_kernel<0>; }
 
 template <int ARAW>
@@ -46,6 +51,7 @@ static int launch_slotk_t(const SlotKParams& q, hipStream_t stream) {
   SlotKParams p = q;
   p.tiles_m = (q.M + T::BM - 1) / T::BM;
   p.tiles_n = (q.N + T::BN - 1) / T::BN;
+  p.group_m = slotk_group_m();
   const int64_t grid = (int64_t)p.tiles_m * p.tiles_n;
   if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
   return launch_kernel(kfn, dim3((unsigned)grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) == hipSuccess ? CASCMM_OK
@@ -92,6 +98,7 @@ static int launch_rawk_variant(const GroupParams& p, hipStream_t stream) {
   q.M = p.M; q.N = p.N; q.K = p.K; q.lda = p.lda; q.ldb = p.ldb; q.ldc = p.ldc;
   q.tiles_m = (p.M + T::BM - 1) / T::BM;
   q.tiles_n = (p.N + T::BN - 1) / T::BN;
+  q.group_m = slotk_group_m();
   const int64_t grid = (int64_t)q.tiles_m * q.tiles_n;
   if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
   const int c_vec = p.ldc % 4 == 0 && (uintptr_t)p.C[0] % 16 == 0;

@@ -49,6 +49,7 @@ struct SlotKParams {
   int M, N, K;
   int64_t lda, ldb, ldc;   // ldb: cascmm_rawk_kernel only (raw B)
   int tiles_m, tiles_n;
+  int group_m;             // tile rows an XCD's range of tiles walks down before moving one tile to the right
 };
 
 // Host-checked: K % 16 == 0, K >= 16, the slot buffers 16-byte aligned and below 2 GiB,
@@ -68,9 +69,9 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     const int total = p.tiles_m * p.tiles_n, per = total >> 3;
     int id = blockIdx.x;
     if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    const int group = T::GROUP_M * p.tiles_n;
-    const int gi = id / group, first = gi * T::GROUP_M;
-    const int rows = (p.tiles_m - first) < T::GROUP_M ? (p.tiles_m - first) : T::GROUP_M;
+    const int group = p.group_m * p.tiles_n;
+    const int gi = id / group, first = gi * p.group_m;
+    const int rows = (p.tiles_m - first) < p.group_m ? (p.tiles_m - first) : p.group_m;
     const int in = id - gi * group;
     tm = first + in % rows;
     tn = in / rows;
@@ -338,9 +339,9 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     const int total = p.tiles_m * p.tiles_n, per = total >> 3;
     int id = blockIdx.x;
     if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    const int group = T::GROUP_M * p.tiles_n;
-    const int gi = id / group, first = gi * T::GROUP_M;
-    const int rows = (p.tiles_m - first) < T::GROUP_M ? (p.tiles_m - first) : T::GROUP_M;
+    const int group = p.group_m * p.tiles_n;
+    const int gi = id / group, first = gi * p.group_m;
+    const int rows = (p.tiles_m - first) < p.group_m ? (p.tiles_m - first) : p.group_m;
     const int in = id - gi * group;
     tm = first + in % rows;
     tn = in / rows;

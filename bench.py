@@ -44,12 +44,40 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 SEED = 1
 METRIC = {"ffn": "fp32-equiv TFLOP/s + % of MFMA roofline at SDXL FFN shape; rel-Frobenius err",
           "attn": "fp32-equiv TFLOP/s + % of MFMA roofline at SDXL self-attention projection shape; rel-Frobenius err"}
-# HBM-side traffic of one launch of the dominant kernel, measured with rocprofv3 counters (the
-# summaries under profiles/ give the commands and the calibration); keyed by (workload, launch label).
-TRAFFIC_BYTES_PER_LAUNCH = {
-    ("ffn", "ff.net.0.proj (W1)"): 2 * 72854.0 * 1024 + 83968.0 * 1024,
-    ("attn", "to_q/to_k/to_v grouped"): 2 * 21930.0 * 1024 + 30720.0 * 1024,
-}
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "counter_traffic.txt")
+
+
+def counter_traffic():
+    """HBM-side traffic per launch as rocprofv3 counter runs measured it: the rows of
+    profiles/counter_traffic.txt, keyed by (workload, launch label).  Every row names the kernel variant
+    it was measured on, the commit of that build and the summary under profiles/ it comes from; the bench
+    reports a figure only for the kernel it actually ran (another kernel: null)."""
+    rows = {}
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for line in f:
+                if line.startswith("#") or "|" not in line:
+                    continue
+                c = [x.strip() for x in line.split("|")]
+                if len(c) != 9:
+                    continue
+                wl, launch, kernel, fetch_kib, f_fac, write_kib, w_fac, commit, profile = c
+                rows[(wl, launch)] = {"kernel": kernel, "commit": commit, "profile": profile,
+                                      "bytes": (float(fetch_kib) * float(f_fac) + float(write_kib) * float(w_fac)) * 1024.0}
+    except OSError:
+        pass
+    return rows
+
+
+def traffic_for(workload_name, launch, kernel):
+    """(bytes or None, where it comes from) for one launch of `kernel`"""
+    row = counter_traffic().get((workload_name, launch))
+    if row is None:
+        return None, "no counter run recorded for this launch in profiles/counter_traffic.txt"
+    if row["kernel"] != kernel:
+        return None, f"the recorded counter run ({row['profile']}) is of kernel {row['kernel']}, not of the one that ran"
+    return row["bytes"], (f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same counters read for a 256 MiB "
+                          f"copy; build {row['commit']}; {row['profile']}")
 
 
 class Launch:
@@ -198,9 +226,6 @@ def measured_peaks(dev):
                    "events around 5 launches after 0.2 s of the same launches"}
 
 
-KV_TRAFFIC_BYTES = {1280: 21034047.0, 640: 18076444.0}   # HBM-side bytes per launch from rocprofv3 counters (see profiles/), when measured
-
-
 def bench_kv(dev, check=True):
     """cfg4: the two cross-attention K/V projections of the text tokens; bandwidth-style figures
     over the algorithmic bytes 4 (MK + KN + MN)."""
@@ -300,6 +325,117 @@ def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False),
             "configs": rows}
 
 
+def bench_attn(dev, check=True):
+    """cfg2: the four self-attention projections of the 64x64 stage on one GPU's patch share, as the step of
+    `--workload attn` runs them (to_q / to_k / to_v of the same tokens in one grouped launch, to_out on a
+    second activation tensor), each launch timed on its own and the two together."""
+    import torch
+    from basedxl_amd import cascaded_lowp_matmul, cascaded_lowp_matmul_grouped, _lib
+    from oracle import cascade as oc
+
+    l = _lib.lib()
+    g = torch.Generator().manual_seed(SEED + 2)
+    x_cpu, x2_cpu = torch.randn(4096, 640, generator=g), torch.randn(4096, 640, generator=g)
+    w_cpu = [torch.randn(640, 640, generator=g) * 0.02 for _ in range(4)]
+    x, x2, w = x_cpu.to(dev), x2_cpu.to(dev), [t.to(dev) for t in w_cpu]
+    outs = [torch.empty(4096, 640, device=dev) for _ in range(4)]
+    qkv = lambda: cascaded_lowp_matmul_grouped([x, x, x], w[:3], outs=outs[:3])      # noqa: E731
+    o = lambda: cascaded_lowp_matmul(x2, w[3], out=outs[3])                          # noqa: E731
+
+    def step():
+        qkv()
+        o()
+
+    us_qkv, us_o, us_step = _graph_time_us(qkv, reps=10), _graph_time_us(o, reps=10), _graph_time_us(step, reps=10)
+    flop = 2.0 * 4096 * 640 * 640
+    names = _lib.variant_names()
+    k_qkv = names[l.cascmm_select_variant_grouped(3, 4096, 640, 640, 640, 640, 640, 0, 0, 2, 0) & 0xFFFF]
+    k_o = names[l.cascmm_select_variant(4096, 640, 640, 640, 640, 640, 0, 0, 2, 0) & 0xFFFF]
+    rec = {"workload": "cfg2: SDXL 64x64-stage self-attention projections on one GPU's patch share: X fp32 [4096,640] ~N(0,1) x W fp32 "
+                       "[640,640] ~N(0,0.02), to_q/to_k/to_v as one grouped launch + to_out; 2-term bf16 cascade (3 products), both "
+                       "operands split inside the kernels",
+           "us_per_step": round(us_step, 2), "fp32_equiv_tflops": round(4 * flop / us_step * 1e-6, 1),
+           "launches": [
+               {"launch": "to_q/to_k/to_v grouped", "kernel": k_qkv, "launch_us": round(us_qkv, 2),
+                "mfma_tflops": round(9 * flop / us_qkv * 1e-6, 1), "frac_of_mfma_peak": round(9 * flop / us_qkv * 1e-6 / PEAK_BF16_TFLOPS, 4),
+                "traffic": traffic_for("attn", "to_q/to_k/to_v grouped", k_qkv)[0]},
+               {"launch": "to_out", "kernel": k_o, "launch_us": round(us_o, 2), "mfma_tflops": round(3 * flop / us_o * 1e-6, 1),
+                "frac_of_mfma_peak": round(3 * flop / us_o * 1e-6 / PEAK_BF16_TFLOPS, 4)}]}
+    if check:
+        exp = oc.fp64_matmul(x2_cpu, w_cpu[3])
+        ek, eo = oc.error_metrics(outs[3].cpu(), exp), oc.error_metrics(oc.cascade_matmul_ref(x2_cpu, w_cpu[3]), exp)
+        if not (ek["rel_fro"] <= 1.25 * eo["rel_fro"] and ek["max_abs"] <= 1.25 * eo["max_abs"]):
+            sys.exit(f"bench.py: attn kernel error {ek} exceeds 1.25x the oracle cascade's {eo}")
+        rec["kernel_rel_fro"], rec["oracle_rel_fro"] = ek["rel_fro"], eo["rel_fro"]
+    return rec
+
+
+def bench_ffn_modes(dev, check=True):
+    """cfg3 as the model runs it -- the gate between the two GEMMs is real: h = X W1 + b1, G = value x
+    gelu(gate), Y = G W2 + b2 -- in the modes the library offers for it.  The headline step multiplies a
+    synthetic G and applies no gate; these are labelled modes beside it, with the same 80.5 GFLOP
+    (fp32-equivalent) of GEMM work per step:
+      * layer by layer: the gated store writes G as fp32, the second GEMM reads and splits it;
+      * chained: the gated store writes G as the second GEMM's operand slots, the second GEMM multiplies slots
+        by slots (its weight split once: the chained GEMM has no other form); W1 split in every call, or
+        kept split as well."""
+    import torch
+    from basedxl_amd import (ChainedWeight, LeftSlots, PreparedWeight, cascaded_lowp_matmul, cascaded_lowp_matmul_chained,
+                             cascaded_lowp_matmul_glu_chained)
+    from basedxl_amd.cascaded_lowp_matmul import cascaded_lowp_matmul_glu
+    from oracle import cascade as oc
+
+    M, K, inner, N2 = 2048, 1280, 5120, 1280
+    g = torch.Generator().manual_seed(SEED + 3)
+    x_cpu = torch.randn(M, K, generator=g)
+    w1_cpu, b1_cpu = torch.randn(K, 2 * inner, generator=g) * 0.02, torch.randn(2 * inner, generator=g) * 0.1
+    w2_cpu, b2_cpu = torch.randn(inner, N2, generator=g) * 0.02, torch.randn(N2, generator=g) * 0.1
+    x, w1, b1, w2, b2 = (t.to(dev) for t in (x_cpu, w1_cpu, b1_cpu, w2_cpu, b2_cpu))
+    pw1, pw2, cw2 = PreparedWeight(w1, glu=True), PreparedWeight(w2), ChainedWeight(w2)
+    gbuf, y = torch.empty(M, inner, device=dev), torch.empty(M, N2, device=dev)
+    slots = LeftSlots.empty((M,), inner, dev)
+    modes = [
+        ("geglu, layer by layer, weights split in every call",
+         lambda: cascaded_lowp_matmul_glu(x, w1, bias=b1, out=gbuf), lambda: cascaded_lowp_matmul(gbuf, w2, bias=b2, out=y)),
+        ("geglu, layer by layer, weights kept split",
+         lambda: cascaded_lowp_matmul(x, pw1, bias=b1, out=gbuf), lambda: cascaded_lowp_matmul(gbuf, pw2, bias=b2, out=y)),
+        ("geglu, chained (slots), W1 split in every call, W2 kept split",
+         lambda: cascaded_lowp_matmul_glu_chained(x, w1, bias=b1, out=slots), lambda: cascaded_lowp_matmul_chained(slots, cw2, bias=b2, out=y)),
+        ("geglu, chained (slots), weights kept split",
+         lambda: cascaded_lowp_matmul_glu_chained(x, pw1, bias=b1, out=slots), lambda: cascaded_lowp_matmul_chained(slots, cw2, bias=b2, out=y)),
+    ]
+    flops = 2.0 * M * K * 2 * inner + 2.0 * M * inner * N2
+    exp = ref_err = None
+    if check:
+        h = x_cpu.double() @ w1_cpu.double() + b1_cpu.double()
+        gate = h[:, inner:]
+        exp = (h[:, :inner] * (0.5 * gate * (1.0 + torch.erf(gate / 2.0 ** 0.5)))) @ w2_cpu.double() + b2_cpu.double()
+        ref_err = oc.error_metrics(oc.cascade_matmul_ref(oc.gated_projection_ref(x_cpu, w1_cpu, b1_cpu), w2_cpu) + b2_cpu, exp)
+    rows = []
+    for label, first, second in modes:
+        def step():
+            first()
+            second()
+        step()
+        torch.cuda.synchronize()
+        row = {"mode": label}
+        if check:
+            ek = oc.error_metrics(y.cpu(), exp)
+            if not (ek["rel_fro"] <= 1.25 * ref_err["rel_fro"] and ek["max_abs"] <= 1.25 * ref_err["max_abs"]):
+                sys.exit(f"bench.py: ffn mode '{label}': error {ek} exceeds 1.25x the oracle composition's {ref_err}")
+            row.update(kernel_rel_fro=ek["rel_fro"], oracle_rel_fro=ref_err["rel_fro"], kernel_max_abs=ek["max_abs"],
+                       oracle_max_abs=ref_err["max_abs"])
+        us1, us2, us = _graph_time_us(first, reps=10), _graph_time_us(second, reps=10), _graph_time_us(step, reps=10)
+        row.update(us_per_step=round(us, 2), first_gemm_us=round(us1, 2), second_gemm_us=round(us2, 2),
+                   fp32_equiv_tflops=round(flops / us * 1e-6, 1),
+                   second_gemm_mfma_tflops=round(3 * 2.0 * M * inner * N2 / us2 * 1e-6, 1))
+        rows.append(row)
+    return {"workload": "cfg3 with the real gate: X fp32 [2048,1280] ~N(0,1) x W1 [1280,10240] ~N(0,0.02) + b1, value x gelu(gate), "
+                        "x W2 [5120,1280] ~N(0,0.02) + b2; 2-term bf16 cascades; the gate is applied in the first GEMM's store in every "
+                        "mode; checked against the oracle's gated projection followed by its cascade (1.25x on both metrics vs fp64)",
+            "gflop_fp32_equiv_per_step": round(flops * 1e-9, 2), "modes": rows}
+
+
 def bench_sweep(dev, sizes=(256, 512, 1024, 2048, 4096, 8192)):
     """The reference's self-benchmark (basedxl/triton/cascaded_lowp_matmul.py:204-242): square
     problems M = N = K against the vendor GEMM.  Here: the two-term bf16 cascade on fp32 tensors
@@ -364,7 +500,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=["ffn", "attn", "kv", "unet", "sweep"], default="ffn",
+    ap.add_argument("--workload", choices=["ffn", "attn", "kv", "unet", "sweep", "ffn-modes"], default="ffn",
                     help="ffn: the two GEMMs of the 32x32-stage GEGLU feed-forward block (the shape the metric is quoted on); "
                          "attn: the four 64x64-stage self-attention projections of one GPU's patch share; kv: the skinny "
                          "cross-attention K/V projections (GB/s); unet: the Linear path of one whole UNet step; sweep: square "
@@ -400,7 +536,7 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = torch.device("cuda:0")
-    if args.workload in ("kv", "unet", "sweep"):
+    if args.workload in ("kv", "unet", "sweep", "ffn-modes"):
         base = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
                 "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
         if args.workload == "kv":
@@ -410,9 +546,18 @@ def main():
                                   value=kv["hbm_gbs"], unit="GB/s", ms_per_step=round(kv["us_both"] * 1e-3, 5),
                                   config={"workload": kv["workload"], "launch": "hip graph replay (20 launches per graph)"},
                                   roofline={"bound": "hbm", "kernel": worst["kernel"], "achieved": worst["hbm_gbs"], "peak": 8000.0,
-                                            "unit": "GB/s", "frac": worst["frac_of_8TBs"], "traffic": KV_TRAFFIC_BYTES.get(worst["N"]),
+                                            "unit": "GB/s", "frac": worst["frac_of_8TBs"],
+                                            "traffic": traffic_for("kv", f"N={worst['N']}", worst["kernel"])[0],
+                                            "traffic_is": traffic_for("kv", f"N={worst['N']}", worst["kernel"])[1],
                                             "launch_us": worst["launch_us"], "algorithmic_bytes_per_launch": worst["algorithmic_bytes"]},
                                   gemms=kv["gemms"])))
+        elif args.workload == "ffn-modes":
+            fm = bench_ffn_modes(dev)
+            head = fm["modes"][-1]
+            print(json.dumps(dict(base, metric="fp32-equiv TFLOP/s of the SDXL FFN block with its gate, chained GEMMs",
+                                  value=head["fp32_equiv_tflops"], unit="TFLOP/s", ms_per_step=round(head["us_per_step"] * 1e-3, 5),
+                                  config={"workload": fm["workload"], "launch": "hip graph replay (10 steps per graph); mode: " + head["mode"]},
+                                  modes=fm["modes"])))
         elif args.workload == "sweep":
             sw = bench_sweep(dev)
             head = sw["sizes"][-1]
@@ -615,9 +760,8 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(dom["mfma_tflops"] / PEAK_BF16_TFLOPS, 4),
-            "traffic": TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dom["launch"])),
-            "traffic_is": "HBM-side bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE (x2.0) + WRITE_SIZE "
-                          "(x1.0), factors from a 256 MiB copy in the same runs; see profiles/",
+            "traffic": traffic_for(args.workload, dom["launch"], dom["kernel"])[0],
+            "traffic_is": traffic_for(args.workload, dom["launch"], dom["kernel"])[1],
             "launch_us": dom["launch_us"],
             "launch_us_is": "HIP events on the launch stream around graph replays of this launch alone (10 launches per "
                             "graph) / launches",
@@ -668,7 +812,9 @@ def main():
     if args.workload == "ffn" and not args.no_graph and not args.no_other_workloads:
         del sets, a_dev, w_dev
         torch.cuda.empty_cache()
-        result["other_workloads"] = {"kv": bench_kv(dev), "unet": bench_unet(dev), "eager_launch": bench_eager_launch(dev)}
+        result["ffn_modes"] = bench_ffn_modes(dev)
+        result["other_workloads"] = {"attn": bench_attn(dev), "kv": bench_kv(dev), "unet": bench_unet(dev),
+                                     "eager_launch": bench_eager_launch(dev)}
     if args.workload == "ffn" and not args.no_graph:
         # the published peak beside what the board holds: `peak` and `frac` stay the published ones
         torch.cuda.empty_cache()

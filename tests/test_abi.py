@@ -121,6 +121,8 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
     assert grouped == "t256x128x32_w4x1x1_d2_bf16x2_tri"                           # cfg2, to_q / to_k / to_v
     assert pick(4096, 640, 640) == "t64x160x64_w2x1x2_d2_p8_bf16x2_tri"            # cfg2, to_out
     assert pick(8192, 640, 5120) == "t256x320x32_w512_bf16x2_tri"                  # cfg5: the 640-stage feed-forward, whole large tiles
+    # one 64 x 160 tile per CU and K split over the waves: cfg3's second GEMM and the 1280-channel projections
+    assert pick(2048, 5120, 1280) == "k64x160x16_wk4_bf16x2_tri" and pick(2048, 1280, 1280) == "k64x160x16_wk4_bf16x2_tri"
     # three fp8 terms, weights kept split: the tile of the fp8-rate kernel that a sweep over the UNet's
     # shapes measured faster (256 rows where the tiles fill the chip, 128 rows where they would not)
     pick8 = lambda M, K, N: names[l.cascmm_select_variant_prepared(1, M, N, K, K, N, 0, 2, 3, 0) & 0xFFFF]
@@ -131,6 +133,7 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
         assert pick8(M, K, N) == "t128x160x64_f8k64_fp8x3_tri_bpre", (M, K, N)
     pickp = lambda M, K, N: names[l.cascmm_select_variant_prepared(1, M, N, K, K, N, 0, 0, 2, 0) & 0xFFFF]
     assert pickp(2048, 1280, 10240) == "t256x320x32_w512_bf16x2_tri_bpre"
+    assert pickp(2048, 5120, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre" and pickp(2048, 1280, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre"
 
 
 def test_scale_search_argument_validation():
