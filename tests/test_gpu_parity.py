@@ -21,10 +21,24 @@ pytestmark = pytest.mark.gpu
 TOL = 1.25  # kernel error may be at most this multiple of the oracle cascade's error
 # v_mfma_f32_32x32x16_fp8_fp8 adds the 8 products of one lane in a window of about 15 bits below
 # the largest of them (measured: 448*448 + 2^2 returns 448*448, + 2^3 is kept; across the two
-# lane groups and into the accumulator it adds in full fp32).  That truncation, about 1.5e-5
-# relative, is below the error of the fp8 cascades that drop products, but it is what is left
-# when all nine products of three terms are kept: that one cascade gets a wider bound.
-TOL_FP8_FULL = 2.0
+# lane groups and into the accumulator it adds in full fp32), the fp8-rate instruction in windows of
+# 15 to 18 bits.  That truncation, about 1.5e-5 relative, widens the error DISTRIBUTION of the three-term
+# fp8 cascades by a constant factor -- relative Frobenius error x1.105 .. 1.109 of the oracle's for the
+# six kept products, x1.226 .. 1.237 when all nine are kept, on every shape measured -- which the 1.25x
+# bound on that metric covers.  The largest single error of a result is an extreme-value statistic of
+# that distribution and scatters around the same factor from case to case: where a case's measured
+# ratio exceeds 1.25 the bar below is that case's own number (measured value in the comment), not a
+# blanket factor.  Every fp8 x 3 `tri` case on a baseline shape meets 1.25 on both metrics.
+MAX_ABS_BAR_FP8X3_FULL = {      # all nine products kept (not a cascade the baseline names): measured, bar
+    "cfg1 1024^3": 1.25,               # 1.213
+    "cfg2 self-attn proj": 1.57,       # 1.538
+    "cfg3 geglu up (N/4)": 1.38,       # 1.350
+    "cfg3 ff down": 1.33,              # 1.302
+    "cfg4 cross-attn kv 1280": 1.25,   # 1.183
+    "cfg4 cross-attn kv 640": 1.35,    # 1.315
+    "ragged": 1.25,                    # 1.202
+}
+MAX_ABS_BAR_AUTOSCALE = {(512, 640, 320): 1.58}   # measured 1.553 (164 k results, no baseline shape); every other shape: 1.25
 
 
 def _say(*a):
@@ -194,12 +208,11 @@ def test_fp8_gemm_that_finds_its_activation_scale_equals_the_two_calls(gpu_devic
         exp64 = oc.fp64_matmul(a, b) + bias.cpu().double()
         ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "fp8", 3, "tri") + bias.cpu(), exp64)
         got = oc.error_metrics(outs[0].cpu(), exp64)
-        # The relative Frobenius error at the usual factor.  The largest single error of these small
-        # results is a tail statistic, and the fp8-rate MFMA widens the tail: it adds the 64 products
-        # of a lane pair inside a window of 15 to 18 bits below the largest of them, noise of about
-        # half the size of this cascade's own error; that one gets the wider factor here (the
-        # 1.25 x bound on both metrics is tested at the full sizes of the baseline configurations).
-        assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL_FP8_FULL * ref["max_abs"], (got, ref)
+        # 1.25x on both metrics (measured: relative Frobenius error x1.104 .. 1.109 on every shape; largest
+        # single error x1.184 at 2048 x 1280 x 1280, x1.116 at 8192 x 640 x 640, x1.059 at 154 x 2048 x 1280,
+        # x1.204 at 300 x 192 x 200); the one shape whose largest error lands further out has its own bar
+        _say(f"   autoscale ratios {shape} prepared={prepared}: rel_fro x{got['rel_fro'] / ref['rel_fro']:.3f} max_abs x{got['max_abs'] / ref['max_abs']:.3f}")
+        assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= MAX_ABS_BAR_AUTOSCALE.get(shape, TOL) * ref["max_abs"], (got, ref)
 
 
 # ---------------------------------------------------------------------------------------
@@ -443,9 +456,10 @@ def test_error_vs_fp64_within_bound_of_oracle(gpu_device, case, fmt, terms, prod
     got = oc.error_metrics(out.cpu(), exp)
     _say(f"   rel_fro kernel {got['rel_fro']:.3e} oracle {ref['rel_fro']:.3e}  max_abs kernel {got['max_abs']:.3e} "
          f"oracle {ref['max_abs']:.3e}")
-    tol = TOL_FP8_FULL if (fmt, terms, products) == ("fp8", 3, "full") else TOL
-    assert got["rel_fro"] <= tol * ref["rel_fro"], (got["rel_fro"], ref["rel_fro"])
-    assert got["max_abs"] <= tol * ref["max_abs"], (got["max_abs"], ref["max_abs"])
+    _say(f"   ratios: rel_fro x{got['rel_fro'] / ref['rel_fro']:.3f} max_abs x{got['max_abs'] / ref['max_abs']:.3f}")
+    tol_max = MAX_ABS_BAR_FP8X3_FULL[name] if (fmt, terms, products) == ("fp8", 3, "full") else TOL
+    assert got["rel_fro"] <= TOL * ref["rel_fro"], (got["rel_fro"], ref["rel_fro"])
+    assert got["max_abs"] <= tol_max * ref["max_abs"], (got["max_abs"], ref["max_abs"])
 
 
 @pytest.mark.parametrize("fmt,terms", [("bf16", 2), ("fp16", 3)])
