@@ -362,11 +362,21 @@ def routed_calls(model: nn.Module, *inputs) -> List[dict]:
     calls: List[dict] = []
     hooks = []
     for name, m in model.named_modules():
-        if not is_routed(m):
+        chained = type(m).__name__ == "BasedXLChainedFeedForward"
+        if not is_routed(m) and not chained:
             continue
 
         def hook(mod, args, name=name):
             x = args[0]
+            if type(mod).__name__ == "BasedXLChainedFeedForward":
+                # a feed-forward block that runs as a chain is ONE record of two GEMMs (M x in x 2 inner, then
+                # M x inner x out); where it falls back, its two inner modules are called and record themselves
+                if not mod._chain_ok(x):
+                    return
+                M, K, N = x.numel() // x.shape[-1], mod.in_features, 2 * mod.inner
+                calls.append({"name": name, "module": mod, "input_shape": tuple(x.shape), "M": M, "K": K, "N": N,
+                              "extra_flops": 2.0 * M * mod.inner * mod.out_features})
+                return
             if type(mod).__name__ == "BasedXLLowPConv1x1":
                 M, K, N = x.shape[0] * x.shape[2] * x.shape[3], mod.in_channels, mod.out_channels
             elif type(mod).__name__ == "BasedXLLowPGEGLU":

@@ -266,7 +266,7 @@ def bench_kv(dev, check=True):
 
 
 def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False), ("bf16", 2, True, False), ("fp8", 3, True, False),
-                              ("bf16", 2, False, True)),
+                              ("bf16", 2, False, True), ("bf16", 2, True, "chain")),
                latents=(("full latent", None), ("half-latent share", 64)), forward=True):
     """cfg5: the routed layers of one UNet step.  The module tree is built on the GPU with random
     weights and patched through the config switch; one forward pass records every routed call; those
@@ -281,7 +281,9 @@ def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False),
     rows = []
     for lowp, terms, prepared, geglu in cascades:
         model = SDXLUNetSkeleton(device=dev, seed=SEED)
-        unet = BasedXLUnet(model, BasedXLConfig(fp16_acc_matmul=True, lowp=lowp, terms=terms, prepared=prepared, fuse_geglu=geglu))
+        chain = geglu == "chain"     # the two GEMMs of every feed-forward block chained (gate in the first one's store, result as slots)
+        unet = BasedXLUnet(model, BasedXLConfig(fp16_acc_matmul=True, lowp=lowp, terms=terms, prepared=prepared,
+                                                fuse_geglu=bool(geglu) and not chain, chain_ffn=chain))
         for label, latent_rows in latents:
             inp = synthetic_inputs(model, latent=128, latent_rows=latent_rows, seed=SEED, device=dev)
             calls = routed_calls(unet, *inp)
@@ -305,9 +307,11 @@ def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False),
                         unet(*inp)
                     torch.cuda.synchronize()
                     fwd_ms = (time.perf_counter() - t0) * 1e3 / 2
-            flops = sum(2.0 * c["M"] * c["K"] * c["N"] for c in calls)
+            flops = sum(2.0 * c["M"] * c["K"] * c["N"] + c.get("extra_flops", 0.0) for c in calls)
             rows.append({"cascade": f"{lowp}x{terms} tri", "weights": "kept split (prepared once)" if prepared else "split in every call",
-                         "geglu": "value * gelu(gate) in the store of the projection's GEMM (this figure includes the gate)" if geglu
+                         "geglu": "feed-forward blocks chained: value * gelu(gate) in the store of the projection's GEMM, written as the operand "
+                                  "slots of the block's second GEMM (this figure includes the gate)" if chain
+                         else "value * gelu(gate) in the store of the projection's GEMM (this figure includes the gate)" if geglu
                          else "projection routed as a Linear; the gate stays with torch (two elementwise kernels, in no figure but "
                               "whole_forward_ms_eager)",
                          "latent": label, "routed_calls": len(calls), "distinct_shapes": len(shapes),
@@ -520,7 +524,7 @@ def main():
                          "every step, resident in the Infinity Cache; 8 = every step reads HBM-cold data)")
     ap.add_argument("--unet-select", default="",
                     help="unet only: run one configuration instead of all ten, as cascade:weights:latent, e.g. "
-                         "bf16x2:raw:full, fp8x3:prepared:half or bf16x2:raw+geglu:full (what a profiler run wants)")
+                         "bf16x2:raw:full, fp8x3:prepared:half, bf16x2:raw+geglu:full or bf16x2:prepared+chain:full (what a profiler run wants)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -568,8 +572,8 @@ def main():
             if args.unet_select:
                 casc, wts, lat = args.unet_select.split(":")
                 lowp, terms = casc.split("x")
-                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts == "prepared" else False if wts == "raw+geglu" else None,
-                                                wts == "raw+geglu"),),
+                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts in ("prepared", "prepared+chain") else False if wts == "raw+geglu" else None,
+                                                "chain" if wts == "prepared+chain" else wts == "raw+geglu"),),
                                 latents=(("full latent", None),) if lat == "full" else (("half-latent share", 64),), forward=False)
             else:
                 un = bench_unet(dev)
