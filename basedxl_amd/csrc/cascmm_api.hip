@@ -8,7 +8,6 @@
 #include <vector>
 
 #include "cascmm_variants.h"
-#include "cascmm_slotk_kernel.h"
 
 namespace cascmm {
 

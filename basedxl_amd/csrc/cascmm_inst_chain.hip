@@ -30,28 +30,18 @@ int launch_prepare_left(const float* A, int M, int K, int64_t lda, void* out, hi
                                                                                                                  : CASCMM_ERR_LAUNCH;
 }
 
-static int slotk_group_m() {
-  if (const char* e = getenv("SLOTK_GROUP_M")) return atoi(e) > 0 ? atoi(e) : SlotK::GROUP_M;
-  return SlotK::GROUP_M;
-}
-
 const void* slotk_kernel_handle(int araw) { return araw ? (const void*)cascmm_slotk_kernel<1> : (const void*)cascmm_slotk_kernel<0>; }
 
 template <int ARAW>
 static int launch_slotk_t(const SlotKParams& q, hipStream_t stream) {
   typedef SlotK T;
   auto kfn = cascmm_slotk_kernel<ARAW>;
-  if (const char* e = getenv("SLOTK_ABL")) {
-    if (e[0] == '1') kfn = cascmm_slotk_kernel<ARAW, 1>;
-    if (e[0] == '2') kfn = cascmm_slotk_kernel<ARAW, 2>;
-    (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
-  }
   static LdsFlags lds_set;
   if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
   SlotKParams p = q;
   p.tiles_m = (q.M + T::BM - 1) / T::BM;
   p.tiles_n = (q.N + T::BN - 1) / T::BN;
-  p.group_m = slotk_group_m();
+  p.group_m = SlotK::GROUP_M;
   const int64_t grid = (int64_t)p.tiles_m * p.tiles_n;
   if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
   return launch_kernel(kfn, dim3((unsigned)grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, p) == hipSuccess ? CASCMM_OK
@@ -79,17 +69,12 @@ static int launch_slotk_variant(const GroupParams& p, hipStream_t stream) {
 // both operands raw fp32
 static int launch_rawk_variant(const GroupParams& p, hipStream_t stream) {
   typedef SlotK T;
-  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_rawk_kernel<0>; return CASCMM_OK; }
+  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_rawk_kernel; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
   if (p.K % T::BK != 0 || p.K < T::BK || p.N % 4 != 0) return CASCMM_ERR_BAD_VARIANT;
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
-  auto kfn = cascmm_rawk_kernel<0>;
-  if (const char* e = getenv("SLOTK_ABL")) {
-    if (e[0] == '1') kfn = cascmm_rawk_kernel<1>;
-    if (e[0] == '2') kfn = cascmm_rawk_kernel<2>;
-    (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS_BYTES);
-  }
+  auto kfn = cascmm_rawk_kernel;
   static LdsFlags lds_set;
   if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
   SlotKParams q;
@@ -98,7 +83,7 @@ static int launch_rawk_variant(const GroupParams& p, hipStream_t stream) {
   q.M = p.M; q.N = p.N; q.K = p.K; q.lda = p.lda; q.ldb = p.ldb; q.ldc = p.ldc;
   q.tiles_m = (p.M + T::BM - 1) / T::BM;
   q.tiles_n = (p.N + T::BN - 1) / T::BN;
-  q.group_m = slotk_group_m();
+  q.group_m = SlotK::GROUP_M;
   const int64_t grid = (int64_t)q.tiles_m * q.tiles_n;
   if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
   const int c_vec = p.ldc % 4 == 0 && (uintptr_t)p.C[0] % 16 == 0;

@@ -31,31 +31,10 @@
 
 namespace cascmm {
 
-struct SlotK {
-  static constexpr int BM = 64, BN = 160, BK = 16, NW = 4, NT = 256, D = 4, GROUP_M = 8;
-  static constexpr int MT = 2, NTL = 5, BLOCKS = MT * NTL;
-  static constexpr int BLOCK_BYTES = 16 * 64 * 4;                  // one wave's 32 x 32 partial block
-  static constexpr int RED_BYTES = BLOCKS * 3 * BLOCK_BYTES;       // 120 KB: every block from its three non-owners
-  static constexpr int RA = 8, A_STAGE = BM * BK * 4;              // raw A: ring of 8 stages of 4 KB per wave
-  static constexpr int RING = RA * A_STAGE;
-  static constexpr int LDS_BYTES = NW * RING > RED_BYTES ? NW * RING : RED_BYTES;   // 128 KB
-};
-
-struct SlotKParams {
-  const void* a;         // ARAW = 0: slots [2][K/8][M] x 16 bytes; ARAW = 1: fp32 [M][lda]
-  const void* b_slots;   // [2][K/8][N] x 16 bytes
-  float* C;
-  const float* bias;
-  int M, N, K;
-  int64_t lda, ldb, ldc;   // ldb: cascmm_rawk_kernel only (raw B)
-  int tiles_m, tiles_n;
-  int group_m;             // tile rows an XCD's range of tiles walks down before moving one tile to the right
-};
-
 // Host-checked: K % 16 == 0, K >= 16, the slot buffers 16-byte aligned and below 2 GiB,
 // raw A 16-byte aligned with lda % 4 == 0 and M * lda * 4 below 2 GiB, C rows addressable with 32-bit
 // byte offsets inside a tile.
-template <int ARAW, int ABL = 0>
+template <int ARAW>
 __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_slotk_kernel(const SlotKParams p) {
   typedef SlotK T;
   extern __shared__ __attribute__((aligned(1024))) unsigned char slotk_smem[];
@@ -184,7 +163,6 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   }
 
   auto mfma = [&](u32x4 a, u32x4 b, f32x16 c) -> f32x16 {
-    if (ABL == 1) { asm volatile("" ::"v"(a), "v"(b)); return c; }
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   };
   // Stage i multiplies B from ring buffer i % D.  Its six MFMAs of column block ni are interleaved with
@@ -216,13 +194,11 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], Br[u][ni][1], acc[mi][ni]);
 #pragma unroll
         for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], Br[u][ni][0], acc[mi][ni]);
-        if (ABL != 2) {
-          if (ni == 0) issue_b(i + P, (u + P) % T::D, T::NTL - 1);
-          else issue_b(i + T::D, u, ni - 1);
-          if (ni < 4) {
-            if (ARAW) dma_a(i + AHEAD, ni);
-            else issue_a1(i + P, (u + P) % T::D, ni >> 1, ni & 1);
-          }
+        if (ni == 0) issue_b(i + P, (u + P) % T::D, T::NTL - 1);
+        else issue_b(i + T::D, u, ni - 1);
+        if (ni < 4) {
+          if (ARAW) dma_a(i + AHEAD, ni);
+          else issue_a1(i + P, (u + P) % T::D, ni >> 1, ni & 1);
         }
         if (ARAW) {
           if (ni < T::MT) read_a(i + 1, ni);
@@ -327,7 +303,6 @@ struct RawK {
 // Host-checked: fp32 operands, K % 16 == 0, K >= 16, N % 4 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
 // aligned, M * lda * 4 and K * ldb * 4 below 2 GiB, C rows addressable with 32-bit byte offsets inside a
 // tile.  c_vec: ldc % 4 == 0 and C 16-byte aligned (16-byte stores).
-template <int ABL = 0>
 __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_rawk_kernel(const SlotKParams p, int c_vec) {
   typedef SlotK T;
   constexpr int D = RawK::D, AHEAD = RawK::AHEAD;
@@ -441,7 +416,6 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   }
 
   auto mfma = [&](u32x4 a, u32x4 b, f32x16 c) -> f32x16 {
-    if (ABL == 1) { asm volatile("" ::"v"(a), "v"(b)); return c; }
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   };
   // Stage i, ring buffer u = i % D.  During column block ni: the MFMAs of the block; the split of the next
@@ -474,16 +448,14 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         for (int mi = 0; mi < T::MT; ++mi) acc[mi][ni] = mfma(Ar[ab][mi][0], H[cur], acc[mi][ni]);
         if (ni < T::NTL - 1) split_b(u, ni + 1, cur ^ 1);
         else split_b((u + 1) % D, 0, cur ^ 1);
-        if (ABL != 2) {
-          if (ni < 3) {
+        if (ni < 3) {
 #pragma unroll
-            for (int e = 3 * ni; e < (ni == 2 ? 8 : 3 * ni + 3); ++e) issue_bs(i + P, (u + P) % D, e);
-          } else {
+          for (int e = 3 * ni; e < (ni == 2 ? 8 : 3 * ni + 3); ++e) issue_bs(i + P, (u + P) % D, e);
+        } else {
 #pragma unroll
-            for (int e = 4 * (ni - 3); e < 4 * (ni - 3) + 4; ++e) issue_bq(i + D, u, e);
-          }
-          if (ni < 4) dma_a(i + AHEAD, ni);
+          for (int e = 4 * (ni - 3); e < 4 * (ni - 3) + 4; ++e) issue_bq(i + D, u, e);
         }
+        if (ni < 4) dma_a(i + AHEAD, ni);
         if (ni < T::MT) read_a(i + 1, ni);
         if (ni >= 1 && ni <= T::MT) split_a(ab ^ 1, ni - 1);
         // loads of this block: 4, 4, 3, 5, 4 -- one behind each of the first MFMAs

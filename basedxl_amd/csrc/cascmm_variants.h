@@ -375,8 +375,29 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
    LdsLayoutA<TileBD<BM, WN, BK, DEPTH, NP>, TERMS>::kBytes, true, false,                               \
    &launch_bdirect<TileBD<BM, WN, BK, DEPTH, NP>, FMT, TERMS, FULL, true>}
 
-// the chained feed-forward path (cascmm_inst_chain.hip)
-struct SlotKParams;
+// the kernels with K split over the waves of a workgroup and the chained feed-forward path
+// (cascmm_slotk_kernel.h, cascmm_inst_chain.hip)
+struct SlotK {
+  static constexpr int BM = 64, BN = 160, BK = 16, NW = 4, NT = 256, D = 4, GROUP_M = 8;
+  static constexpr int MT = 2, NTL = 5, BLOCKS = MT * NTL;
+  static constexpr int BLOCK_BYTES = 16 * 64 * 4;                  // one wave's 32 x 32 partial block
+  static constexpr int RED_BYTES = BLOCKS * 3 * BLOCK_BYTES;       // 120 KB: every block from its three non-owners
+  static constexpr int RA = 8, A_STAGE = BM * BK * 4;              // raw A: ring of 8 stages of 4 KB per wave
+  static constexpr int RING = RA * A_STAGE;
+  static constexpr int LDS_BYTES = NW * RING > RED_BYTES ? NW * RING : RED_BYTES;   // 128 KB
+};
+
+struct SlotKParams {
+  const void* a;         // ARAW = 0: slots [2][K/8][M] x 16 bytes; ARAW = 1: fp32 [M][lda]
+  const void* b_slots;   // [2][K/8][N] x 16 bytes
+  float* C;
+  const float* bias;
+  int M, N, K;
+  int64_t lda, ldb, ldc;   // ldb: cascmm_rawk_kernel only (raw B)
+  int tiles_m, tiles_n;
+  int group_m;             // tile rows an XCD's range of tiles walks down before moving one tile to the right
+};
+
 int launch_slotk(const SlotKParams& q, int araw, hipStream_t stream);
 int launch_prepare_left(const float* A, int M, int K, int64_t lda, void* out, hipStream_t stream);
 const void* slotk_kernel_handle(int araw);

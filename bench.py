@@ -76,8 +76,8 @@ def traffic_for(workload_name, launch, kernel):
         return None, "no counter run recorded for this launch in profiles/counter_traffic.txt"
     if row["kernel"] != kernel:
         return None, f"the recorded counter run ({row['profile']}) is of kernel {row['kernel']}, not of the one that ran"
-    return row["bytes"], (f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same counters read for a 256 MiB "
-                          f"copy; build {row['commit']}; {row['profile']}")
+    return row["bytes"], (f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same counters read for a device "
+                          f"copy of known size; build {row['commit']}; {row['profile']}")
 
 
 class Launch:

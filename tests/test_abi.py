@@ -136,6 +136,33 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
     assert pickp(2048, 5120, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre" and pickp(2048, 1280, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre"
 
 
+def test_counter_traffic_table_names_real_kernels_and_summaries():
+    """The table behind the bench's `roofline.traffic`: every row parses, names a kernel of the variant
+    table and a summary file that exists, and the rows of the pinned shapes name the kernels the
+    selection above pins for them (otherwise the bench would report null for them)."""
+    import os
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, root)
+    try:
+        import bench
+    finally:
+        sys.path.remove(root)
+    rows = bench.counter_traffic()
+    names = set(_lib.variant_names())
+    assert {("ffn", "ff.net.0.proj (W1)"), ("ffn", "ff.net.2 (W2)"), ("attn", "to_q/to_k/to_v grouped"), ("kv", "N=1280"), ("kv", "N=640")} <= set(rows)
+    for key, row in rows.items():
+        assert row["kernel"] in names, key
+        assert os.path.isfile(os.path.join(root, row["profile"])), key
+        assert row["bytes"] > 0 and len(row["commit"]) >= 7
+    assert rows[("ffn", "ff.net.0.proj (W1)")]["kernel"] == "t256x320x32_w512_bf16x2_tri"
+    assert rows[("ffn", "ff.net.2 (W2)")]["kernel"] == "k64x160x16_wk4_bf16x2_tri"
+    assert rows[("kv", "N=1280")]["kernel"] == "t32x32x32_wavek_bf16x2_tri"
+    got, why = bench.traffic_for("ffn", "ff.net.0.proj (W1)", "some_other_kernel")
+    assert got is None and "not of the one that ran" in why
+
+
 def test_scale_search_argument_validation():
     l = _lib.lib()
     ok = 16   # any non-NULL value: these calls return before touching the device
