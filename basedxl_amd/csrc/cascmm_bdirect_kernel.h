@@ -262,7 +262,7 @@ struct BDirectGemm {
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            llvm_raw_buffer_store_f32(v[4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+            llvm_raw_buffer_store_f32(v[4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kResultStoreAux);
       }
       return;
     }

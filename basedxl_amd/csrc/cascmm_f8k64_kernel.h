@@ -400,7 +400,7 @@ __global__ __launch_bounds__(F8K64T<MT>::NT) __attribute__((amdgpu_waves_per_eu(
         for (int q = 0; q < 4; ++q)
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            llvm_raw_buffer_store_f32(acc[mi][ni][4 * q + e] * out_scale + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+            llvm_raw_buffer_store_f32(acc[mi][ni][4 * q + e] * out_scale + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kLargeTileStoreAux);
     }
     return;
   }

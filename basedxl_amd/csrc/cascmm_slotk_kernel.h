@@ -272,7 +272,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          llvm_raw_buffer_store_f32(sum[4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+          llvm_raw_buffer_store_f32(sum[4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kResultStoreAux);
     }
   };
   if (wave == 0) reduce_and_store(std::integral_constant<int, 0>{});
@@ -525,12 +525,12 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         const int soff = (mi * 32 + W * 8 + e) * ldc_bytes;
         const f32x4 v4 = {sum[mi][0][e] + bq[0], sum[mi][1][e] + bq[1], sum[mi][2][e] + bq[2], sum[mi][3][e] + bq[3]};
         if (c_vec) {
-          llvm_raw_buffer_store_v4f32(v4, rc, voq, soff, 0);
+          llvm_raw_buffer_store_v4f32(v4, rc, voq, soff, kResultStoreAux);
         } else {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) llvm_raw_buffer_store_f32(v4[j], rc, inq ? voq + 4 * j : c_bytes, soff, 0);
+          for (int j = 0; j < 4; ++j) llvm_raw_buffer_store_f32(v4[j], rc, inq ? voq + 4 * j : c_bytes, soff, kResultStoreAux);
         }
-        llvm_raw_buffer_store_f32(sum[mi][4][e] + bs, rc, vos, soff, 0);
+        llvm_raw_buffer_store_f32(sum[mi][4][e] + bs, rc, vos, soff, kResultStoreAux);
       }
   };
   if (wave == 0) reduce_and_store(std::integral_constant<int, 0>{});

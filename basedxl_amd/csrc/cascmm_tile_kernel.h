@@ -131,6 +131,15 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 __device__ void llvm_raw_buffer_store_v2f32(f32x2 v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v2f32");
 __device__ void llvm_raw_buffer_store_i16(short v, i32x4 rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.i16");
 
+// Cache policy of the result stores: sc1 (agent scope) for the kernels with small tiles, the default for the
+// large ones.  A/B on one box, whole kernels: 2048x1280x1280 27.1 -> 26.4 us, 4096x640x640 18.2 -> 17.6 us,
+// 8192x640x640 31.7 -> 30.5 us, 2048x5120x1280 83.3 -> 82.7 us with sc1; the 256x320 and the fp8-rate tiles,
+// whose workgroups store 160-320 KB each at the same moment, measured 0.0-0.4 % slower with it and keep the
+// default.  (A bare store loop of the large tile's pattern is faster with sc1, 16.5 -> 13.9 us for 84 MB, and
+// slower with nt, 18.2 us.)
+constexpr int kResultStoreAux = 16;
+constexpr int kLargeTileStoreAux = 0;
+
 // gfx9-family raw buffer descriptor: 48-bit base, stride 0, byte count, 32-bit data format
 __device__ __forceinline__ i32x4 make_rsrc(const void* base, int64_t bytes) {
   const uint64_t b = (uint64_t)base;
@@ -794,8 +803,8 @@ struct TileGemm {
               for (int e = 0; e < 4; ++e) {
                 const float y = gated(res[mi][2 * nj][4 * q + e] + bv, res[mi][2 * nj + 1][4 * q + e] + bg);
                 const int soff = (mi * 32 + q * 8 + e) * ldc_bytes;
-                if constexpr (IODT == CASCMM_DT_F32) llvm_raw_buffer_store_f32(y, rc, voff, soff, 0);
-                else llvm_raw_buffer_store_i16(__builtin_bit_cast(short, (IoT)y), rc, voff, soff, 0);
+                if constexpr (IODT == CASCMM_DT_F32) llvm_raw_buffer_store_f32(y, rc, voff, soff, kResultStoreAux);
+                else llvm_raw_buffer_store_i16(__builtin_bit_cast(short, (IoT)y), rc, voff, soff, kResultStoreAux);
               }
         }
         return;
@@ -843,10 +852,10 @@ struct TileGemm {
               if constexpr (RUN == 4) {
                 const f32x4 v = {res[mi][r0][4 * q + e] + bv[0], res[mi][r0 + 1][4 * q + e] + bv[1],
                                  res[mi][r0 + 2][4 * q + e] + bv[2], res[mi][r0 + 3][4 * q + e] + bv[3]};
-                llvm_raw_buffer_store_v4f32(v, rc, voff, soff, 0);
+                llvm_raw_buffer_store_v4f32(v, rc, voff, soff, kResultStoreAux);
               } else {
                 const f32x2 v = {res[mi][r0][4 * q + e] + bv[0], res[mi][r0 + 1][4 * q + e] + bv[1]};
-                llvm_raw_buffer_store_v2f32(v, rc, voff, soff, 0);
+                llvm_raw_buffer_store_v2f32(v, rc, voff, soff, kResultStoreAux);
               }
             }
       }
@@ -862,7 +871,7 @@ struct TileGemm {
           for (int q = 0; q < 4; ++q)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              llvm_raw_buffer_store_f32(res[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+              llvm_raw_buffer_store_f32(res[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kResultStoreAux);
       }
       return;
     }
@@ -882,7 +891,7 @@ struct TileGemm {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const IoT h = (IoT)(res[mi][ni][4 * q + e] + bv);
-              llvm_raw_buffer_store_i16(__builtin_bit_cast(short, h), rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+              llvm_raw_buffer_store_i16(__builtin_bit_cast(short, h), rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kResultStoreAux);
             }
       }
       return;

@@ -363,8 +363,8 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
           }
           u32x4 t[2];
           split8<CASCMM_FMT_BF16, 2>(r8, t);
-          llvm_raw_buffer_store_v4f32(__builtin_bit_cast(f32x4, t[0]), rc, voff + mi * 512, soff, 0);
-          llvm_raw_buffer_store_v4f32(__builtin_bit_cast(f32x4, t[1]), rc, voff + mi * 512, soff + term1, 0);
+          llvm_raw_buffer_store_v4f32(__builtin_bit_cast(f32x4, t[0]), rc, voff + mi * 512, soff, kLargeTileStoreAux);
+          llvm_raw_buffer_store_v4f32(__builtin_bit_cast(f32x4, t[1]), rc, voff + mi * 512, soff + term1, kLargeTileStoreAux);
         }
       }
     };
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
           for (int e = 0; e < 4; ++e) {
             const int r = 4 * q + e;
             const float gl = gate_in_lds ? xbuf[(mi * 16 + r) * 64 + elane] : gelu_value(acc[mi][gb][r] + bg);
-            llvm_raw_buffer_store_f32((acc[mi][vb][r] + bv) * gl, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+            llvm_raw_buffer_store_f32((acc[mi][vb][r] + bv) * gl, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kLargeTileStoreAux);
           }
     };
     if ((wave & 1) == 0) {
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
       for (int q = 0; q < 4; ++q)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          llvm_raw_buffer_store_f32(acc[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, 0);
+          llvm_raw_buffer_store_f32(acc[mi][ni][4 * q + e] + bv, rc, voff, (mi * 32 + q * 8 + e) * ldc_bytes, kLargeTileStoreAux);
   }
 }
 
