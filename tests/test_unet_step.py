@@ -297,6 +297,29 @@ def test_fp8x3_whole_results_at_every_linear_shape_of_a_step(gpu_device, prepare
         del ad, bd, y, exact
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("prepared", [False, True], ids=["weights split per call", "weights kept split"])
+def test_bf16x2_whole_results_at_every_linear_shape_of_a_step(gpu_device, prepared):
+    """The same for the two-term bf16 cascade, whose kernels differ from shape to shape (large tile, K split
+    over the waves of a workgroup, LDS-tiled, skinny): 1.25x on both metrics over the whole result, no exceptions."""
+    from basedxl_amd import PreparedWeight, cascaded_lowp_matmul
+    torch.set_num_threads(min(16, torch.get_num_threads() or 16))
+    for (M, K, N) in FP8_STEP_SHAPES:
+        if prepared and M < 32:
+            continue
+        a, b = oc.make_operands(M, K, N, seed=200 + M + N, w_std=0.02)
+        ad, bd = a.to(gpu_device), b.to(gpu_device)
+        exact = (ad.double() @ bd.double()).cpu()
+        e_ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exact)
+        y = cascaded_lowp_matmul(ad, PreparedWeight(bd, lowp="bf16", terms=2) if prepared else bd)
+        e_got = oc.error_metrics(y.cpu(), exact)
+        _say(f"  bf16x2 whole result {M}x{K}x{N}: rel_fro x{e_got['rel_fro'] / e_ref['rel_fro']:.3f} max_abs "
+             f"x{e_got['max_abs'] / e_ref['max_abs']:.3f}")
+        assert e_got["rel_fro"] <= TOL * e_ref["rel_fro"], (M, K, N)
+        assert e_got["max_abs"] <= TOL * e_ref["max_abs"], (M, K, N)
+        del ad, bd, y, exact
+
+
 def _integer_layer(kind, K, N, gen):
     """A routed module of the given kind and shape whose weights are small integers."""
     w = torch.randint(-4, 5, (N, K), generator=gen).float()
