@@ -670,6 +670,17 @@ def glu_chained_supported(a: torch.Tensor, N: int) -> bool:
                 and K >= 32 and chained_supported(M, 32, N // 2) and 4 * M * (N // 2) < 2 ** 31)
 
 
+def glu_chained_worthwhile(a: torch.Tensor, N: int) -> bool:
+    """Whether the library's cost estimates put the large-tile kernel with the gate in its store -- the
+    only kernel that can write operand slots -- ahead of the best plain kernel plus a gate pass for ``a``
+    times a ``[K, N]`` gated weight.  With few tiles on many CUs (1024 rows) they do not, and a
+    feed-forward block is faster layer by layer."""
+    K = a.shape[-1]
+    M = a.numel() // K if K else 0
+    return glu_chained_supported(a, N) and _lib.lib().cascmm_select_variant_glu(
+        M, N, K, K, N, N // 2, _lib.DT_F32, _lib.FMT_BF16, 2, _lib.PROD_TRI) >= 0
+
+
 def cascaded_lowp_matmul_glu_chained(a: torch.Tensor, w, *, bias: Optional[torch.Tensor] = None,
                                      out: Optional[LeftSlots] = None) -> LeftSlots:
     """``h = a @ w + bias; value, gate = h.chunk(2, -1); value * gelu(gate)`` like

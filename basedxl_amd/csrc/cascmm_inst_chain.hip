@@ -56,7 +56,7 @@ int launch_slotk(const SlotKParams& q, int araw, hipStream_t stream) {
 static int launch_slotk_variant(const GroupParams& p, hipStream_t stream) {
   if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_slotk_kernel<1>; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
-  if (p.K % SlotK::BK != 0 || p.K < SlotK::BK) return CASCMM_ERR_BAD_VARIANT;
+  if (p.K % (2 * SlotK::BK) != 0 || p.K < 2 * SlotK::BK) return CASCMM_ERR_BAD_VARIANT;   // raw A comes in pairs of stages
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.N * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(SlotK::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
   SlotKParams q;
@@ -71,7 +71,7 @@ static int launch_rawk_variant(const GroupParams& p, hipStream_t stream) {
   typedef SlotK T;
   if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_rawk_kernel; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
-  if (p.K % T::BK != 0 || p.K < T::BK || p.N % 4 != 0) return CASCMM_ERR_BAD_VARIANT;
+  if (p.K % (2 * T::BK) != 0 || p.K < 2 * T::BK || p.N % 4 != 0) return CASCMM_ERR_BAD_VARIANT;   // raw A comes in pairs of stages
   if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.ldb * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
     return CASCMM_ERR_TOO_LARGE;
   auto kfn = cascmm_rawk_kernel;

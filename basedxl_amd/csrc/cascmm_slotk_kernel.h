@@ -31,7 +31,7 @@
 
 namespace cascmm {
 
-// Host-checked: K % 16 == 0, K >= 16, the slot buffers 16-byte aligned and below 2 GiB,
+// Host-checked: K % 16 == 0, K >= 16 (raw A: K % 32 == 0), the slot buffers 16-byte aligned and below 2 GiB,
 // raw A 16-byte aligned with lda % 4 == 0 and M * lda * 4 below 2 GiB, C rows addressable with 32-bit
 // byte offsets inside a tile.
 template <int ARAW>
@@ -58,13 +58,19 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int kgroups = p.K >> 3;
   const int ksteps = p.K >> 4;
-  const int n_own = (ksteps - wave + T::NW - 1) / T::NW;   // 0 for the last waves of a very short K: they add zeros
-  // Own stage i is stage wave + 4 i of the problem.  The loop below runs in trips of D stages and has no
-  // branch inside a trip (a branch costs the compiler its count of the loads in flight, and it then waits
-  // for all of them).  A wave whose number of stages is not a multiple of D runs up to D - 1 stages past
-  // its last one: their slot loads point beyond the end of the buffers and return zeros, whose products
-  // add nothing (raw A: the last stage again, times the zero slots of B).
-  auto step_of = [&](int i) { return wave + T::NW * (i < n_own ? i : (n_own > 0 ? n_own - 1 : 0)); };
+  // Which 16-k stages of the problem a wave owns.  A as slots: every fourth one, own stage i = stage
+  // wave + 4 i.  A raw: every fourth PAIR of stages, own stage i = stage 8 (i / 2) + 2 wave + i % 2, so that
+  // what the wave fetches of a row for a pair is one whole 128-byte line (with every fourth stage it was half
+  // a line, and the L1 fetched the whole line for either half: 1.8 requests per line of A, counted).
+  // n_own: the number of own stages, 0 for the last waves of a very short K (they add zeros).
+  const int n_own = ARAW ? 2 * (ksteps >> 3) + (((ksteps & 7) - 2 * wave) < 0 ? 0 : ((ksteps & 7) - 2 * wave) > 2 ? 2 : ((ksteps & 7) - 2 * wave))
+                         : (ksteps - wave + T::NW - 1) / T::NW;
+  auto stage_of = [&](int i) { return ARAW ? 8 * (i >> 1) + 2 * wave + (i & 1) : wave + T::NW * i; };
+  // The loop below runs in trips of D stages and has no branch inside a trip (a branch costs the compiler
+  // its count of the loads in flight, and it then waits for all of them).  A wave whose number of stages is
+  // not a multiple of D runs up to D - 1 stages past its last one: their slot loads point beyond the end of
+  // the buffers and return zeros, whose products add nothing (raw A: finite values of the problem's first
+  // stage, times the zero slots of B).
 
   // ---- right operand: lane (l31, g) reads k group 2 step + g, column block ni 512 bytes further ----
   const i32x4 rb = make_rsrc(p.b_slots, (int64_t)2 * kgroups * p.N * 16);
@@ -74,7 +80,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   u32x4 Br[T::D][T::NTL][2];               // [ring buffer][column block][term]
   const int b_end = 2 * b_term;            // the buffer's size: every offset from there on is outside
   auto issue_b = [&](int i, int buf, int ni) {
-    const int base = i < n_own ? (wave + T::NW * i) * b_step : b_end;
+    const int base = i < n_own ? stage_of(i) * b_step : b_end;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
       Br[buf][ni][t] = __builtin_bit_cast(u32x4, llvm_raw_buffer_load_v4f32(rb, vb + ni * 512, base + t * b_term, 0));
@@ -86,7 +92,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int a_term = kgroups * p.M * 16, a_step = 2 * p.M * 16;
   u32x4 Ar[ARAW ? 2 : T::D][T::MT][2];     // slots: [ring buffer][row block][term]; raw: [stage parity] after the split
   auto issue_a1 = [&](int i, int buf, int mi, int t) {
-    const int base = i < n_own ? (wave + T::NW * i) * a_step : 2 * a_term;
+    const int base = i < n_own ? stage_of(i) * a_step : 2 * a_term;
     Ar[buf][mi][t] = __builtin_bit_cast(u32x4, llvm_raw_buffer_load_v4f32(ra, va + mi * 512, base + t * a_term, 0));
   };
 
@@ -96,20 +102,35 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const __amdgpu_buffer_rsrc_t rar =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, ARAW ? (int)(a_bytes > 0x7FFFFFFF ? 0x7FFFFFFF : a_bytes) : 0, 0x00020000);
   unsigned char* ring = slotk_smem + wave * T::RING;
-  // load j of a stage: rows 16 j + lane / 4, LDS position 4 row + pos holds chunk (pos - row / 4) mod 4
-  const int dma_voff = (int)(((int64_t)(m0 + (lane >> 2)) * p.lda + (((lane & 3) - (lane >> 4)) & 3) * 4) * 4);
-  const int dma_rows16 = (int)p.lda * 64;   // bytes from one load's rows to the next one's
-  auto dma_a = [&](int i, int j) {
-    wavek_load_lds(rar, ring + (i & (T::RA - 1)) * T::A_STAGE + j * 1024, dma_voff, step_of(i) * (T::BK * 4) + j * dma_rows16);
+  // A pair of stages in LDS: 64 rows x 128 bytes (eight 16-byte chunks of 4 k).  Load j of a pair (0 .. 7)
+  // brings rows 8 j + lane / 8; position pos of a row holds chunk (pos - row / 2) mod 8, which spreads the
+  // fragment reads of 16 consecutive rows over all banks.  (row / 2) mod 8 = (4 j + lane / 16) mod 8: two
+  // offsets per lane, by the parity of j.  K % 32 == 0 (host-checked for raw A), so a wave's pairs are whole.
+  int dma_voff[2];
+#pragma unroll
+  for (int jp = 0; jp < 2; ++jp)
+    dma_voff[jp] = (int)(((int64_t)(m0 + (lane >> 3)) * p.lda + (((lane & 7) - (4 * jp + (lane >> 4))) & 7) * 4) * 4);
+  const int dma_rows8 = (int)p.lda * 32;   // bytes from one load's rows to the next one's
+  // the part ni (0 .. 3) of own stage i's share of its pair's loads: load 4 sp + ni of pair i / 2, sp = i % 2
+  // (passed separately: a constant where i is not); past the wave's last pair: the problem's first pair
+  // (finite values for the zero slots of B to multiply, whatever lies beyond K)
+  auto dma_a = [&](int i, int ni, int sp) {
+    const int q = i >> 1, j = 4 * sp + ni;
+    const int koff = 2 * q < n_own ? stage_of(2 * q) * (T::BK * 4) : 0;
+    wavek_load_lds(rar, ring + (q & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + j * 1024, dma_voff[ni & 1], koff + j * dma_rows8);
   };
-  // fragment of lane (l31, g), row block mi: row 32 mi + l31, chunks 2 g and 2 g + 1 at their rotated places
-  const int a_frag0 = l31 * 64 + ((2 * g + (l31 >> 2)) & 3) * 16;
-  const int a_frag1 = l31 * 64 + ((2 * g + 1 + (l31 >> 2)) & 3) * 16;
+  // fragment of lane (l31, g), row block mi, stage parity s: row 32 mi + l31, chunks 4 s + 2 g and 4 s + 2 g + 1
+  // at their rotated places
+  int a_frag[2][2];
+#pragma unroll
+  for (int sp = 0; sp < 2; ++sp)
+#pragma unroll
+    for (int x = 0; x < 2; ++x) a_frag[sp][x] = l31 * 128 + ((4 * sp + 2 * g + x + (l31 >> 1)) & 7) * 16;
   f32x4 X[T::MT][2];   // raw fragments of the next stage on their way to the split
-  auto read_a = [&](int i, int mi) {
-    const unsigned char* st = ring + (i & (T::RA - 1)) * T::A_STAGE + mi * 2048;
-    X[mi][0] = *(const f32x4*)(st + a_frag0);
-    X[mi][1] = *(const f32x4*)(st + a_frag1);
+  auto read_a = [&](int i, int mi, int sp) {   // sp = i % 2
+    const unsigned char* st = ring + ((i >> 1) & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + mi * 4096;
+    X[mi][0] = *(const f32x4*)(st + a_frag[sp][0]);
+    X[mi][1] = *(const f32x4*)(st + a_frag[sp][1]);
   };
   auto split_a = [&](int buf, int mi) {
     float r[8] = {X[mi][0][0], X[mi][0][1], X[mi][0][2], X[mi][0][3], X[mi][1][0], X[mi][1][1], X[mi][1][2], X[mi][1][3]};
@@ -122,16 +143,17 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // ---- prologue ---------------------------------------------------------------------------------------
   // B: stages 0 .. D - 2 whole, of stage D - 1 the column blocks 0 .. 3 (its last column block is loaded
   // during stage 0, like that of every later stage: see the loop).  A as slots: stages 0 .. D - 2.
-  // A raw: stages 0 .. AHEAD - 1 FIRST, then stage 0 of B, then the rest: the wait below names exactly the
-  // rest, so everything the first AHEAD - 1 stages read from LDS has landed when the loop starts (later
-  // stages: see the wait at the top of a stage).
-  constexpr int AHEAD = T::RA - 2;   // raw A: stage i + AHEAD is requested during stage i
+  // A raw: stages 0 .. AHEAD - 1 (three pairs) FIRST, then stage 0 of B, then the rest: the wait below names
+  // exactly the rest, so everything the first AHEAD - 1 stages read from LDS has landed when the loop starts
+  // (later stages: see the wait at the top of a stage).
+  constexpr int AHEAD = T::RA - 2;   // raw A: stage i + AHEAD's share of its pair is requested during stage i
+  static_assert(AHEAD % 2 == 0, "a stage and the one AHEAD of it sit at the same place of their pairs");
   f32x16 acc[T::MT][T::NTL];
   if (ARAW) {
 #pragma unroll
     for (int d = 0; d < AHEAD; ++d)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dma_a(d, j);
+      for (int j = 0; j < 4; ++j) dma_a(d, j, d & 1);
 #pragma unroll
     for (int ni = 0; ni < T::NTL; ++ni) issue_b(0, 0, ni);
     __builtin_amdgcn_sched_barrier(0);   // (the wait below counts on everything above being older than everything below)
@@ -157,7 +179,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (LATER & 0xF) | ((LATER >> 4) << 14));
 #pragma unroll
-    for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi);
+    for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi, 0);
 #pragma unroll
     for (int mi = 0; mi < T::MT; ++mi) split_a(0, mi);
   }
@@ -169,17 +191,18 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // loads into registers that are free by then: the two slots of column block ni - 1 of stage i + D
   // (same buffer; ni = 0: the last column block of the previous buffer's next stage) and, A as slots,
   // one of the four row slots of the previous buffer's next stage, i + D - 1.  A raw: one of the four
-  // loads of stage i + AHEAD into the ring (its place was last read during stage i - 3), and the
-  // fragments of stage i + 1.  Those were requested during stage i + 1 - AHEAD; a stage issues 14 loads and
-  // nothing moves across a stage's end, so once at most 14 (AHEAD - 2) loads are outstanding at the top of
-  // stage i they have landed (the wait is explicit: the compiler does not connect a load into LDS with the
-  // read of that LDS address).
+  // loads of stage i + AHEAD's pair into the ring (its place was last read during stage i - 2 or earlier),
+  // and the fragments of stage i + 1.  An odd stage reads the first fragments of a new pair, whose last loads
+  // were requested during stage i + 2 - AHEAD; a stage issues 14 loads and nothing moves across a stage's end,
+  // so once at most 14 (AHEAD - 3) loads are outstanding at the top of an odd stage the pair has landed, for
+  // the even stage after it as well (the wait is explicit: the compiler does not connect a load into LDS
+  // with the read of that LDS address).
   for (int i0 = 0; i0 < n_own; i0 += T::D) {
 #pragma unroll
     for (int u = 0; u < T::D; ++u) {
       const int i = i0 + u;
-      if (ARAW) {
-        constexpr int YOUNGER = 14 * (AHEAD - 2);   // 56
+      if (ARAW && (u & 1)) {
+        constexpr int YOUNGER = 14 * (AHEAD - 3);   // 42
         static_assert(YOUNGER <= 63, "the wait counter has six bits");
         __builtin_amdgcn_s_waitcnt(0x0F70 | (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14));
       }
@@ -197,11 +220,11 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         if (ni == 0) issue_b(i + P, (u + P) % T::D, T::NTL - 1);
         else issue_b(i + T::D, u, ni - 1);
         if (ni < 4) {
-          if (ARAW) dma_a(i + AHEAD, ni);
+          if (ARAW) dma_a(i + AHEAD, ni, u & 1);
           else issue_a1(i + P, (u + P) % T::D, ni >> 1, ni & 1);
         }
         if (ARAW) {
-          if (ni < T::MT) read_a(i + 1, ni);
+          if (ni < T::MT) read_a(i + 1, ni, (u + 1) & 1);
           if (ni >= 1 && ni <= T::MT) split_a(ab ^ 1, ni - 1);
         }
         // two MFMAs, one load, three times (the last block has two loads)
@@ -297,10 +320,10 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 // the same LDS traffic, and the 16-byte stores stay possible.
 // ---------------------------------------------------------------------------------------------------
 struct RawK {
-  static constexpr int D = 4, AHEAD = 5;   // B ring in registers; raw A requested this many stages ahead
+  static constexpr int D = 4, AHEAD = 6;   // B ring in registers; raw A requested this many stages ahead (even: whole pairs)
 };
 
-// Host-checked: fp32 operands, K % 16 == 0, K >= 16, N % 4 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
+// Host-checked: fp32 operands, K % 32 == 0, N % 4 == 0, lda % 4 == 0, ldb % 4 == 0, A and B 16-byte
 // aligned, M * lda * 4 and K * ldb * 4 below 2 GiB, C rows addressable with 32-bit byte offsets inside a
 // tile.  c_vec: ldc % 4 == 0 and C 16-byte aligned (16-byte stores).
 __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void cascmm_rawk_kernel(const SlotKParams p, int c_vec) {
@@ -323,7 +346,10 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   }
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int ksteps = p.K >> 4;
-  const int n_own = (ksteps - wave + T::NW - 1) / T::NW;   // 0 for the last waves of a very short K: they add zeros
+  // a wave owns every fourth PAIR of 16-k stages (see the kernel above): own stage i = stage 8 (i / 2) + 2 wave + i % 2
+  const int own_tail = (ksteps & 7) - 2 * wave;
+  const int n_own = 2 * (ksteps >> 3) + (own_tail < 0 ? 0 : own_tail > 2 ? 2 : own_tail);   // 0 for the last waves of a very short K: they add zeros
+  auto stage_of = [&](int i) { return 8 * (i >> 1) + 2 * wave + (i & 1); };
   const int ldb_bytes = (int)p.ldb * 4;
 
   // ---- B: rows 8 g .. 8 g + 7 of a stage; beyond the last stage the loads point past the end of the
@@ -335,7 +361,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int vbs = 8 * g * ldb_bytes + (n0 + 128 + l31) * 4;
   f32x4 Bq[D][8];   // [ring buffer][k]: columns 4 l31 .. 4 l31 + 3
   float Bs[D][8];   // column 128 + l31
-  auto b_base = [&](int i) { return i < n_own ? (wave + T::NW * i) * (T::BK * ldb_bytes) : b_bytes; };
+  auto b_base = [&](int i) { return i < n_own ? stage_of(i) * (T::BK * ldb_bytes) : b_bytes; };
   auto issue_bq = [&](int i, int buf, int e) { Bq[buf][e] = llvm_raw_buffer_load_v4f32(rb, vbq, b_base(i) + e * ldb_bytes, 0); };
   auto issue_bs = [&](int i, int buf, int e) { Bs[buf][e] = llvm_raw_buffer_load_f32(rb, vbs, b_base(i) + e * ldb_bytes, 0); };
   u32x4 H[2], L[2];   // the split operand of the current / next block
@@ -354,20 +380,27 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const __amdgpu_buffer_rsrc_t rar =
       __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)(a_bytes > 0x7FFFFFFF ? 0x7FFFFFFF : a_bytes), 0x00020000);
   unsigned char* ring = slotk_smem + wave * T::RING;
-  const int dma_voff = (int)(((int64_t)(m0 + (lane >> 2)) * p.lda + (((lane & 3) - (lane >> 4)) & 3) * 4) * 4);
-  const int dma_rows16 = (int)p.lda * 64;
-  auto dma_a = [&](int i, int j) {
-    const int step = wave + T::NW * (i < n_own ? i : (n_own > 0 ? n_own - 1 : 0));
-    wavek_load_lds(rar, ring + (i & (T::RA - 1)) * T::A_STAGE + j * 1024, dma_voff, step * (T::BK * 4) + j * dma_rows16);
+  int dma_voff[2];
+#pragma unroll
+  for (int jp = 0; jp < 2; ++jp)
+    dma_voff[jp] = (int)(((int64_t)(m0 + (lane >> 3)) * p.lda + (((lane & 7) - (4 * jp + (lane >> 4))) & 7) * 4) * 4);
+  const int dma_rows8 = (int)p.lda * 32;
+  auto dma_a = [&](int i, int ni, int sp) {   // sp = i % 2
+    const int q = i >> 1, j = 4 * sp + ni;
+    const int koff = 2 * q < n_own ? stage_of(2 * q) * (T::BK * 4) : 0;
+    wavek_load_lds(rar, ring + (q & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + j * 1024, dma_voff[ni & 1], koff + j * dma_rows8);
   };
-  const int a_frag0 = l31 * 64 + ((2 * g + (l31 >> 2)) & 3) * 16;
-  const int a_frag1 = l31 * 64 + ((2 * g + 1 + (l31 >> 2)) & 3) * 16;
+  int a_frag[2][2];
+#pragma unroll
+  for (int sp = 0; sp < 2; ++sp)
+#pragma unroll
+    for (int x = 0; x < 2; ++x) a_frag[sp][x] = l31 * 128 + ((4 * sp + 2 * g + x + (l31 >> 1)) & 7) * 16;
   f32x4 X[T::MT][2];
   u32x4 Ar[2][T::MT][2];   // [stage parity][row block][term]
-  auto read_a = [&](int i, int mi) {
-    const unsigned char* st = ring + (i & (T::RA - 1)) * T::A_STAGE + mi * 2048;
-    X[mi][0] = *(const f32x4*)(st + a_frag0);
-    X[mi][1] = *(const f32x4*)(st + a_frag1);
+  auto read_a = [&](int i, int mi, int sp) {   // sp = i % 2
+    const unsigned char* st = ring + ((i >> 1) & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + mi * 4096;
+    X[mi][0] = *(const f32x4*)(st + a_frag[sp][0]);
+    X[mi][1] = *(const f32x4*)(st + a_frag[sp][1]);
   };
   auto split_a = [&](int buf, int mi) {
     float r[8] = {X[mi][0][0], X[mi][0][1], X[mi][0][2], X[mi][0][3], X[mi][1][0], X[mi][1][1], X[mi][1][2], X[mi][1][3]};
@@ -377,13 +410,13 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     Ar[buf][mi][1] = t[1];
   };
 
-  // ---- prologue: raw A of stages 0 .. AHEAD - 1 and stage 0 of B first (36 loads), then the rest of B
-  // (40 loads: the wait below names exactly those) ----
+  // ---- prologue: raw A of stages 0 .. AHEAD - 1 (three pairs) and stage 0 of B first (40 loads), then the
+  // rest of B (40 loads: the wait below names exactly those) ----
   f32x16 acc[T::MT][T::NTL];
 #pragma unroll
   for (int d = 0; d < AHEAD; ++d)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dma_a(d, j);
+    for (int j = 0; j < 4; ++j) dma_a(d, j, d & 1);
 #pragma unroll
   for (int e = 0; e < 8; ++e) issue_bq(0, 0, e);
 #pragma unroll
@@ -409,7 +442,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0x0F70 | (LATER & 0xF) | ((LATER >> 4) << 14));
 #pragma unroll
-    for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi);
+    for (int mi = 0; mi < T::MT; ++mi) read_a(0, mi, 0);
 #pragma unroll
     for (int mi = 0; mi < T::MT; ++mi) split_a(0, mi);
     split_b(0, 0, 0);
@@ -423,15 +456,16 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // the single column of the PREVIOUS buffer's next stage (its last reader was the split during the
   // previous stage's block 3), ni = 3, 4: the four adjacent columns of this buffer's next stage (last read
   // by the split during block 2); ni = 0 .. 3: one load of raw A into the LDS ring; ni = 0, 1: the A
-  // fragments of the next stage, split during ni = 1, 2.  Those fragments were requested during stage
-  // i + 1 - AHEAD; a stage issues 20 loads and nothing moves across a stage's end, so once at most
-  // 20 (AHEAD - 2) = 60 loads are outstanding at the top of stage i they have landed.
+  // fragments of the next stage, split during ni = 1, 2.  An odd stage reads the first fragments of a new
+  // pair, whose last loads were requested during stage i + 2 - AHEAD; a stage issues 20 loads and nothing
+  // moves across a stage's end, so once at most 20 (AHEAD - 3) = 60 loads are outstanding at the top of an
+  // odd stage the pair has landed, for the even stage after it as well.
   for (int i0 = 0; i0 < n_own; i0 += D) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
       const int i = i0 + u;
-      {
-        constexpr int YOUNGER = 20 * (AHEAD - 2);
+      if (u & 1) {
+        constexpr int YOUNGER = 20 * (AHEAD - 3);
         static_assert(YOUNGER <= 63, "the wait counter has six bits");
         __builtin_amdgcn_s_waitcnt(0x0F70 | (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14));
       }
@@ -455,8 +489,8 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #pragma unroll
           for (int e = 4 * (ni - 3); e < 4 * (ni - 3) + 4; ++e) issue_bq(i + D, u, e);
         }
-        if (ni < 4) dma_a(i + AHEAD, ni);
-        if (ni < T::MT) read_a(i + 1, ni);
+        if (ni < 4) dma_a(i + AHEAD, ni, u & 1);
+        if (ni < T::MT) read_a(i + 1, ni, (u + 1) & 1);
         if (ni >= 1 && ni <= T::MT) split_a(ab ^ 1, ni - 1);
         // loads of this block: 4, 4, 3, 5, 4 -- one behind each of the first MFMAs
         constexpr int kLoads[5] = {4, 4, 3, 5, 4};

@@ -15,7 +15,7 @@ import torch
 import torch.nn as nn
 
 from ..cascaded_lowp_matmul import (ChainedWeight, PreparedWeight, cascaded_lowp_matmul_chained, cascaded_lowp_matmul_glu_chained,
-                                    chained_supported, glu_chained_supported)
+                                    chained_supported, glu_chained_worthwhile)
 from .geglu import BasedXLLowPGEGLU
 from .lowp_linear import BasedXLLowPLinear
 
@@ -25,7 +25,8 @@ class BasedXLChainedFeedForward(nn.Module):
     and ``out`` ([inner] -> [out]) are the two ``nn.Linear`` layers of the block.
 
     The chain runs for fp32 activations on the GPU, two bf16 terms, rows % 256 == 0, inner % 160 == 0,
-    in % 32 == 0; anything else goes through :class:`BasedXLLowPGEGLU` and :class:`BasedXLLowPLinear`,
+    in % 32 == 0, and where the library's estimates favour the large-tile kernel with the gate in its store
+    over a plain kernel plus a gate pass (few rows on many CUs: they do not); anything else goes through :class:`BasedXLLowPGEGLU` and :class:`BasedXLLowPLinear`,
     which this module also holds (same weights).  ``prepared=True`` keeps the first weight split as
     well (the second one always is: the chained GEMM has no other form)."""
 
@@ -45,7 +46,7 @@ class BasedXLChainedFeedForward(nn.Module):
         if not (self.chainable and x.is_cuda and x.dtype == torch.float32) or torch.compiler.is_compiling():
             return False
         M = x.numel() // self.in_features
-        return glu_chained_supported(x, 2 * self.inner) and chained_supported(M, self.out_features, self.inner)
+        return glu_chained_worthwhile(x, 2 * self.inner) and chained_supported(M, self.out_features, self.inner)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if not self._chain_ok(x):

@@ -266,7 +266,7 @@ def bench_kv(dev, check=True):
 
 
 def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False), ("bf16", 2, True, False), ("fp8", 3, True, False),
-                              ("bf16", 2, False, True), ("bf16", 2, True, "chain")),
+                              ("bf16", 2, False, True), ("bf16", 2, True, True), ("bf16", 2, True, "chain")),
                latents=(("full latent", None), ("half-latent share", 64)), forward=True):
     """cfg5: the routed layers of one UNet step.  The module tree is built on the GPU with random
     weights and patched through the config switch; one forward pass records every routed call; those
@@ -524,7 +524,7 @@ def main():
                          "every step, resident in the Infinity Cache; 8 = every step reads HBM-cold data)")
     ap.add_argument("--unet-select", default="",
                     help="unet only: run one configuration instead of all ten, as cascade:weights:latent, e.g. "
-                         "bf16x2:raw:full, fp8x3:prepared:half, bf16x2:raw+geglu:full or bf16x2:prepared+chain:full (what a profiler run wants)")
+                         "bf16x2:raw:full, fp8x3:prepared:half, bf16x2:raw+geglu:full, bf16x2:prepared+geglu:full or bf16x2:prepared+chain:full (what a profiler run wants)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -572,8 +572,8 @@ def main():
             if args.unet_select:
                 casc, wts, lat = args.unet_select.split(":")
                 lowp, terms = casc.split("x")
-                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts in ("prepared", "prepared+chain") else False if wts == "raw+geglu" else None,
-                                                "chain" if wts == "prepared+chain" else wts == "raw+geglu"),),
+                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts in ("prepared", "prepared+chain", "prepared+geglu") else False if wts == "raw+geglu" else None,
+                                                "chain" if wts == "prepared+chain" else wts in ("raw+geglu", "prepared+geglu")),),
                                 latents=(("full latent", None),) if lat == "full" else (("half-latent share", 64),), forward=False)
             else:
                 un = bench_unet(dev)

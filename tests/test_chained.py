@@ -302,9 +302,9 @@ def test_chained_feed_forward_module_and_its_fallback(gpu_device, prepared):
     ff = BasedXLChainedFeedForward(proj, out, prepared=prepared).to(DEV)
     ff.geglu.weight, ff.geglu.bias = ff.geglu.weight.to(DEV), ff.geglu.bias.to(DEV)
     ff.linear.weight, ff.linear.bias = ff.linear.weight.to(DEV), ff.linear.bias.to(DEV)
-    x = torch.randn(2, 512, 640, device=DEV)
+    x = torch.randn(2, 2048, 640, device=DEV)
     y = ff(x)
-    assert ff.chained_calls == 1 and y.shape == (2, 512, 640)
+    assert ff.chained_calls == 1 and y.shape == (2, 2048, 640)
     want = ff.linear(ff.geglu(x))                        # the same layers one by one
     torch.testing.assert_close(y, want, rtol=0, atol=2e-4)
     xr = x.cpu().reshape(-1, 640)
@@ -318,6 +318,11 @@ def test_chained_feed_forward_module_and_its_fallback(gpu_device, prepared):
     y2 = ff(x[:, :100])
     assert ff.chained_calls == 1
     torch.testing.assert_close(y2, want[:, :100], rtol=0, atol=2e-4)
+    # 1024 rows make 64 large tiles for 256 CUs: the cost estimates prefer a smaller tile and a gate pass, so
+    # the block runs layer by layer although the chain would take the shape
+    y3 = ff(x[:, :512])
+    assert ff.chained_calls == 1
+    torch.testing.assert_close(y3, want[:, :512], rtol=0, atol=2e-4)
 
 
 @pytest.mark.gpu
