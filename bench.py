@@ -364,7 +364,8 @@ def bench_attn(dev, check=True):
                 "mfma_tflops": round(9 * flop / us_qkv * 1e-6, 1), "frac_of_mfma_peak": round(9 * flop / us_qkv * 1e-6 / PEAK_BF16_TFLOPS, 4),
                 "traffic": traffic_for("attn", "to_q/to_k/to_v grouped", k_qkv)[0]},
                {"launch": "to_out", "kernel": k_o, "launch_us": round(us_o, 2), "mfma_tflops": round(3 * flop / us_o * 1e-6, 1),
-                "frac_of_mfma_peak": round(3 * flop / us_o * 1e-6 / PEAK_BF16_TFLOPS, 4)}]}
+                "frac_of_mfma_peak": round(3 * flop / us_o * 1e-6 / PEAK_BF16_TFLOPS, 4),
+                "traffic": traffic_for("attn", "to_out", k_o)[0]}]}
     if check:
         exp = oc.fp64_matmul(x2_cpu, w_cpu[3])
         ek, eo = oc.error_metrics(outs[3].cpu(), exp), oc.error_metrics(oc.cascade_matmul_ref(x2_cpu, w_cpu[3]), exp)
