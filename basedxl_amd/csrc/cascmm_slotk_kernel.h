@@ -4,8 +4,8 @@
 // The right operand comes as MFMA operand slots (cascmm_prepare_weight: 16 bytes = 8 k of one column
 // of one term, [term][K/8][N]): a lane's operand is one 16-byte load and 32 consecutive lanes read 512
 // contiguous bytes, so B needs no transposition through LDS.  One workgroup computes a 64 x 160 tile of
-// C; its four waves split K: wave w takes the 16-k stages w, w + 4, w + 8, ... and owns the whole tile
-// (ten 32 x 32 accumulator blocks) over them.  Nothing is shared between waves until the end, so every
+// C; its four waves split K: wave w takes the 16-k stages w, w + 4, w + 8, ... (raw left operand: the pairs
+// of stages w, w + 4, ...) and owns the whole tile (ten 32 x 32 accumulator blocks) over them.  Nothing is shared between waves until the end, so every
 // wave streams its own operands, B straight into registers four stages deep, and the main loop has no
 // barrier.  A 2048 x 1280 result is 256 tiles, one per CU, whatever K is: no partial results through
 // memory, no second kernel.  At the end the four partial tiles meet in LDS: every wave owns two or three
@@ -16,14 +16,15 @@
 //   ARAW = 0: operand slots as well, [term][K/8][M] (written by the gated store of the preceding GEMM
 //     or by cascmm_prepare_left): loaded like B, straight into registers; no LDS access and no VALU
 //     work in the loop.  The order of k inside a 16-k stage is whatever the two slot buffers agree on.
-//   ARAW = 1: raw fp32 rows.  A stage's 64 rows x 64 bytes go to a private LDS ring of the wave without
-//     passing registers (four `buffer_load ... lds` of 1 KB: four consecutive lanes fetch the four
-//     16-byte chunks of a row, rotated by row / 4 so that fragment reads spread over all banks), six
-//     stages ahead; the fragments of the next stage are read and split in registers between the MFMAs
-//     of the current one.
+//   ARAW = 1: raw fp32 rows.  A pair of stages, 64 rows x 128 bytes (whole lines: with 64 bytes per row the
+//     L1 fetched every line of A twice), goes to a private LDS ring of the wave without passing registers
+//     (eight `buffer_load ... lds` of 1 KB, four per stage: eight consecutive lanes fetch the eight 16-byte
+//     chunks of a row, rotated by row / 2 so that fragment reads spread over all banks), six stages ahead;
+//     the fragments of the next stage are read and split in registers between the MFMAs of the current one.
 //
 // What bounds it: a workgroup pulls (64 + 160) x 4 bytes per k through its CU's vector memory path,
-// which for 256 CUs is 84 % of what the eight L2s can deliver while the MFMAs of that k take as long.
+// which for 256 CUs is 84 % of what the eight L2s can deliver while the MFMAs of that k take as long; with
+// both operands raw (cascmm_rawk_kernel below) the two splits fill the issue slots beside the MFMAs first.
 #pragma once
 #include <type_traits>
 
