@@ -12,8 +12,9 @@ namespace cascmm {
 // a wave writes 256-byte runs of 16 consecutive rows.
 __global__ __launch_bounds__(256) void prepare_left_kernel(const float* A, int M, int K, int64_t lda, u32x4* out) {
   const int kgroups = K >> 3;
-  const int kg = blockIdx.y * 4 + (threadIdx.x & 3);
-  const int m = blockIdx.x * 64 + (threadIdx.x >> 2);
+  const int row_blocks = (M + 63) / 64;   // a one-dimensional grid: row blocks fastest (the other grid dimensions end at 65535)
+  const int kg = (int)(blockIdx.x / row_blocks) * 4 + (threadIdx.x & 3);
+  const int m = (int)(blockIdx.x % row_blocks) * 64 + (threadIdx.x >> 2);
   if (m >= M || kg >= kgroups) return;
   const float* src = A + (int64_t)m * lda + 16 * (kg >> 1) + 4 * (kg & 1);
   const f32x4 x0 = *(const f32x4*)src, x1 = *(const f32x4*)(src + 8);
@@ -25,9 +26,11 @@ __global__ __launch_bounds__(256) void prepare_left_kernel(const float* A, int M
 }
 
 int launch_prepare_left(const float* A, int M, int K, int64_t lda, void* out, hipStream_t stream) {
-  const dim3 grid((unsigned)((M + 63) / 64), (unsigned)(((K >> 3) + 3) / 4));
-  return launch_kernel(prepare_left_kernel, grid, dim3(256), 0, stream, A, M, K, lda, (u32x4*)out) == hipSuccess ? CASCMM_OK
-                                                                                                                 : CASCMM_ERR_LAUNCH;
+  const int64_t blocks = (int64_t)((M + 63) / 64) * (((K >> 3) + 3) / 4);   // < 2^18: the caller keeps 4 M K below 2 GiB
+  if (blocks <= 0 || blocks > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  return launch_kernel(prepare_left_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, A, M, K, lda, (u32x4*)out) == hipSuccess
+             ? CASCMM_OK
+             : CASCMM_ERR_LAUNCH;
 }
 
 const void* slotk_kernel_handle(int araw) { return araw ? (const void*)cascmm_slotk_kernel<1> : (const void*)cascmm_slotk_kernel<0>; }
