@@ -185,10 +185,11 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
     w = {
         "tile": rn(640, 640) * 0.02, "ksplit": rn(5120, 1280) * 0.02, "skinny": rn(2048, 640) * 0.02,
         "h": (rn(640, 640) * 0.02).half(), "glu": rn(640, 1280) * 0.02, "fp8": rn(320, 640) * 0.02,
+        "kwave": rn(1280, 1280) * 0.02,     # with 2048 rows: one 64 x 160 tile per CU, K split over the waves of a workgroup
     }
     x = {"tile": rn(2048, 640), "ksplit": rn(1024, 5120), "skinny": rn(154, 2048), "h": rn(1024, 640).half(),
-         "glu": rn(512, 640), "fp8": rn(512, 320)}
-    pw, pg = PreparedWeight(w["tile"]), PreparedWeight(w["glu"], glu=True)
+         "glu": rn(512, 640), "fp8": rn(512, 320), "kwave": rn(2048, 1280)}
+    pw, pg, pk = PreparedWeight(w["tile"]), PreparedWeight(w["glu"], glu=True), PreparedWeight(w["kwave"])
     p8 = PreparedWeight(w["fp8"], lowp="fp8", terms=3)   # (holds the weight's kept scale exponent too)
 
     def run():
@@ -204,6 +205,8 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
             # the activation scale found inside the call (maxima, split, GEMM: all on the stream), weight raw / kept split
             cascaded_lowp_matmul(x["fp8"], w["fp8"], lowp="fp8", terms=3, b_exp=p8.exp),
             cascaded_lowp_matmul(x["fp8"], p8),
+            cascaded_lowp_matmul(x["kwave"], w["kwave"]),      # both operands raw
+            cascaded_lowp_matmul(x["kwave"], pk),              # raw rows through the LDS ring, weight as slots
         ]
 
     run()                                            # warm-up: workspaces exist before the capture
@@ -222,7 +225,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
         outs = run()
     grown = torch.cuda.memory_allocated() - before
     assert {k: v.data_ptr() for k, v in _workspaces.items()} == ws_before        # no workspace was created or replaced
-    # what the capture allocated: the ten results plus the grouped launches' other results and the
+    # what the capture allocated: the twelve results plus the grouped launches' other results and the
     # two-int exponent tensor, each rounded up to the allocator's 512-byte granule -- far below the
     # 21 MB K-split workspace a capture-time allocation would add
     results = sum(o.numel() * o.element_size() for o in outs)
