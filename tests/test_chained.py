@@ -326,6 +326,40 @@ def test_chained_feed_forward_module_and_its_fallback(gpu_device, prepared):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("form", ["raw x raw", "raw x slots", "slots x slots"])
+def test_non_finite_operands_poison_their_row_or_column_only_on_the_k_over_waves_kernels(gpu_device, form):
+    """As for the other kernels: a NaN or an infinity in A spoils exactly its row, one in B exactly its
+    column.  K = 96 leaves the fourth wave of a workgroup without a stage of its own: it multiplies the
+    problem's first columns of A (where the infinity sits) by zeros, which must not reach any other row."""
+    from basedxl_amd import ChainedWeight, LeftSlots, PreparedWeight, cascaded_lowp_matmul, cascaded_lowp_matmul_chained
+    names = _lib.variant_names()
+    g = torch.Generator().manual_seed(23)
+    a = torch.randn(100, 96, generator=g)
+    b = torch.randn(96, 84, generator=g) * 0.02
+
+    def run(a_, b_):
+        ad, bd = a_.to(DEV), b_.to(DEV)
+        if form == "raw x raw":
+            return cascaded_lowp_matmul(ad, bd, variant=names.index("k64x160x16_wk4_bf16x2_tri")).cpu()
+        if form == "raw x slots":
+            return cascaded_lowp_matmul(ad, PreparedWeight(bd, lowp="bf16", terms=2), variant=names.index("k64x160x16_wk4_bf16x2_tri_bpre")).cpu()
+        return cascaded_lowp_matmul_chained(LeftSlots.from_tensor(ad), ChainedWeight(bd)).cpu()
+
+    clean = run(a, b)
+    a2, b2 = a.clone(), b.clone()
+    a2[5, 40] = float("nan")
+    a2[70, 3] = float("inf")
+    b2[77, 9] = -float("inf")
+    got = run(a2, b2)
+    want = oc.cascade_matmul_ref(a2, b2, "bf16", 2, "tri")
+    bad = torch.zeros(100, 84, dtype=torch.bool)
+    bad[5, :] = bad[70, :] = True
+    bad[:, 9] = True
+    assert torch.isnan(got[bad]).all() and torch.isnan(want[bad]).all()
+    assert torch.equal(got[~bad], clean[~bad])
+
+
+@pytest.mark.gpu
 def test_chain_replays_from_a_captured_graph(gpu_device):
     from basedxl_amd import ChainedWeight, LeftSlots, cascaded_lowp_matmul_chained, cascaded_lowp_matmul_glu_chained
     g = torch.Generator(device=DEV).manual_seed(17)
