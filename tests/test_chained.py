@@ -357,6 +357,18 @@ def test_non_finite_operands_poison_their_row_or_column_only_on_the_k_over_waves
     bad[:, 9] = True
     assert torch.isnan(got[bad]).all() and torch.isnan(want[bad]).all()
     assert torch.equal(got[~bad], clean[~bad])
+    # what lies between the rows of a strided left operand is never multiplied, not even by zeros
+    padded = torch.full((100, 104), float("nan"))
+    padded[:, :96] = a
+    pd = padded.to(DEV)[:, :96]
+    bd = b.to(DEV)
+    if form == "raw x raw":
+        again = cascaded_lowp_matmul(pd, bd, variant=names.index("k64x160x16_wk4_bf16x2_tri"))
+    elif form == "raw x slots":
+        again = cascaded_lowp_matmul(pd, PreparedWeight(bd, lowp="bf16", terms=2), variant=names.index("k64x160x16_wk4_bf16x2_tri_bpre"))
+    else:
+        again = cascaded_lowp_matmul_chained(LeftSlots.from_tensor(pd), ChainedWeight(bd))
+    assert torch.equal(again.cpu(), clean)
 
 
 @pytest.mark.gpu
