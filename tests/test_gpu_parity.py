@@ -807,6 +807,35 @@ def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
     assert ran >= (4 if K % 64 == 0 else 2)
 
 
+@pytest.mark.parametrize("shape", [(256, 192, 320), (154, 256, 64), (96, 128, 160)])
+def test_padding_between_the_rows_of_a_strided_left_operand_is_never_read(gpu_device, shape):
+    """Every kernel that takes fp32 tensors, forced by name: with NaNs in the gap between the rows of A
+    (lda = K + 8) the result keeps the bits it has on a contiguous A.  A kernel that fetched past K --
+    a stage too many, a whole cache line where half of it belongs to the row -- would turn its rows into NaNs."""
+    M, K, N = shape
+    a, b = oc.make_operands(M, K, N, seed=77, w_std=0.02)
+    ad, bd = _gpu(a), _gpu(b)
+    padded = torch.full((M, K + 8), float("nan"))
+    padded[:, :K] = a
+    pd = _gpu(padded)[:, :K]
+    ran = 0
+    for vi, name in enumerate(_lib.variant_names()):
+        if "_io" in name or "_bpre" in name:
+            continue
+        fmt, terms = _fmt_of(name)
+        kw = dict(lowp=fmt, terms=terms, products="full" if "_full" in name else "tri", variant=vi)
+        try:
+            want = cascaded_lowp_matmul(ad, bd, **kw)
+        except _lib.CascmmError as e:
+            assert e.status in (-4, -8), (name, e)       # this kernel does not take the shape
+            continue
+        _say("padded rows", shape, name)
+        got = cascaded_lowp_matmul(pd, bd, **kw)
+        assert torch.isfinite(want).all() and torch.equal(got, want), (name, shape)
+        ran += 1
+    assert ran >= 8
+
+
 def test_prepared_weight_equals_raw_weight_bit_for_bit(gpu_device):
     """Same tile, same consumer layout: the prepared path does the same split and accumulates
     in the same order as the on-the-fly path, so the bits agree (the large-tile kernel, which takes
