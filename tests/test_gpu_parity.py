@@ -808,7 +808,7 @@ def test_prepared_weights_integer_exact_on_every_variant(gpu_device, shape):
 
 
 @pytest.mark.parametrize("shape", [(256, 192, 320), (154, 256, 64), (96, 128, 160)])
-def test_padding_between_the_rows_of_a_strided_left_operand_is_never_read(gpu_device, shape):
+def test_gaps_between_rows_are_neither_read_nor_written(gpu_device, shape):
     """Every kernel that takes fp32 tensors, forced by name: with NaNs in the gap between the rows of A
     (lda = K + 8) the result keeps the bits it has on a contiguous A.  A kernel that fetched past K --
     a stage too many, a whole cache line where half of it belongs to the row -- would turn its rows into NaNs."""
@@ -832,6 +832,10 @@ def test_padding_between_the_rows_of_a_strided_left_operand_is_never_read(gpu_de
         _say("padded rows", shape, name)
         got = cascaded_lowp_matmul(pd, bd, **kw)
         assert torch.isfinite(want).all() and torch.equal(got, want), (name, shape)
+        # ... and a result with gaps between its rows (ldc = N + 3: no 16-byte stores) is written inside its rows only
+        frame = torch.full((M + 1, N + 3), -77.0, device=ad.device)
+        cascaded_lowp_matmul(pd, bd, out=frame[:M, :N], **kw)
+        assert torch.equal(frame[:M, :N], want) and bool((frame[:M, N:] == -77.0).all()) and bool((frame[M] == -77.0).all()), (name, shape)
         ran += 1
     assert ran >= 8
 
