@@ -819,10 +819,23 @@ def test_gaps_between_rows_are_neither_read_nor_written(gpu_device, shape):
     padded[:, :K] = a
     pd = _gpu(padded)[:, :K]
     ran = 0
+    prepared = {}
     for vi, name in enumerate(_lib.variant_names()):
-        if "_io" in name or "_bpre" in name:
+        if "_io" in name:
             continue
         fmt, terms = _fmt_of(name)
+        if "_bpre" in name:        # weight kept split: the same check on the left operand (the result must be contiguous there)
+            if (fmt, terms) not in prepared:
+                prepared[(fmt, terms)] = PreparedWeight(bd, lowp=fmt, terms=terms)
+            try:
+                want = cascaded_lowp_matmul(ad, prepared[(fmt, terms)], variant=vi)
+            except _lib.CascmmError as e:
+                assert e.status in (-4, -8), (name, e)
+                continue
+            _say("padded rows", shape, name)
+            assert torch.isfinite(want).all() and torch.equal(cascaded_lowp_matmul(pd, prepared[(fmt, terms)], variant=vi), want), (name, shape)
+            ran += 1
+            continue
         kw = dict(lowp=fmt, terms=terms, products="full" if "_full" in name else "tri", variant=vi)
         try:
             want = cascaded_lowp_matmul(ad, bd, **kw)
