@@ -162,6 +162,8 @@ static const TunedCost kTuned[] = {
 };
 
 constexpr int kMaxTileSplits = 4;
+// the fp8-rate kernel with K over the waves: us per 64-k stage of a wave, and per round of tiles
+constexpr double kF8WKStageUs = 2.25, kF8WKFixedUs = 6.0;   // (fit: 2048 x {1280, 5120} x 1280, 4096 x {640, 2560} x 640)
 
 static const std::vector<VariantInfo>& variant_info() {
   static const std::vector<VariantInfo> info = [] {
@@ -233,8 +235,11 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     const int sp = f8k64_splits(q.M, q.N, q.K, v.BM);
     const double items = tiles * sp;
     const double rounds_ = items <= kNumCUs ? 1.0 : (double)(int64_t)(items / kNumCUs) + ((int64_t)items % kNumCUs ? 0.8 : 0.0);
-    double us = rounds_ * ((double)(q.K / 64 / sp) * f8k64_stage_us(v.BM) + (v.BM == 256 ? 6.0 : 4.0)) + 6.0 +
-                (double)q.M * q.K * 7.0 / 4.0e6;
+    // (the 64-row tile splits K over the four waves of its workgroup: a quarter of the stages per wave, in pairs,
+    // and rounds of one tile per CU that do not overlap)
+    const double gemm_us = v.BM == F8WK::BM ? rounds_ * ((double)((q.K / 64 + 7) / 8 * 2) * kF8WKStageUs + kF8WKFixedUs)
+                                            : rounds_ * ((double)(q.K / 64 / sp) * f8k64_stage_us(v.BM) + (v.BM == 256 ? 6.0 : 4.0));
+    double us = gemm_us + 6.0 + (double)q.M * q.K * 7.0 / 4.0e6;
     if (!q.bpre) us += 3.0 + (double)q.K * q.N * 7.0 / 4.0e6;
     if (sp > 1) us += 3.0 + (double)(sp + 1) * q.M * q.N * 4.0 / 4.0e6;
     return us;

@@ -12,6 +12,8 @@ static const VariantDesc kTable[] = {
     CASCMM_F8K64_VARIANT("t256x160x64_f8k64_fp8x3_tri_bpre", true, 2),
     CASCMM_F8K64_VARIANT("t128x160x64_f8k64_fp8x3_tri", false, 1),
     CASCMM_F8K64_VARIANT("t128x160x64_f8k64_fp8x3_tri_bpre", true, 1),
+    CASCMM_F8K64_VARIANT("k64x160x64_f8k64wk4_fp8x3_tri", false, 0),
+    CASCMM_F8K64_VARIANT("k64x160x64_f8k64wk4_fp8x3_tri_bpre", true, 0),
     // three terms (12 significand bits), six products.  name, BM, BN, BK, WM, WN, WK, DEPTH
     CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp8x3_tri", 128, 128, 32, 4, 2, 1, 2, F32, F8, 3, false, true),
     CASCMM_TILE_VARIANT("t64x64x64_w2x2x1_d2_fp8x3_tri", 64, 64, 64, 2, 2, 1, 2, F32, F8, 3, false, true),

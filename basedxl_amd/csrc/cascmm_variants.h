@@ -7,6 +7,7 @@
 #include "cascmm_bdirect_kernel.h"
 #include "cascmm_w512_kernel.h"
 #include "cascmm_f8k64_kernel.h"
+#include "cascmm_f8wk_kernel.h"
 #include "cascmm_wavek_kernel.h"
 
 namespace cascmm {
@@ -236,7 +237,12 @@ int launch_wavek(const GroupParams& p, hipStream_t stream) {
 // the split count that minimises stages-per-workgroup x the stage time + the round trip of the
 // partial results at ~4 TB/s
 inline double f8k64_stage_us(int bm) { return bm == 256 ? 2.1 : 1.15; }
+// the tile of a variant: MT = 2, 1: the LDS-tiled kernel's 256 / 128 rows; MT = 0: the 64 x 160 tile whose K is split over
+// the waves of a workgroup (cascmm_f8wk_kernel.h: one launch, never a K split over workgroups)
+template <int MT> struct F8Tile { typedef F8K64T<MT> T; };
+template <> struct F8Tile<0> { typedef F8WK T; };
 inline int f8k64_splits(int64_t M, int64_t N, int64_t K, int bm) {
+  if (bm == F8WK::BM) return 1;
   const int64_t tiles = ((M + bm - 1) / bm) * ((N + F8K64::BN - 1) / F8K64::BN);
   const int64_t steps = K / F8K64::BK;
   int best = 1;
@@ -266,14 +272,14 @@ inline size_t f8k64_workspace_bytes(int64_t M, int64_t N, int64_t K, bool bpre, 
 // the fp8-rate kernel: split A (and B) into operand slots, then the GEMM on the slots
 template <bool BPRE, int MT>
 int launch_f8k64(const GroupParams& p, hipStream_t stream) {
-  typedef F8K64T<MT> T;
-  if (p.kernel_out) { *p.kernel_out = (const void*)cascmm_f8k64_kernel<MT>; return CASCMM_OK; }
+  typedef typename F8Tile<MT>::T T;
+  void (*kfn)(const F8K64Params) = MT == 0 ? cascmm_f8wk_kernel<0> : cascmm_f8k64_kernel<(MT == 0 ? 1 : MT)>;
+  if (p.kernel_out) { *p.kernel_out = (const void*)kfn; return CASCMM_OK; }
   if (p.count != 1 || p.glu || p.k_splits > 1 || p.K % T::BK != 0 || p.K == 0) return CASCMM_ERR_BAD_VARIANT;
   const size_t need = f8k64_workspace_bytes(p.M, p.N, p.K, BPRE, T::BM);
   if (!p.workspace || p.workspace_bytes < need) return CASCMM_ERR_WORKSPACE;
   if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
   if (f8k64_slot_bytes(p.M, p.K) > 0x7FFFFFFF || f8k64_slot_bytes(p.N, p.K) > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
-  auto kfn = cascmm_f8k64_kernel<MT>;
   static LdsFlags lds_set;
   if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
   u32x4* a_slots = (u32x4*)p.workspace;
@@ -331,8 +337,8 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
 }
 
 #define CASCMM_F8K64_VARIANT(NAME, BPRE, MT)                                                                                  \
-  {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8K64T<MT>::BM, F8K64T<MT>::BN, F8K64T<MT>::BK, F8K64T<MT>::NT, \
-   F8K64T<MT>::LDS_BYTES, true, false, &launch_f8k64<BPRE, MT>, BPRE}
+  {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8Tile<MT>::T::BM, F8Tile<MT>::T::BN, F8Tile<MT>::T::BK, \
+   F8Tile<MT>::T::NT, F8Tile<MT>::T::LDS_BYTES, true, false, &launch_f8k64<BPRE, MT>, BPRE}
 
 #define CASCMM_WAVEK_VARIANT(NAME, NB)                                                                                \
   {NAME, KIND_WAVEK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, WaveK<NB>::BM, WaveK<NB>::BN, WaveK<NB>::BK, WaveK<NB>::NT, \
