@@ -190,6 +190,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
     x = {"tile": rn(2048, 640), "ksplit": rn(1024, 5120), "skinny": rn(154, 2048), "h": rn(1024, 640).half(),
          "glu": rn(512, 640), "fp8": rn(512, 320), "kwave": rn(2048, 1280)}
     pw, pg, pk = PreparedWeight(w["tile"]), PreparedWeight(w["glu"], glu=True), PreparedWeight(w["kwave"])
+    pk8 = PreparedWeight(w["kwave"], lowp="fp8", terms=3)
     p8 = PreparedWeight(w["fp8"], lowp="fp8", terms=3)   # (holds the weight's kept scale exponent too)
 
     def run():
@@ -207,6 +208,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
             cascaded_lowp_matmul(x["fp8"], p8),
             cascaded_lowp_matmul(x["kwave"], w["kwave"]),      # both operands raw
             cascaded_lowp_matmul(x["kwave"], pk),              # raw rows through the LDS ring, weight as slots
+            cascaded_lowp_matmul(x["kwave"], pk8),             # three fp8 terms: scale search, split of the rows, K over the waves
         ]
 
     run()                                            # warm-up: workspaces exist before the capture
@@ -225,7 +227,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
         outs = run()
     grown = torch.cuda.memory_allocated() - before
     assert {k: v.data_ptr() for k, v in _workspaces.items()} == ws_before        # no workspace was created or replaced
-    # what the capture allocated: the twelve results plus the grouped launches' other results and the
+    # what the capture allocated: the thirteen results plus the grouped launches' other results and the
     # two-int exponent tensor, each rounded up to the allocator's 512-byte granule -- far below the
     # 21 MB K-split workspace a capture-time allocation would add
     results = sum(o.numel() * o.element_size() for o in outs)
