@@ -101,6 +101,10 @@ static bool variant_matches(const VariantDesc& v, const Problem& q, bool fast) {
   if (v.kind == KIND_F8K64 && (q.products != CASCMM_PROD_TRI || q.K % v.BK != 0 || q.K == 0 || q.glu ||
                                f8k64_slot_bytes(q.M, q.K) > INT32_MAX || f8k64_slot_bytes(q.N, q.K) > INT32_MAX))
     return false;
+  if (v.kind == KIND_F16K && (q.products != CASCMM_PROD_TRI || q.K % v.BK != 0 || q.K == 0 || q.glu || q.bpre ||
+                              (v.BM == F16K::BM && q.K > F16K::MAX_K) || q.K * q.ldb * 4 > INT32_MAX ||
+                              f16k_slot_bytes(q.M, q.K) > INT32_MAX || f16k_slot_bytes(q.N, q.K) > INT32_MAX))
+    return false;
   if (v.bpre && v.kind != KIND_F8K64 && prepared_as_k16_slots(q.K, q.fmt, q.terms, q.glu)) return false;   // other layout
   if (v.kind == KIND_W512 && (q.M % v.BM != 0 || q.N % v.BN != 0 || q.M * q.lda * 4 > INT32_MAX ||
                               (!q.bpre && q.K * q.ldb * 4 > INT32_MAX) || q.ldc * (int64_t)(v.BM * 4) > INT32_MAX))
@@ -244,6 +248,14 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     if (sp > 1) us += 3.0 + (double)(sp + 1) * q.M * q.N * 4.0 / 4.0e6;
     return us;
   }
+  if (v.kind == KIND_F16K) {
+    // stages of 32 k that take what the fp8-rate kernels' stages of 64 k take (the same bytes, the same MFMA
+    // cycles), and the passes around the GEMM: two scale searches, two splits (4 bytes read, 6 written per element)
+    const double rounds_ = tiles <= kNumCUs ? 1.0 : (double)(int64_t)(tiles / kNumCUs) + ((int64_t)tiles % kNumCUs ? 0.8 : 0.0);
+    const double gemm_us = v.BM == F16WK::BM ? rounds_ * ((double)((q.K / 32 + 7) / 8 * 2) * kF8WKStageUs + kF8WKFixedUs)
+                                             : rounds_ * ((double)(q.K / 32) * f8k64_stage_us(256) + 6.0);
+    return gemm_us + 12.0 + ((double)q.M * q.K + (double)q.K * q.N) * 14.0 / 4.0e6;
+  }
   if (info.tuned) {
     const TunedCost& t = *info.tuned;
     const double tail = full == 0 ? t.tail_first : t.tail_later;
@@ -370,6 +382,7 @@ static int select_variant_uncached(const Problem& q, bool fast, int count, size_
         skinny_workspace_bytes(q.M, q.N, q.K, t[i].BM, t[i].BN, t[i].BK) > ws_bytes)
       continue;
     if (t[i].kind == KIND_F8K64 && f8k64_workspace_bytes(q.M, q.N, q.K, q.bpre, t[i].BM) > ws_bytes) continue;
+    if (t[i].kind == KIND_F16K && f16k_workspace_bytes(q.M, q.N, q.K) > ws_bytes) continue;
     int sp = 1;
     const double c = variant_cost(i, q, count, ws_bytes, &sp);
     if (best < 0 || c < best_cost) {
@@ -711,7 +724,8 @@ int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
     int splits = 1;
     int v = select_variant(q, fast_ok(q, A, B), 1, (size_t)-1, &splits);
     if (v < 0) return v;
-    if (table()[v].kind == KIND_F8K64 && f8k64_workspace_bytes(M, N, K, false, table()[v].BM) > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) {
+    if ((table()[v].kind == KIND_F8K64 && f8k64_workspace_bytes(M, N, K, false, table()[v].BM) > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) ||
+        (table()[v].kind == KIND_F16K && f16k_workspace_bytes(M, N, K) > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES)) {
       // the fp8-rate kernel is a choice, not a need: without room for its operand slots the choice is
       // made among the kernels that split inside the GEMM
       v = select_variant(q, fast_ok(q, A, B), 1, (size_t)CASCMM_NOALLOC_SCRATCH_BYTES, &splits);
@@ -720,6 +734,7 @@ int cascmm_gemm_noalloc(const void* A, const void* B, void* C, const void* bias,
     const VariantDesc& d = table()[v];
     if (d.kind == KIND_SPLITK) need = skinny_workspace_bytes(M, N, K, d.BM, d.BN, d.BK);
     else if (d.kind == KIND_F8K64) need = f8k64_workspace_bytes(M, N, K, false, d.BM);
+    else if (d.kind == KIND_F16K) need = f16k_workspace_bytes(M, N, K);
     else if (splits > 1) need = (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
   }
   if (need > (size_t)CASCMM_NOALLOC_SCRATCH_BYTES) return CASCMM_ERR_SCRATCH_LIMIT;
@@ -875,6 +890,12 @@ size_t cascmm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype, int fm
   for (const auto& v : table()) {
     if (v.kind != KIND_F8K64 || v.bpre || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
     const size_t n = f8k64_workspace_bytes(M, N, K, false, v.BM);
+    need = n > need ? n : need;
+  }
+  // three fp16 terms on operand slots: the slots of A and B
+  for (const auto& v : table()) {
+    if (v.kind != KIND_F16K || !variant_matches(v, q, fast_ok(q, nullptr, nullptr))) continue;
+    const size_t n = f16k_workspace_bytes(M, N, K);
     need = n > need ? n : need;
   }
   // 16-bit tensors as one term of their own format: room for B re-laid as operand slots

@@ -228,13 +228,15 @@ template <int FMT, int TERMS, bool FULL> struct AccClasses {
 // fp8 tensor scale: max|x| as a bit pattern (non-negative floats order like their bit patterns)
 // ---------------------------------------------------------------------------------------
 // bit pattern of max|x| over the elements this thread visits, reduced over its wave
-template <int IODT>
-__device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64_t cols, int64_t ld) {
+// (FINITE_ONLY: infinities and NaNs are passed over, so that the scale serves the finite elements)
+template <int IODT, bool FINITE_ONLY = false>
+__device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64_t cols, int64_t ld, unsigned block, unsigned blocks) {
   typedef typename IoType<IODT>::T T;
   const T* src = (const T*)x;
   unsigned best = 0;
   auto fold = [&](float v) {
-    const unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7FFFFFFFu;
+    unsigned bits = __builtin_bit_cast(unsigned, v) & 0x7FFFFFFFu;
+    if (FINITE_ONLY && bits >= 0x7F800000u) bits = 0;
     best = bits > best ? bits : best;
   };
   if (ld == cols) {
@@ -242,8 +244,8 @@ __device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64
     const int64_t total = rows * cols;
     if (IODT == CASCMM_DT_F32 && ((uintptr_t)x % 16) == 0) {
       const int64_t quads = total / 4;
-      const int64_t step = (int64_t)gridDim.x * blockDim.x;
-      int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+      const int64_t step = (int64_t)blocks * blockDim.x;
+      int64_t i = (int64_t)block * blockDim.x + threadIdx.x;
       // four independent loads in flight per thread
       for (; i + 3 * step < quads; i += 4 * step) {
         f32x4 v[4];
@@ -256,13 +258,13 @@ __device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64
         const f32x4 v = ((const f32x4*)x)[i];
         fold(v[0]); fold(v[1]); fold(v[2]); fold(v[3]);
       }
-      if (blockIdx.x == 0 && threadIdx.x < total - quads * 4) fold(IoType<IODT>::load(src + quads * 4 + threadIdx.x));
+      if (block == 0 && threadIdx.x < total - quads * 4) fold(IoType<IODT>::load(src + quads * 4 + threadIdx.x));
     } else {
-      for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x)
+      for (int64_t i = (int64_t)block * blockDim.x + threadIdx.x; i < total; i += (int64_t)blocks * blockDim.x)
         fold(IoType<IODT>::load(src + i));
     }
   } else {
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x)
+    for (int64_t r = block; r < rows; r += blocks)
       for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) fold(IoType<IODT>::load(src + r * ld + c));
   }
 #pragma unroll
@@ -271,6 +273,11 @@ __device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64
     best = other > best ? other : best;
   }
   return best;
+}
+
+template <int IODT, bool FINITE_ONLY = false>
+__device__ __forceinline__ unsigned amax_scan(const void* x, int64_t rows, int64_t cols, int64_t ld) {
+  return amax_scan<IODT, FINITE_ONLY>(x, rows, cols, ld, blockIdx.x, gridDim.x);
 }
 
 // the exponent e with max|x| * 2^e in (224, 448], from the bit pattern of max|x|

@@ -17,6 +17,9 @@ static const VariantDesc kTable[] = {
     CASCMM_TILE_VARIANT("t128x128x32_w4x2x1_d2_fp16x2_full", 128, 128, 32, 4, 2, 1, 2, F32, FP, 2, true, true),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp16x2_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, FP, 2, true, false),
     CASCMM_TILE_VARIANT("t64x64x32_w2x2x1_d1_fp16x3_full_generic", 64, 64, 32, 2, 2, 1, 1, F32, FP, 3, true, false),
+    // both operands split into pre-scaled operand slots first (cascmm_f16k_kernel.h)
+    CASCMM_F16K_VARIANT("t256x160x32_f16k_fp16x3_tri", false),
+    CASCMM_F16K_VARIANT("k64x160x32_f16wk4_fp16x3_tri", true),
 };
 
 const VariantDesc* variants_fp16(int* n) {

@@ -7,16 +7,17 @@
 #include "cascmm_bdirect_kernel.h"
 #include "cascmm_w512_kernel.h"
 #include "cascmm_f8k64_kernel.h"
-#include "cascmm_f8wk_kernel.h"
+#include "cascmm_f16k_kernel.h"
 #include "cascmm_wavek_kernel.h"
 
 namespace cascmm {
 
 // KIND_W512: the large-tile kernel (whole 256 x 320 tiles only, one problem per launch)
 // KIND_F8K64: three fp8 terms on the fp8-rate MFMA; splits its operands into the workspace first
+// KIND_F16K: three fp16 terms on operand slots; finds both scales and splits its operands into the workspace first
 // KIND_WAVEK: skinny problems in one launch, K split over the waves of a workgroup (no workspace)
 // KIND_SLOTK: prepared right operand, K split over the waves of a workgroup (64 x 160 tiles, one problem per launch)
-enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3, KIND_WAVEK = 4, KIND_SLOTK = 5 };
+enum VariantKind { KIND_TILE = 0, KIND_SPLITK = 1, KIND_W512 = 2, KIND_F8K64 = 3, KIND_WAVEK = 4, KIND_SLOTK = 5, KIND_F16K = 6 };
 constexpr int kNumCUs = 256;  // MI355X: what the cost model's constants were measured on
 constexpr int kMaxDevices = 64;
 
@@ -335,6 +336,64 @@ int launch_f8k64(const GroupParams& p, hipStream_t stream) {
   }
   return CASCMM_OK;
 }
+
+// Workspace of the three-term fp16 kernels on operand slots: the slots of A and of B (each rounded up to 256 bytes),
+// the per-workgroup maxima of the two scale searches, the two exponents
+inline size_t f16k_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  return f8k64_up(f16k_slot_bytes(M, K)) + f8k64_up(f16k_slot_bytes(N, K)) + 2 * kF8K64AmaxGroups * sizeof(unsigned) + 256;
+}
+
+// the three-term fp16 kernels on operand slots: find both scales, split A and B into slots, then the GEMM on the slots
+// (WK: the 64 x 160 tile with K over the waves of a workgroup; otherwise the 256 x 160 tile staged through LDS)
+template <bool WK>
+int launch_f16k(const GroupParams& p, hipStream_t stream) {
+  typedef typename std::conditional<WK, F16WK, F16K>::type T;
+  void (*kfn)(const F8K64Params) = WK ? cascmm_f16wk_kernel<0> : cascmm_f16k_kernel<0>;
+  if (p.kernel_out) { *p.kernel_out = (const void*)kfn; return CASCMM_OK; }
+  if (p.count != 1 || p.glu || p.k_splits > 1 || p.K % T::BK != 0 || p.K == 0 || (!WK && p.K > F16K::MAX_K)) return CASCMM_ERR_BAD_VARIANT;
+  const size_t need = f16k_workspace_bytes(p.M, p.N, p.K);
+  if (!p.workspace || p.workspace_bytes < need) return CASCMM_ERR_WORKSPACE;
+  if ((uintptr_t)p.workspace % 16 != 0) return CASCMM_ERR_ALIGNMENT;
+  if (f16k_slot_bytes(p.M, p.K) > 0x7FFFFFFF || f16k_slot_bytes(p.N, p.K) > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
+  char* ws = (char*)p.workspace;
+  u32x4* a_slots = (u32x4*)ws;
+  ws += f8k64_up(f16k_slot_bytes(p.M, p.K));
+  u32x4* b_slots = (u32x4*)ws;
+  ws += f8k64_up(f16k_slot_bytes(p.N, p.K));
+  unsigned* amax_a = (unsigned*)ws;
+  unsigned* amax_b = amax_a + kF8K64AmaxGroups;
+  int32_t* exps = (int32_t*)(amax_b + kF8K64AmaxGroups);
+  const int n_a = (int)std::max<int64_t>(1, std::min<int64_t>(((int64_t)p.M * p.K + 8191) / 8192, kF8K64AmaxGroups));
+  const int n_b = (int)std::max<int64_t>(1, std::min<int64_t>(((int64_t)p.K * p.N + 8191) / 8192, kF8K64AmaxGroups));
+  if (launch_kernel(f16k_amax_kernel<0>, dim3((unsigned)(n_a + n_b)), dim3(1024), 0, stream, (const float*)p.A[0], (int64_t)p.M,
+                    (int64_t)p.K, p.lda, n_a, (const float*)p.B[0], (int64_t)p.N, p.ldb, amax_a, amax_b) != hipSuccess)
+    return CASCMM_ERR_LAUNCH;
+  const int kus = p.K >> 3;
+  const int a_blocks = ((p.M + 63) / 64) * ((kus + 3) / 4);
+  const int64_t b_blocks = ((int64_t)kus * p.N + 255) / 256;
+  if (launch_kernel(f16k_split_kernel<0>, dim3((unsigned)(a_blocks + b_blocks)), dim3(256), 0, stream, (const float*)p.A[0], p.M, p.K,
+                    p.lda, a_slots, (const unsigned*)amax_a, n_a, a_blocks, (const float*)p.B[0], p.N, p.ldb, b_slots,
+                    (const unsigned*)amax_b, n_b, exps) != hipSuccess)
+    return CASCMM_ERR_LAUNCH;
+  F8K64Params q;
+  q.a_slots = a_slots; q.b_slots = b_slots; q.C = (float*)p.C[0]; q.bias = (const float*)p.bias[0];
+  q.tensor_exps = exps;
+  q.M = p.M; q.N = p.N; q.K = p.K; q.ldc = p.ldc;
+  q.tiles_m = (p.M + T::BM - 1) / T::BM; q.tiles_n = (p.N + T::BN - 1) / T::BN;
+  q.k_splits = 1;
+  q.partials = nullptr;
+  const unsigned grid = (unsigned)(q.tiles_m * q.tiles_n);
+  if (launch_kernel(kfn, dim3(grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q) != hipSuccess) return CASCMM_ERR_LAUNCH;
+  return CASCMM_OK;
+}
+
+#define CASCMM_F16K_VARIANT(NAME, WK)                                                                                      \
+  {NAME, KIND_F16K, CASCMM_DT_F32, CASCMM_FMT_FP16, 3, false, std::conditional<WK, F16WK, F16K>::type::BM,              \
+   std::conditional<WK, F16WK, F16K>::type::BN, std::conditional<WK, F16WK, F16K>::type::BK,                           \
+   std::conditional<WK, F16WK, F16K>::type::NT, std::conditional<WK, F16WK, F16K>::type::LDS_BYTES, true, false,       \
+   &launch_f16k<WK>, false}
 
 #define CASCMM_F8K64_VARIANT(NAME, BPRE, MT)                                                                                  \
   {NAME, KIND_F8K64, CASCMM_DT_F32, CASCMM_FMT_FP8, 3, false, F8Tile<MT>::T::BM, F8Tile<MT>::T::BN, F8Tile<MT>::T::BK, \

@@ -133,6 +133,12 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
     # ... and where 64 x 160 tiles make about one per CU, the kernel that splits K over the waves of a workgroup
     for M, K, N in [(2048, 1280, 1280), (2048, 5120, 1280), (4096, 640, 640), (4096, 2560, 640)]:
         assert pick8(M, K, N) == "k64x160x64_f8k64wk4_fp8x3_tri_bpre", (M, K, N)
+    # three fp16 terms (cfg3 names them): both operands split into pre-scaled slots first; the 256 x 160 tile where
+    # the tiles fill the chip several times over, K over the waves of a workgroup where there is about one tile per CU
+    pick16 = lambda M, K, N: names[l.cascmm_select_variant(M, N, K, K, N, N, 0, 1, 3, 0) & 0xFFFF]
+    assert pick16(2048, 1280, 10240) == "t256x160x32_f16k_fp16x3_tri"
+    assert pick16(2048, 5120, 1280) == "k64x160x32_f16wk4_fp16x3_tri" and pick16(2048, 1280, 1280) == "k64x160x32_f16wk4_fp16x3_tri"
+    assert "f16" not in pick16(128, 128, 128).split("_")[1]   # a small problem is not worth the passes
     pickp = lambda M, K, N: names[l.cascmm_select_variant_prepared(1, M, N, K, K, N, 0, 0, 2, 0) & 0xFFFF]
     assert pickp(2048, 1280, 10240) == "t256x320x32_w512_bf16x2_tri_bpre"
     assert pickp(2048, 5120, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre" and pickp(2048, 1280, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre"

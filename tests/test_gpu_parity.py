@@ -477,6 +477,56 @@ def test_ffn_shape_at_full_size_meets_the_bound(gpu_device, fmt, terms):
     assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
 
 
+F16_SLOT_VARIANTS = ("t256x160x32_f16k_fp16x3_tri", "k64x160x32_f16wk4_fp16x3_tri")
+
+
+@pytest.mark.parametrize("name", F16_SLOT_VARIANTS)
+@pytest.mark.parametrize("shape", [(1024, 640, 640), (300, 1280, 200), (2048, 1280, 1280), (512, 5120, 320)])
+def test_fp16_slot_kernels_meet_the_bound(gpu_device, name, shape):
+    """The three-term fp16 kernels that split both operands into pre-scaled slots (their terms carry a tensor scale
+    and the factors 2^11, 1, 2^-11, which the oracle's terms do not): the same bound against the oracle's cascade,
+    on whole and ragged tiles and at the deepest K each is offered for."""
+    M, K, N = shape
+    if name.startswith("t256") and K > 1536:
+        pytest.skip("the LDS-tiled kernel is offered up to K = 1536")
+    _say("accuracy", name, shape)
+    a, b = oc.make_operands(M, K, N, seed=31, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "fp16", 3, "tri"), exp)
+    got = oc.error_metrics(cascaded_lowp_matmul(_gpu(a), _gpu(b), lowp="fp16", terms=3, variant=_lib.variant_names().index(name)).cpu(), exp)
+    _say(f"   ratios: rel_fro x{got['rel_fro'] / ref['rel_fro']:.3f} max_abs x{got['max_abs'] / ref['max_abs']:.3f}")
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"], (got, ref)
+
+
+@pytest.mark.parametrize("name", F16_SLOT_VARIANTS)
+def test_fp16_slot_kernels_scale_with_their_operands(gpu_device, name):
+    """Scaling an operand by a power of two moves its tensor scale and nothing else: the result is the scaled result
+    bit for bit, for tensors far outside fp16's own range as well; and a non-finite element spoils its own row (or
+    column) only, the other results staying what they were."""
+    v = _lib.variant_names().index(name)
+    g = torch.Generator(device="cuda:0").manual_seed(5)
+    a = torch.randn(320, 256, device="cuda:0", generator=g)
+    b = torch.randn(256, 200, device="cuda:0", generator=g) * 0.02
+    run = lambda x, y: cascaded_lowp_matmul(x, y, lowp="fp16", terms=3, variant=v)
+    c = run(a, b)
+    for ka, kb in [(10, 0), (-30, 0), (0, 40), (25, -25), (40, 30)]:
+        _say("scaled operands", name, ka, kb)
+        assert torch.equal(run(a * 2.0 ** ka, b * 2.0 ** kb), c * 2.0 ** (ka + kb))
+    bad_a = a.clone()
+    bad_a[7, 100] = float("nan")
+    bad_a[200, 3] = float("inf")
+    cb = run(bad_a, b)
+    keep = torch.ones(320, dtype=torch.bool, device="cuda:0")
+    keep[7] = keep[200] = False
+    assert torch.equal(cb[keep], c[keep]) and not torch.isfinite(cb[7]).any() and not torch.isfinite(cb[200]).any()
+    bad_b = b.clone()
+    bad_b[5, 77] = float("nan")
+    cb = run(a, bad_b)
+    keep = torch.ones(200, dtype=torch.bool, device="cuda:0")
+    keep[77] = False
+    assert torch.equal(cb[:, keep], c[:, keep]) and torch.isnan(cb[:, 77]).all()
+
+
 def test_every_headline_variant_meets_the_bound(gpu_device):
     a, b = oc.make_operands(1024, 640, 640, seed=9, w_std=0.02)
     exp = oc.fp64_matmul(a, b)
