@@ -224,6 +224,20 @@ def test_fast_kernels_are_not_chosen_when_offsets_would_overflow():
     assert big >= 0 and "generic" in names[big]
 
 
+def test_slot_kernels_of_the_three_term_fp16_cascade_are_sized_and_bounded():
+    """The fp16 kernels that split both operands into operand slots first: the workspace the library asks for holds
+    both operands' slots (6 bytes per element); they are offered only where a slot buffer stays below 2 GiB (32-bit
+    offsets), K is a multiple of their 32-k stage, and -- the LDS-tiled one -- K is at most 1536."""
+    l = _lib.lib()
+    names = _lib.variant_names()
+    pick16 = lambda M, K, N: names[l.cascmm_select_variant(M, N, K, K, N, N, 0, 1, 3, 0) & 0xFFFF]
+    M, K, N = 2048, 1280, 10240
+    assert l.cascmm_workspace_bytes(M, N, K, _lib.DT_F32, _lib.FMT_FP16, 3, _lib.PROD_TRI) >= 6 * (M * K + K * N)
+    assert pick16(4096, 2560, 5120) == "k64x160x32_f16wk4_fp16x3_tri"       # deep K: never the LDS-tiled kernel
+    assert "_f16" not in pick16(2048, 1296, 1280)                            # K % 32 != 0
+    assert "_f16" not in pick16(65536, 8192, 1280)                           # the slots of A would pass 2 GiB
+
+
 def test_library_tables_are_consistent():
     """Every entry of the measured-cost table names exactly one compiled variant (a renamed kernel
     would otherwise fall back to the analytic estimate without a word), and no variant name repeats."""
