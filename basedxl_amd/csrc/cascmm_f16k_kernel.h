@@ -525,8 +525,12 @@ __global__ __launch_bounds__(F16WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 
   // Stage i, register set u = i % 2 of the left operand.  Every column block is folded into the running sums after
   // the stages with u = 1 (every 64 k of the wave's own: the same k for every block), behind the MFMAs of the block
-  // that follows it, and its next MFMA starts from zero.  Behind the MFMAs of column block ni also: the slots of
-  // block ni - 1 for stage i + 1 (ni = 0: block 4, into the other set) and, ni < 3, a third of the left operand's.
+  // that follows it, and its next MFMA starts from zero.  A block is twelve pairs of MFMAs; behind pair x, between
+  // scheduling fences: one operand of stage i + 1 (two 16-byte loads: the three terms of column block ni - 1, or of
+  // block 4 into the other set when ni = 0, behind pairs 0, 2, 4; ni < 3: two of the six (term, row block) operands
+  // of A behind pairs 6, 8) and a share of the fold -- chunk c of its eight (four accumulator registers of a block)
+  // is read from LDS behind pair c and added and written back behind pair c + 2.
+  f32x4 fold_in[3];
   for (int i0 = 0; i0 < n_own; i0 += 2) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -535,12 +539,38 @@ __global__ __launch_bounds__(F16WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       for (int ni = 0; ni < T::NTL; ++ni) {
         const bool from_zero = u == 0;                      // folded after the stage before
         const bool fold_prev = ni == 0 ? u == 0 : u == 1;   // the block before this one is folded now
+        const int pni = ni == 0 ? T::NTL - 1 : ni - 1;
         auto bop = [&](int t) { return ni < T::NTL - 1 ? b[t][ni < T::NTL - 1 ? ni : 0] : b4[u][t]; };
+        int x = 0;
+        auto gap = [&]() {
+          __builtin_amdgcn_sched_barrier(0);
+          if (x == 0 || x == 2 || x == 4) {
+            if (ni == 0) issue_b4(i + 1, u ^ 1, x >> 1);
+            else issue_b(i + 1, x >> 1, ni - 1);
+          }
+          if (ni < 3 && (x == 6 || x == 8)) {
+            const int o = 2 * ni + (x == 8 ? 1 : 0);
+            issue_a(i + 1, u ^ 1, o >> 1, o & 1);
+          }
+          if (fold_prev) {
+            if (x >= 2 && x <= 9) {
+              const int c = x - 2, mi = c >> 2, r4 = c & 3;
+              const f32x4 v = fold_in[c % 3];
+              *(f32x4*)(own + (mi * T::NTL + pni) * T::BLOCK_BYTES + r4 * 1024) =
+                  (f32x4){v[0] + X[mi][pni][4 * r4], v[1] + X[mi][pni][4 * r4 + 1], v[2] + X[mi][pni][4 * r4 + 2], v[3] + X[mi][pni][4 * r4 + 3]};
+            }
+            if (x <= 7) fold_in[x % 3] = *(const f32x4*)(own + ((x >> 2) * T::NTL + pni) * T::BLOCK_BYTES + (x & 3) * 1024);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          ++x;
+        };
 #define F16WK_PRODUCT(I, J, FIRST)                                                                                        \
-  _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2)                                                                        \
+  _Pragma("unroll") for (int s2 = 0; s2 < 2; ++s2) {                                                                      \
     _Pragma("unroll") for (int mi = 0; mi < T::MT; ++mi)                                                                  \
       X[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f16k_half(a[u][I][mi], s2), f16k_half(bop(J), s2),              \
-                                                         (FIRST) && s2 == 0 && from_zero ? zero : X[mi][ni], 0, 0, 0);
+                                                         (FIRST) && s2 == 0 && from_zero ? zero : X[mi][ni], 0, 0, 0);   \
+    gap();                                                                                                                \
+  }
         F16WK_PRODUCT(0, 2, true)
         F16WK_PRODUCT(1, 1, false)
         F16WK_PRODUCT(2, 0, false)
@@ -548,25 +578,7 @@ __global__ __launch_bounds__(F16WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
         F16WK_PRODUCT(1, 0, false)
         F16WK_PRODUCT(0, 0, false)
 #undef F16WK_PRODUCT
-        if (fold_prev) fold(ni == 0 ? T::NTL - 1 : ni - 1);
-#pragma unroll
-        for (int t = 0; t < T::TERMS; ++t) {
-          if (ni == 0) issue_b4(i + 1, u ^ 1, t);
-          else issue_b(i + 1, t, ni - 1);
-        }
-        if (ni < 3) {
-#pragma unroll
-          for (int x = 2 * ni; x < 2 * ni + 2; ++x) issue_a(i + 1, u ^ 1, x >> 1, x & 1);
-        }
-        // two MFMAs, a load (10, 10, 10, 6, 6 of them)
-        constexpr int kLoads[5] = {10, 10, 10, 6, 6};
-#pragma unroll
-        for (int x = 0; x < 12; ++x) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-          if (x < kLoads[ni]) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
   }
   // What the temporaries still hold.  The loop runs whole trips of two stages, so the last stage had u = 1: blocks
