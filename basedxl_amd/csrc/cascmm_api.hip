@@ -249,12 +249,13 @@ static double variant_cost(int vi, const Problem& q, int count, size_t ws_bytes 
     return us;
   }
   if (v.kind == KIND_F16K) {
-    // stages of 32 k that take what the fp8-rate kernels' stages of 64 k take (the same bytes, the same MFMA
-    // cycles), and the passes around the GEMM: two scale searches, two splits (4 bytes read, 6 written per element)
+    // Stages of 32 k (the K-over-waves kernel: a wave's own stages, in pairs) at the measured 3.0 / 2.45 us with 10 / 8 us
+    // per round beside them (fit: 2048 x {1280, 5120} x 1280, 2048 x 1280 x {3840, 10240}, 8192 x 640 x 5120), and the
+    // two passes around the GEMM: both operands read twice and written once as slots, 14 bytes per element at 5.7 TB/s.
     const double rounds_ = tiles <= kNumCUs ? 1.0 : (double)(int64_t)(tiles / kNumCUs) + ((int64_t)tiles % kNumCUs ? 0.8 : 0.0);
-    const double gemm_us = v.BM == F16WK::BM ? rounds_ * ((double)((q.K / 32 + 7) / 8 * 2) * kF8WKStageUs + kF8WKFixedUs)
-                                             : rounds_ * ((double)(q.K / 32) * f8k64_stage_us(256) + 6.0);
-    return gemm_us + 12.0 + ((double)q.M * q.K + (double)q.K * q.N) * 14.0 / 4.0e6;
+    const double gemm_us = v.BM == F16WK::BM ? rounds_ * ((double)((q.K / 32 + 7) / 8 * 2) * 3.0 + 10.0)
+                                             : rounds_ * ((double)(q.K / 32) * 2.45 + 8.0);
+    return gemm_us + 4.0 + ((double)q.M * q.K + (double)q.K * q.N) * 14.0 / 5.7e6;
   }
   if (info.tuned) {
     const TunedCost& t = *info.tuned;
