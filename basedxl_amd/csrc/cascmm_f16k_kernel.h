@@ -523,22 +523,27 @@ __global__ __launch_bounds__(F16WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       }
   };
 
-  // Stage i, register set u = i % 2 of the left operand.  Every column block is folded into the running sums after
-  // the stages with u = 1 (every 64 k of the wave's own: the same k for every block), behind the MFMAs of the block
+  // The wave's stages run in trips of four, then in trips of two while stages are left (so a wave runs at most one
+  // stage of zeros past its last one); stage u of a trip uses register set u % 2 of the left operand.
+  // Every column block is folded into the running sums after the last stage of a trip (every 128 k of the wave's
+  // own: the same k for every block, and the same whatever zeros are appended to K), behind the MFMAs of the block
   // that follows it, and its next MFMA starts from zero.  A block is twelve pairs of MFMAs; behind pair x, between
   // scheduling fences: one operand of stage i + 1 (two 16-byte loads: the three terms of column block ni - 1, or of
   // block 4 into the other set when ni = 0, behind pairs 0, 2, 4; ni < 3: two of the six (term, row block) operands
   // of A behind pairs 6, 8) and a share of the fold -- chunk c of its eight (four accumulator registers of a block)
   // is read from LDS behind pair c and added and written back behind pair c + 2.
   f32x4 fold_in[3];
-  for (int i0 = 0; i0 < n_own; i0 += 2) {
+  auto trip = [&](int i0, auto fold_tag) {
+    constexpr int FOLD = decltype(fold_tag)::value;
+    static_assert(FOLD == 2 || FOLD == 4, "whole pairs of stages: the register sets alternate");
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int i = i0 + u;
+    for (int uu = 0; uu < FOLD; ++uu) {
+      const int i = i0 + uu;
+      const int u = uu & 1;
 #pragma unroll
       for (int ni = 0; ni < T::NTL; ++ni) {
-        const bool from_zero = u == 0;                      // folded after the stage before
-        const bool fold_prev = ni == 0 ? u == 0 : u == 1;   // the block before this one is folded now
+        const bool from_zero = uu == 0;                             // folded after the stage before
+        const bool fold_prev = ni == 0 ? uu == 0 : uu == FOLD - 1;  // the block before this one is folded now
         const int pni = ni == 0 ? T::NTL - 1 : ni - 1;
         auto bop = [&](int t) { return ni < T::NTL - 1 ? b[t][ni < T::NTL - 1 ? ni : 0] : b4[u][t]; };
         int x = 0;
@@ -580,8 +585,11 @@ __global__ __launch_bounds__(F16WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #undef F16WK_PRODUCT
       }
     }
-  }
-  // What the temporaries still hold.  The loop runs whole trips of two stages, so the last stage had u = 1: blocks
+  };
+  const int n4 = n_own & ~3;
+  for (int i0 = 0; i0 < n4; i0 += 4) trip(i0, std::integral_constant<int, 4>{});
+  for (int i0 = n4; i0 < n_own; i0 += 2) trip(i0, std::integral_constant<int, 2>{});
+  // What the temporaries still hold.  The loop runs whole trips, so the last stage was the last of a trip: blocks
   // 0 .. 3 were folded behind the blocks that followed them, block 4 waits for its fold.
   fold(4);
 
