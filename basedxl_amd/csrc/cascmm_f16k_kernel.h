@@ -452,17 +452,7 @@ __global__ __launch_bounds__(F16WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int tm, tn;
-  {
-    const int total = p.tiles_m * p.tiles_n, per = total >> 3;
-    int id = blockIdx.x;
-    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    const int group = T::GROUP_M * p.tiles_n;
-    const int gi = id / group, first = gi * T::GROUP_M;
-    const int rows = (p.tiles_m - first) < T::GROUP_M ? (p.tiles_m - first) : T::GROUP_M;
-    const int in = id - gi * group;
-    tm = first + in % rows;
-    tn = in / rows;
-  }
+  tile_coords((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn, T::GROUP_M);
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int kus = p.K >> 3;          // 8-k slot columns
   const int ksteps = p.K >> 5;       // 32-k stages

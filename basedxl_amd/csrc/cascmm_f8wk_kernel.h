@@ -39,17 +39,7 @@ __global__ __launch_bounds__(F8WK::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   // tile order as in cascmm_slotk_kernel: one contiguous range of tile ids per XCD, GROUP_M tile rows down
   // before one tile to the right
   int tm, tn;
-  {
-    const int total = p.tiles_m * p.tiles_n, per = total >> 3;
-    int id = blockIdx.x;
-    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    const int group = T::GROUP_M * p.tiles_n;
-    const int gi = id / group, first = gi * T::GROUP_M;
-    const int rows = (p.tiles_m - first) < T::GROUP_M ? (p.tiles_m - first) : T::GROUP_M;
-    const int in = id - gi * group;
-    tm = first + in % rows;
-    tn = in / rows;
-  }
+  tile_coords((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn, T::GROUP_M);
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int kus = p.K >> 4;          // 16-k slot columns
   const int ksteps = p.K >> 6;       // 64-k stages

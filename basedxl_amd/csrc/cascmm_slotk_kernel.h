@@ -45,17 +45,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // contiguous range of tile ids, and ids walk GROUP_M tile rows down before moving one tile to the right:
   // a tile's B slots are 2.5 times its A slots, so the block of tiles that share an L2 is taller than wide.
   int tm, tn;
-  {
-    const int total = p.tiles_m * p.tiles_n, per = total >> 3;
-    int id = blockIdx.x;
-    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    const int group = p.group_m * p.tiles_n;
-    const int gi = id / group, first = gi * p.group_m;
-    const int rows = (p.tiles_m - first) < p.group_m ? (p.tiles_m - first) : p.group_m;
-    const int in = id - gi * group;
-    tm = first + in % rows;
-    tn = in / rows;
-  }
+  tile_coords((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn, p.group_m);
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int kgroups = p.K >> 3;
   const int ksteps = p.K >> 4;
@@ -334,17 +324,7 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   int tm, tn;
-  {
-    const int total = p.tiles_m * p.tiles_n, per = total >> 3;
-    int id = blockIdx.x;
-    if (id < (per << 3)) id = (id & 7) * per + (id >> 3);
-    const int group = p.group_m * p.tiles_n;
-    const int gi = id / group, first = gi * p.group_m;
-    const int rows = (p.tiles_m - first) < p.group_m ? (p.tiles_m - first) : p.group_m;
-    const int in = id - gi * group;
-    tm = first + in % rows;
-    tn = in / rows;
-  }
+  tile_coords((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn, p.group_m);
   const int m0 = tm * T::BM, n0 = tn * T::BN;
   const int ksteps = p.K >> 4;
   // a wave owns every fourth PAIR of 16-k stages (see the kernel above): own stage i = stage 8 (i / 2) + 2 wave + i % 2

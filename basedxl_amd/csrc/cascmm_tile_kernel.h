@@ -104,15 +104,15 @@ struct LdsLayout {
 // resident together on one XCD cover a roughly square block and share both A and B tiles in
 // that L2.
 constexpr int kGroupM = 4;
-__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn, int group_m = kGroupM) {
   const int total = tiles_m * tiles_n;
   const int per = total >> 3;
   int id = bid;
   if (bid < (per << 3)) id = (bid & 7) * per + (bid >> 3);
-  const int group = kGroupM * tiles_n;
+  const int group = group_m * tiles_n;
   const int g = id / group;
-  const int first = g * kGroupM;
-  const int rows = (tiles_m - first) < kGroupM ? (tiles_m - first) : kGroupM;
+  const int first = g * group_m;
+  const int rows = (tiles_m - first) < group_m ? (tiles_m - first) : group_m;
   const int in = id - g * group;
   tm = first + in % rows;
   tn = in / rows;
