@@ -209,6 +209,8 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
             cascaded_lowp_matmul(x["kwave"], w["kwave"]),      # both operands raw
             cascaded_lowp_matmul(x["kwave"], pk),              # raw rows through the LDS ring, weight as slots
             cascaded_lowp_matmul(x["kwave"], pk8),             # three fp8 terms: scale search, split of the rows, K over the waves
+            # three fp16 terms on operand slots: both scale searches, both splits, K over the waves
+            cascaded_lowp_matmul(x["kwave"], w["kwave"], lowp="fp16", terms=3),
         ]
 
     run()                                            # warm-up: workspaces exist before the capture
@@ -227,7 +229,7 @@ def test_every_kind_of_launch_replays_from_a_captured_graph(gpu_device):
         outs = run()
     grown = torch.cuda.memory_allocated() - before
     assert {k: v.data_ptr() for k, v in _workspaces.items()} == ws_before        # no workspace was created or replaced
-    # what the capture allocated: the thirteen results plus the grouped launches' other results and the
+    # what the capture allocated: the fourteen results plus the grouped launches' other results and the
     # two-int exponent tensor, each rounded up to the allocator's 512-byte granule -- far below the
     # 21 MB K-split workspace a capture-time allocation would add
     results = sum(o.numel() * o.element_size() for o in outs)
