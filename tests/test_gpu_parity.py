@@ -527,6 +527,23 @@ def test_fp16_slot_kernels_scale_with_their_operands(gpu_device, name):
     assert torch.equal(cb[:, keep], c[:, keep]) and torch.isnan(cb[:, 77]).all()
 
 
+@pytest.mark.parametrize("name,shape", [("t256x160x32_f16k_fp16x3_tri", (2048, 1280, 10240)), ("k64x160x32_f16wk4_fp16x3_tri", (2048, 5120, 1280)),
+                                        ("k64x160x32_f16wk4_fp16x3_tri", (300, 1312, 200))])
+def test_fp16_slot_kernels_repeat_bit_for_bit(gpu_device, name, shape):
+    """Nothing in these kernels or their passes depends on timing (no atomics; maxima and partial tiles are reduced in a
+    fixed order): twenty launches on the same operands, with other work between them, return the same bits."""
+    M, K, N = shape
+    _say("repeat", name, shape)
+    g = torch.Generator(device="cuda:0").manual_seed(8)
+    a = torch.randn(M, K, device="cuda:0", generator=g)
+    b = torch.randn(K, N, device="cuda:0", generator=g) * 0.02
+    v = _lib.variant_names().index(name)
+    first = cascaded_lowp_matmul(a, b, lowp="fp16", terms=3, variant=v).clone()
+    for _ in range(20):
+        cascaded_lowp_matmul(b.t().contiguous()[:64], b)          # another problem through the same workspace
+        assert torch.equal(cascaded_lowp_matmul(a, b, lowp="fp16", terms=3, variant=v), first)
+
+
 def test_every_headline_variant_meets_the_bound(gpu_device):
     a, b = oc.make_operands(1024, 640, 640, seed=9, w_std=0.02)
     exp = oc.fp64_matmul(a, b)
