@@ -61,8 +61,9 @@ inline __host__ __device__ int64_t f16k_slot_bytes(int64_t rows, int64_t K) {
 }
 
 // the exponent e with max|x| 2^e in (7, 14]
-// (kept within +-60 so that the scales and their product stay normal fp32 numbers: a tensor whose largest
-// element lies outside 2^+-57 is split less finely, not wrongly)
+// (kept within +-60 so that the scales and their product stay normal fp32 numbers: a tensor whose largest element
+// is below 2^-57 is split less finely, and one whose largest element is above 2^64 overflows fp16 in its first
+// term, as the cascade without a tensor scale does above 65504)
 __device__ __forceinline__ int f16k_exp_of_amax(unsigned bits) {
   if (bits == 0) return 0;
   const int e = exp_of_amax(bits) - 5;
