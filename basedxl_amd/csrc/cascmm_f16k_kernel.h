@@ -11,10 +11,11 @@
 // S_i S_j, i + j <= 2, then carries the same factor 2^22 on the true product of the scaled operands, so all six go
 // into one sum and no accumulator per scale class is needed; the store multiplies by 2^-(22 + e_A + e_B).
 //
-// Accumulation.  A result at the fp32 rounding floor is spoilt by every addition into a long running sum, so the
-// twelve MFMAs of a 32 x 32 block over one 32-k stage (six products x two 16-k halves, smallest products first) are
-// chained from zero in a temporary block, and the temporary is added to the block's running sum with VALU
-// additions during the next block's MFMAs: one rounding of the running sum per 32 k instead of twelve.
+// Accumulation.  A result at the fp32 rounding floor is spoilt by every addition into a long running sum, whatever
+// the size of what is added.  The MFMAs of a 32 x 32 block (twelve per 32-k stage: six products x two 16-k halves)
+// are chained in a temporary block over four stages, starting from zero; the temporary is then added to the
+// block's running sum by VALU additions placed behind the MFMAs of the next block: one rounding of the running
+// sum per 128 k instead of 48.
 //
 // Slots: 16 bytes = 8 consecutive k of one row (column) of one stored term, [term][K/8][rows]; a stage is four
 // slot columns, 32 k.  A lane's fragment of a stage is slot columns 2 h and 2 h + 1 (h = lane / 32), eight
@@ -40,8 +41,9 @@ struct F16K {
   static constexpr int A_LOADS = TERMS * KU * BM / 64 / 4; // 12 per wave
   static constexpr int B_LOADS_MAX = 8;                    // 30 instructions over 4 waves: 8, 8, 7, 7
   static constexpr int LOADS = A_LOADS + B_LOADS_MAX;      // 20
-  // The running sum of a block takes one addition per 32 k: beyond this depth its rounding errors would pass those
-  // of the chunked sums the three-term cascade is checked against, and the kernel is not offered.
+  // The running sum of a block takes one addition per 128 k and the temporaries are not chained over more: beyond
+  // this depth the kernel is not offered (its error has been checked against the oracle's up to here; the
+  // K-over-waves kernel, whose waves each see a quarter of K, takes deeper problems).
   static constexpr int MAX_K = 1536;
 };
 
