@@ -107,3 +107,17 @@ def test_noalloc_entry_refuses_what_exceeds_its_scratch_and_runs_what_needs_none
     assert _call(l, l.cascmm_gemm_noalloc, a, b, got, None, lambda s: (s,)) == 0
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+    # the three-term cascades' slot kernels are a choice, not a need: where their operand slots would not fit the
+    # scratch (here 26 MB for fp16 x 3), the call runs on a kernel that splits inside the GEMM, as cascmm_gemm
+    # does when it is given no workspace
+    M, K, N = 2048, 1280, 1280
+    a, b = torch.randn(M, K, device=gpu_device), torch.randn(K, N, device=gpu_device) * 0.02
+    want, got = torch.empty(M, N, device=gpu_device), torch.empty(M, N, device=gpu_device)
+    for fmt in (_lib.FMT_FP16, _lib.FMT_FP8):
+        stream = torch.cuda.current_stream().cuda_stream
+        args = (a.data_ptr(), b.data_ptr(), None, None, M, N, K, K, N, N, _lib.DT_F32, fmt, 3, _lib.PROD_TRI, None)
+        assert l.cascmm_workspace_bytes(M, N, K, _lib.DT_F32, fmt, 3, _lib.PROD_TRI) > SCRATCH_BYTES
+        assert l.cascmm_gemm(*args[:2], want.data_ptr(), *args[3:], None, 0, stream) == 0
+        assert l.cascmm_gemm_noalloc(*args[:2], got.data_ptr(), *args[3:], stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), fmt
