@@ -3,6 +3,7 @@
 // writes the same layout directly; this pass is its stand-alone counterpart).
 #include "cascmm_variants.h"
 #include "cascmm_slotk_kernel.h"
+#include "cascmm_slotn_kernel.h"
 
 namespace cascmm {
 
@@ -69,6 +70,30 @@ static int launch_slotk_variant(const GroupParams& p, hipStream_t stream) {
   return launch_slotk_t<1>(q, stream);
 }
 
+// the 64 x 80 tile of the same design, for problems that make too few 64 x 160 tiles to occupy the chip
+static int launch_slotn_variant(const GroupParams& p, hipStream_t stream) {
+  typedef SlotN T;
+  auto kfn = cascmm_slotn_kernel<0>;
+  if (p.kernel_out) { *p.kernel_out = (const void*)kfn; return CASCMM_OK; }
+  if (p.count != 1 || p.glu || p.k_splits > 1) return CASCMM_ERR_BAD_VARIANT;
+  if (p.K % T::BK != 0 || p.K < T::BK) return CASCMM_ERR_BAD_VARIANT;
+  if ((int64_t)p.M * p.lda * 4 > 0x7FFFFFFF || (int64_t)p.K * p.N * 4 > 0x7FFFFFFF || p.ldc * (int64_t)(T::BM * 4) > 0x7FFFFFFF)
+    return CASCMM_ERR_TOO_LARGE;
+  static LdsFlags lds_set;
+  if (!ensure_lds((const void*)kfn, T::LDS_BYTES, lds_set)) return CASCMM_ERR_LAUNCH;
+  SlotKParams q;
+  memset(&q, 0, sizeof(q));
+  q.a = p.A[0]; q.b_slots = p.B[0]; q.C = (float*)p.C[0]; q.bias = (const float*)p.bias[0];
+  q.M = p.M; q.N = p.N; q.K = p.K; q.lda = p.lda; q.ldc = p.ldc;
+  q.tiles_m = (p.M + T::BM - 1) / T::BM;
+  q.tiles_n = (p.N + T::BN - 1) / T::BN;
+  q.group_m = T::GROUP_M;
+  const int64_t grid = (int64_t)q.tiles_m * q.tiles_n;
+  if (grid <= 0 || grid > 0x7FFFFFFF) return CASCMM_ERR_TOO_LARGE;
+  return launch_kernel(kfn, dim3((unsigned)grid), dim3(T::NT), (size_t)T::LDS_BYTES, stream, q) == hipSuccess ? CASCMM_OK
+                                                                                                              : CASCMM_ERR_LAUNCH;
+}
+
 // both operands raw fp32
 static int launch_rawk_variant(const GroupParams& p, hipStream_t stream) {
   typedef SlotK T;
@@ -99,6 +124,8 @@ static const VariantDesc kChainTable[] = {
      SlotK::LDS_BYTES, true, false, &launch_rawk_variant, false, false},
     {"k64x160x16_wk4_bf16x2_tri_bpre", KIND_SLOTK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, SlotK::BM, SlotK::BN, SlotK::BK, SlotK::NT,
      SlotK::LDS_BYTES, true, false, &launch_slotk_variant, true, false},
+    {"k64x80x32_wk4_bf16x2_tri_bpre", KIND_SLOTK, CASCMM_DT_F32, CASCMM_FMT_BF16, 2, false, SlotN::BM, SlotN::BN, SlotN::BK, SlotN::NT,
+     SlotN::LDS_BYTES, true, false, &launch_slotn_variant, true, false},
 };
 
 const VariantDesc* variants_chain(int* n) {

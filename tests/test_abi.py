@@ -123,6 +123,10 @@ def test_baseline_shapes_get_the_kernels_the_measurements_name():
     assert pick(8192, 640, 5120) == "t256x320x32_w512_bf16x2_tri"                  # cfg5: the 640-stage feed-forward, whole large tiles
     # one 64 x 160 tile per CU and K split over the waves: cfg3's second GEMM and the 1280-channel projections
     assert pick(2048, 5120, 1280) == "k64x160x16_wk4_bf16x2_tri" and pick(2048, 1280, 1280) == "k64x160x16_wk4_bf16x2_tri"
+    # weights kept split, 1024 rows (one GPU's half-latent share): 64 x 160 tiles would occupy half the chip; the 64 x 80
+    # tile of the same design
+    pickp = lambda M, K, N: names[l.cascmm_select_variant_prepared(1, M, N, K, K, N, 0, 0, 2, 0) & 0xFFFF]
+    assert pickp(1024, 1280, 1280) == "k64x80x32_wk4_bf16x2_tri_bpre" and pickp(2048, 1280, 1280) == "k64x160x16_wk4_bf16x2_tri_bpre"
     # three fp8 terms, weights kept split: the tile of the fp8-rate kernel that a sweep over the UNet's
     # shapes measured faster (256 rows where the tiles fill the chip, 128 rows where they would not)
     pick8 = lambda M, K, N: names[l.cascmm_select_variant_prepared(1, M, N, K, K, N, 0, 2, 3, 0) & 0xFFFF]

@@ -326,7 +326,7 @@ def test_chained_feed_forward_module_and_its_fallback(gpu_device, prepared):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("form", ["raw x raw", "raw x slots", "slots x slots"])
+@pytest.mark.parametrize("form", ["raw x raw", "raw x slots", "raw x slots, 64 x 80 tile", "slots x slots"])
 def test_non_finite_operands_poison_their_row_or_column_only_on_the_k_over_waves_kernels(gpu_device, form):
     """As for the other kernels: a NaN or an infinity in A spoils exactly its row, one in B exactly its
     column.  K = 96 leaves the fourth wave of a workgroup without a stage of its own: it multiplies the
@@ -343,6 +343,8 @@ def test_non_finite_operands_poison_their_row_or_column_only_on_the_k_over_waves
             return cascaded_lowp_matmul(ad, bd, variant=names.index("k64x160x16_wk4_bf16x2_tri")).cpu()
         if form == "raw x slots":
             return cascaded_lowp_matmul(ad, PreparedWeight(bd, lowp="bf16", terms=2), variant=names.index("k64x160x16_wk4_bf16x2_tri_bpre")).cpu()
+        if form == "raw x slots, 64 x 80 tile":     # (K = 96: three 32-k stages, again none for the fourth wave)
+            return cascaded_lowp_matmul(ad, PreparedWeight(bd, lowp="bf16", terms=2), variant=names.index("k64x80x32_wk4_bf16x2_tri_bpre")).cpu()
         return cascaded_lowp_matmul_chained(LeftSlots.from_tensor(ad), ChainedWeight(bd)).cpu()
 
     clean = run(a, b)
@@ -364,8 +366,9 @@ def test_non_finite_operands_poison_their_row_or_column_only_on_the_k_over_waves
     bd = b.to(DEV)
     if form == "raw x raw":
         again = cascaded_lowp_matmul(pd, bd, variant=names.index("k64x160x16_wk4_bf16x2_tri"))
-    elif form == "raw x slots":
-        again = cascaded_lowp_matmul(pd, PreparedWeight(bd, lowp="bf16", terms=2), variant=names.index("k64x160x16_wk4_bf16x2_tri_bpre"))
+    elif form.startswith("raw x slots"):
+        name = "k64x80x32_wk4_bf16x2_tri_bpre" if "64 x 80" in form else "k64x160x16_wk4_bf16x2_tri_bpre"
+        again = cascaded_lowp_matmul(pd, PreparedWeight(bd, lowp="bf16", terms=2), variant=names.index(name))
     else:
         again = cascaded_lowp_matmul_chained(LeftSlots.from_tensor(pd), ChainedWeight(bd))
     assert torch.equal(again.cpu(), clean)
@@ -419,6 +422,7 @@ def test_k_over_waves_kernels_repeat_bit_for_bit_when_the_launch_has_several_rou
     p8 = PreparedWeight(b, lowp="fp8", terms=3)
     forms = {"raw": lambda: cascaded_lowp_matmul(a, b, variant=names.index("k64x160x16_wk4_bf16x2_tri")),
              "prepared": lambda: cascaded_lowp_matmul(a, pw, variant=names.index("k64x160x16_wk4_bf16x2_tri_bpre")),
+             "prepared, 64 x 80 tile": lambda: cascaded_lowp_matmul(a, pw, variant=names.index("k64x80x32_wk4_bf16x2_tri_bpre")),
              "slots": lambda: cascaded_lowp_matmul_chained(sl, cw),
              # the fp8-rate kernel of the same design (all loads into registers: the compiler's own waits)
              "fp8 slots": lambda: cascaded_lowp_matmul(a, p8, variant=names.index("k64x160x64_f8k64wk4_fp8x3_tri_bpre"))}

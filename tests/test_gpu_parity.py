@@ -963,6 +963,20 @@ def test_prepared_weights_meet_the_bound(gpu_device, fmt, terms):
     assert torch.equal(outs[0], outs[2])
 
 
+@pytest.mark.parametrize("shape", [(1024, 1280, 1280), (300, 2560, 200), (1024, 5120, 1280)])
+def test_the_small_tile_of_the_k_over_waves_kernel_meets_the_bound(gpu_device, shape):
+    """The 64 x 80 tile (sixteen-wide MFMA blocks) for problems of few tiles, forced by name: whole and ragged tiles,
+    the deepest K of a UNet step."""
+    M, K, N = shape
+    a, b = oc.make_operands(M, K, N, seed=33, w_std=0.02)
+    exp = oc.fp64_matmul(a, b)
+    ref = oc.error_metrics(oc.cascade_matmul_ref(a, b, "bf16", 2, "tri"), exp)
+    w = PreparedWeight(_gpu(b))
+    got = oc.error_metrics(cascaded_lowp_matmul(_gpu(a), w, variant=_lib.variant_names().index("k64x80x32_wk4_bf16x2_tri_bpre")).cpu(), exp)
+    _say("64 x 80 tile", shape, got["rel_fro"] / ref["rel_fro"], got["max_abs"] / ref["max_abs"])
+    assert got["rel_fro"] <= TOL * ref["rel_fro"] and got["max_abs"] <= TOL * ref["max_abs"]
+
+
 def test_prepared_weight_rejects_what_its_kernels_cannot_take(gpu_device):
     w = PreparedWeight(_gpu(torch.randn(40, 64)))      # K = 40: no prepared kernel steps by 8
     with pytest.raises(_lib.CascmmError):
