@@ -12,8 +12,8 @@
 //   B: straight into registers, two stages ahead (the ring of two stage buffers is refilled block by block).
 //   A: raw fp32 rows.  A stage of a row is one 128-byte line; `buffer_load ... lds` brings 64 rows x 128 bytes to
 //      a private ring of the wave (eight loads of 1 KB: eight consecutive lanes fetch the eight 16-byte chunks
-//      of a row, rotated by the row number so that the fragment reads of eight consecutive rows spread over
-//      all banks), three stages ahead; the fragments of the next stage are read and split in registers between
+//      of a row, rotated by a function of half the row number so that the sixteen lanes an LDS read serves
+//      together spread over all banks), three stages ahead; the fragments of the next stage are read and split in registers between
 //      the MFMAs of the current one.
 #pragma once
 #include <type_traits>
@@ -71,17 +71,27 @@ __global__ __launch_bounds__(SlotN::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       __builtin_amdgcn_make_buffer_rsrc((void*)p.a, 0, (int)(a_bytes > 0x7FFFFFFF ? 0x7FFFFFFF : a_bytes), 0x00020000);
   unsigned char* ring = slotn_smem + wave * T::RING;
   // Load j of a stage (0 .. 7) brings rows 8 j + lane / 8 to LDS bytes j * 1024 + 16 lane, i.e. lane % 8 is the
-  // position inside the row's 128 bytes; position pos of row r holds chunk (pos - r) mod 8, and r mod 8 = lane / 8.
-  const int dma_voff = (int)(((int64_t)(m0 + (lane >> 3)) * p.lda + (((lane & 7) - (lane >> 3)) & 7) * 4) * 4);
+  // position inside the row's 128 bytes; position pos of row r holds chunk (pos - rot(h)) mod 8 with h = (r / 2) mod 8
+  // = 4 (j mod 2) + lane / 16.  A 16-byte LDS read is served sixteen lanes at a time, and conflict-free when their
+  // sixteen 16-byte units (8 (r mod 2) + position) differ.  The sixteen are not consecutive lanes: lanes 0-3, 12-15,
+  // 20-23 and 24-27 go together, then 4-7, 8-11, 16-19 and 28-31 (likewise in the upper half of the wave) -- here rows
+  // 0-3 and 12-15 of k group 0 with rows 4-11 of k group 1, whose chunks are two further on.  rot = (1, 3, 0, 2, 4, 6,
+  // 5, 7) gives the row pairs 0, 1, 6, 7 the odd rotations and the pairs 2 .. 5 the even ones, so that either sixteen
+  // cover every unit once (a rotation by h itself reads every fragment in eight passes instead of four: counted).
+  auto rot = [](int h) { return (0x75642031u >> (4 * h)) & 7u; };
+  int dma_voff[2];
+#pragma unroll
+  for (int jp = 0; jp < 2; ++jp)
+    dma_voff[jp] = (int)(((int64_t)(m0 + (lane >> 3)) * p.lda + (((lane & 7) - (int)rot(4 * jp + (lane >> 4))) & 7) * 4) * 4);
   const int dma_rows8 = (int)p.lda * 32;
   auto dma_a = [&](int i, int j) {
     const int koff = i < n_own ? (wave + T::NW * i) * (T::BK * 4) : 0;
-    wavek_load_lds(rar, ring + (i & (T::RA - 1)) * T::A_STAGE + j * 1024, dma_voff, koff + j * dma_rows8);
+    wavek_load_lds(rar, ring + (i & (T::RA - 1)) * T::A_STAGE + j * 1024, dma_voff[j & 1], koff + j * dma_rows8);
   };
   // fragment of lane (l15, kg), row block mb: row 16 mb + l15, chunks 2 kg and 2 kg + 1 at their rotated places
   int a_frag[2];
 #pragma unroll
-  for (int x = 0; x < 2; ++x) a_frag[x] = l15 * 128 + ((2 * kg + x + l15) & 7) * 16;
+  for (int x = 0; x < 2; ++x) a_frag[x] = l15 * 128 + ((2 * kg + x + (int)rot(l15 >> 1)) & 7) * 16;
   f32x4 X[T::MB][2];
   u32x4 Ar[2][T::MB][2];   // [stage parity][row block][term]
   auto read_a = [&](int i, int mb) {
