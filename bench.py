@@ -266,26 +266,38 @@ def bench_kv(dev, check=True):
 
 
 def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False), ("bf16", 2, True, False), ("fp8", 3, True, False),
-                              ("bf16", 2, False, True), ("bf16", 2, True, True), ("bf16", 2, True, "chain")),
+                              ("bf16", 2, False, True), ("bf16", 2, True, True), ("bf16", 2, True, "chain"),
+                              ("bf16", 2, True, True, True)),
                latents=(("full latent", None), ("half-latent share", 64)), forward=True):
     """cfg5: the routed layers of one UNet step.  The module tree is built on the GPU with random
     weights and patched through the config switch; one forward pass records every routed call; those
     calls are then replayed in call order on resident inputs from ONE HIP graph, so the figure is the
     Linear / 1x1-convolution path alone (the convolutions, normalisations and attention of the
-    surrounding model are not part of it; the time of a whole eager forward pass is given beside it)."""
+    surrounding model are not part of it; the time of a whole eager forward pass is given beside it).
+    A fifth element of a cascade tuple asks for a LATER step of a sample: the reference projects the text tokens
+    to cross-attention keys and values on a sample's first denoising step only and keeps them for the other 49
+    (basedxl/modules/attn.py:57,74-78); with it the modules keep theirs, the first pass fills them and the
+    recorded step no longer has those calls (neither their time nor their flops)."""
     import torch
     from basedxl_amd.unet import BasedXLUnet
     from basedxl_amd.unet_skeleton import SDXLUNetSkeleton, distinct_shapes, routed_calls, synthetic_inputs
     from basedxl_amd.utils import BasedXLConfig
 
     rows = []
-    for lowp, terms, prepared, geglu in cascades:
+    for lowp, terms, prepared, geglu, *later in cascades:
+        kv_kept = bool(later and later[0])
         model = SDXLUNetSkeleton(device=dev, seed=SEED)
         chain = geglu == "chain"     # the two GEMMs of every feed-forward block chained (gate in the first one's store, result as slots)
         unet = BasedXLUnet(model, BasedXLConfig(fp16_acc_matmul=True, lowp=lowp, terms=terms, prepared=prepared,
-                                                fuse_geglu=bool(geglu) and not chain, chain_ffn=chain))
+                                                fuse_geglu=bool(geglu) and not chain, chain_ffn=chain, cache_cross_kv=kv_kept))
         for label, latent_rows in latents:
             inp = synthetic_inputs(model, latent=128, latent_rows=latent_rows, seed=SEED, device=dev)
+            if kv_kept:
+                for m in unet.modules():
+                    if hasattr(m, "kv_cache"):
+                        m.reset()
+                with torch.no_grad():
+                    unet(*inp)                      # a sample's first step: fills every cross-attention layer's K/V
             calls = routed_calls(unet, *inp)
             shapes = distinct_shapes(calls)
             gen = torch.Generator(device=dev).manual_seed(SEED)
@@ -314,6 +326,8 @@ def bench_unet(dev, cascades=(("bf16", 2, None, False), ("fp8", 3, None, False),
                          else "value * gelu(gate) in the store of the projection's GEMM (this figure includes the gate)" if geglu
                          else "projection routed as a Linear; the gate stays with torch (two elementwise kernels, in no figure but "
                               "whole_forward_ms_eager)",
+                         "step_of_a_sample": "a later one: text-token keys / values kept from the first step" if kv_kept
+                         else "the first: text tokens projected to keys / values (49 of the reference's 50 steps skip this)",
                          "latent": label, "routed_calls": len(calls), "distinct_shapes": len(shapes),
                          "gflop_fp32_equiv": round(flops * 1e-9, 1), "linear_path_ms_per_step": round(us * 1e-3, 3),
                          "fp32_equiv_tflops": round(flops / us * 1e-6, 1),
@@ -525,7 +539,7 @@ def main():
                          "every step, resident in the Infinity Cache; 8 = every step reads HBM-cold data)")
     ap.add_argument("--unet-select", default="",
                     help="unet only: run one configuration instead of all ten, as cascade:weights:latent, e.g. "
-                         "bf16x2:raw:full, fp8x3:prepared:half, bf16x2:raw+geglu:full, bf16x2:prepared+geglu:full or bf16x2:prepared+chain:full (what a profiler run wants)")
+                         "bf16x2:raw:full, fp8x3:prepared:half, bf16x2:raw+geglu:full, bf16x2:prepared+geglu:full, bf16x2:prepared+geglu+kvkept:full (a later step of a sample: text-token K/V kept from the first) or bf16x2:prepared+chain:full (what a profiler run wants)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size kernel that scales "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -573,8 +587,9 @@ def main():
             if args.unet_select:
                 casc, wts, lat = args.unet_select.split(":")
                 lowp, terms = casc.split("x")
-                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts in ("prepared", "prepared+chain", "prepared+geglu") else False if wts == "raw+geglu" else None,
-                                                "chain" if wts == "prepared+chain" else wts in ("raw+geglu", "prepared+geglu")),),
+                un = bench_unet(dev, cascades=((lowp, int(terms), True if wts in ("prepared", "prepared+chain", "prepared+geglu", "prepared+geglu+kvkept") else False if wts == "raw+geglu" else None,
+                                                "chain" if wts == "prepared+chain" else wts in ("raw+geglu", "prepared+geglu", "prepared+geglu+kvkept"),
+                                                wts == "prepared+geglu+kvkept"),),
                                 latents=(("full latent", None),) if lat == "full" else (("half-latent share", 64),), forward=False)
             else:
                 un = bench_unet(dev)
