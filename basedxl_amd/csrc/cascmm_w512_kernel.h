@@ -268,36 +268,43 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
           const int slot = ni * 2 + k;
           if (slot < T::LOADS) issue1(s + j + T::NS - 1, slot);
         };
-        mm(0); W512_FENCE();
-        if (!BPRE) read_raw(R[cur], st2, n2, 0, 4);
-        W512_FENCE();
-        mm(1); W512_FENCE();
-        if (!BPRE) read_raw(R[cur], st2, n2, 4, 8);
-        dl(0); W512_FENCE();
-        mm(2); W512_FENCE();
-        if (ni < 4) {   // row block ni of the next stage
-          const f32x4 x0 = *(const f32x4*)(st1 + a_frag0 + ni * 2048), x1 = *(const f32x4*)(st1 + a_frag1 + ni * 2048);
+        // What goes between MFMA g and MFMA g + 1 of the block.  A wave alone on its SIMD issues one instruction
+        // every four cycles or so, whatever its kind, and an MFMA holds the matrix pipe for 32: more than six
+        // instructions in a gap leave the pipe waiting.  The sixteen half-splits of the block (three VALU
+        // instructions each: B's in gaps 0 .. 7, A's in gaps 4 .. 11) and the LDS reads and loads are spread so
+        // that no gap holds more than six (2202 shader-clock cycles per stage against 2228 with the LDS reads in
+        // gaps 0 .. 2 and all the splits in gaps 3 .. 10; 1920 are the MFMAs).
+        auto gap = [&](int gi) {
+          if (gi == 0 && ni < 4) {   // row block ni of the next stage
+            const f32x4 x0 = *(const f32x4*)(st1 + a_frag0 + ni * 2048), x1 = *(const f32x4*)(st1 + a_frag1 + ni * 2048);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            RA[e] = x0[e];
-            RA[4 + e] = x1[e];
+            for (int e = 0; e < 4; ++e) {
+              RA[e] = x0[e];
+              RA[4 + e] = x1[e];
+            }
           }
-        }
-        W512_FENCE();
-        mm(3); W512_FENCE();
+          if (!BPRE && gi == 1) read_raw(R[cur], st2, n2, 0, 4);
+          if (!BPRE && gi == 2) read_raw(R[cur], st2, n2, 4, 8);
+          if (!BPRE && gi < 8) {
+            if (gi & 1) split_2(R[nxt], H[nxt], L[nxt], gi >> 1);
+            else split_1(R[nxt], H[nxt], gi >> 1);
+          }
+          if (ni < 4 && gi >= 4) {
+            const int h = gi - 4;
+            if (h & 1) split_2(RA, Af[j ^ 1][0][ni], Af[j ^ 1][1][ni], h >> 1);
+            else split_1(RA, Af[j ^ 1][0][ni], h >> 1);
+          }
+          if (BPRE && gi == 4) read_slot_hi(nxt, stn, n1);     // seven MFMAs before the next block's first
+          if (BPRE && gi == 8) read_slot_lo(nxt, stn, n1);
+          // the stage's nine loads: two per block, apart from each other and in gaps that hold one half-split
+          // (several loads in neighbouring gaps of one block cost 30 cycles each: counted)
+          if (gi == 9) dl(0);
+          if (gi == 10) dl(1);
+        };
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (!BPRE) split_1(R[nxt], H[nxt], e);
-          if (ni < 4) split_1(RA, Af[j ^ 1][0][ni], e);
-          W512_FENCE();
-          mm(4 + 2 * e); W512_FENCE();
-          if (!BPRE) split_2(R[nxt], H[nxt], L[nxt], e);
-          if (ni < 4) split_2(RA, Af[j ^ 1][0][ni], Af[j ^ 1][1][ni], e);
-          if (BPRE && e == 0) read_slot_hi(nxt, stn, n1);     // behind MFMA 4: seven MFMAs before the next block's first
-          if (BPRE && e == 2) read_slot_lo(nxt, stn, n1);
-          if (e == 3) dl(1);
-          W512_FENCE();
-          mm(5 + 2 * e); W512_FENCE();
+        for (int gi = 0; gi < 12; ++gi) {
+          mm(gi); W512_FENCE();
+          gap(gi); W512_FENCE();
         }
       }
     }
