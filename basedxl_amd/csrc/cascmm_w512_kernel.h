@@ -90,23 +90,23 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
   const int ldb_bytes = (int)p.ldb * 4;
 
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)p.A[0], 0, 0x7FFFFFFF, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.B[0], 0, 0x7FFFFFFF, 0x00020000);
+  // (one record fewer than A's: with equal words the compiler keeps one copy of them and rebuilds this descriptor from it
+  // in front of every B load)
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)p.B[0], 0, 0x7FFFFFFE, 0x00020000);
   // per wave and stage: 4 loads of A (16 rows x 64 bytes each; LDS position 4 row + pos holds chunk
   // (pos - row / 4) mod 4 of the row) and 5 loads of B (256 consecutive floats of the stage's [16][320]
   // area)
-  int a_voff[4], a_lds[4], b_voff[5], b_lds[5];
+  int a_voff[4], b_voff[5];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int inst = wave * 4 + j;
     const int row = inst * 16 + (lane >> 2);
     const int chunk = ((lane & 3) - (row >> 2)) & 3;
-    a_lds[j] = inst * 1024;
     a_voff[j] = (int)(((int64_t)(m0 + row) * p.lda + chunk * 4) * 4);
   }
 #pragma unroll
   for (int j = 0; j < 5; ++j) {
     const int inst = wave * 5 + j;
-    b_lds[j] = T::A_STAGE + inst * 1024;
     if (BPRE) {
       // run inst = (term * 2 + k group) * 5 + run of 64 columns; lane = column inside the run
       const int tk = inst / 5, run = inst % 5;
@@ -124,14 +124,32 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
   }
   const int b_step = BPRE ? 2 * p.N * 16 : T::BK * ldb_bytes;   // bytes of B per stage
+  // The loads of a wave land in consecutive kilobytes of LDS: the LDS address is M0 plus the instruction's immediate
+  // offset, so a wave's A loads of a stage share one M0 and differ in the immediate; the immediate moves the memory
+  // address too, which the lane offsets make up for (they stay non-negative: load j starts at least j KB into its
+  // operand).  The fifth B load is 4 KB further, beyond the immediate's range, and takes an M0 of its own.
+#pragma unroll
+  for (int j = 1; j < 4; ++j) {
+    a_voff[j] -= j * 1024;
+    b_voff[j] -= j * 1024;
+  }
   auto issue1 = [&](int step_, int j) {
     const int step = step_ < ksteps - 1 ? step_ : ksteps - 1;
     const int st = step_ % T::NS;
-    if (j < 4)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (w512_lds_ptr)(smem + st * T::STAGE + a_lds[j]), 16, a_voff[j], step * T::BK * 4, 0, 0);
-    else
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (w512_lds_ptr)(smem + st * T::STAGE + b_lds[j - 4]), 16, b_voff[j - 4],
-                                               step * b_step, 0, 0);
+    const w512_lds_ptr al = (w512_lds_ptr)(smem + st * T::STAGE + wave * 4096);
+    const w512_lds_ptr bl = (w512_lds_ptr)(smem + st * T::STAGE + T::A_STAGE + wave * 5120);
+    const int as = step * T::BK * 4, bs = step * b_step;
+    switch (j) {
+      case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, al, 16, a_voff[0], as, 0, 0); break;
+      case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, al, 16, a_voff[1], as, 1024, 0); break;
+      case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, al, 16, a_voff[2], as, 2048, 0); break;
+      case 3: __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, al, 16, a_voff[3], as, 3072, 0); break;
+      case 4: __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, bl, 16, b_voff[0], bs, 0, 0); break;
+      case 5: __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, bl, 16, b_voff[1], bs, 1024, 0); break;
+      case 6: __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, bl, 16, b_voff[2], bs, 2048, 0); break;
+      case 7: __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, bl, 16, b_voff[3], bs, 3072, 0); break;
+      default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (w512_lds_ptr)(smem + st * T::STAGE + T::A_STAGE + wave * 5120 + 4096), 16, b_voff[4], bs, 0, 0); break;
+    }
   };
 
   // fragment addresses (bytes inside a stage)
@@ -274,7 +292,12 @@ __global__ __launch_bounds__(W512::NT) __attribute__((amdgpu_waves_per_eu(1, 1))
         // instructions each: B's in gaps 0 .. 7, A's in gaps 4 .. 11) and the LDS reads and loads are spread so
         // that no gap holds more than six (2202 shader-clock cycles per stage against 2228 with the LDS reads in
         // gaps 0 .. 2 and all the splits in gaps 3 .. 10; 1920 are the MFMAs).
+        // LDS answers in order: one wait at the top of a block covers everything the block before it read (the
+        // compiler would put a wait of its own, an instruction each, in front of the first use of every read),
+        // a second one in gap 4 the block's A fragments (younger than them: the raw B reads of gaps 1 and 2)
         auto gap = [&](int gi) {
+          if (gi == 0) { __builtin_amdgcn_s_waitcnt(0xC07F); W512_FENCE(); }                          // lgkmcnt(0)
+          if (gi == 4 && ni < 4) { __builtin_amdgcn_s_waitcnt(BPRE ? 0xC07F : 0xC47F); W512_FENCE(); }   // lgkmcnt(0) / lgkmcnt(4)
           if (gi == 0 && ni < 4) {   // row block ni of the next stage
             const f32x4 x0 = *(const f32x4*)(st1 + a_frag0 + ni * 2048), x1 = *(const f32x4*)(st1 + a_frag1 + ni * 2048);
 #pragma unroll
