@@ -161,7 +161,7 @@ static const TunedCost kTuned[] = {
     // (2048 x {1280, 5120} x 1280: 21.7 / 64.3 us; 1024 x 1280 x 1280: 17.4 us -- 7 % less than with raw A fetched
     // in half lines, A/B on one box)
     {"k64x160x16_wk4_bf16x2_tri_bpre", 0.71, 8.0, 0.65, 0.95},
-    {"k64x80x32_wk4_bf16x2_tri_bpre", 0.47, 7.0, 0.80, 0.95},
+    {"k64x80x32_wk4_bf16x2_tri_bpre", 0.445, 5.4, 0.69, 0.95},
     // ... both operands raw (2048 x {1280, 5120} x 1280: 24.0 / 77.2 us; 8192 x 2560 x 640, two rounds: 79.3 us)
     {"k64x160x16_wk4_bf16x2_tri", 0.887, 6.3, 0.65, 0.95},
 };

@@ -134,17 +134,51 @@ __global__ __launch_bounds__(SlotN::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
     for (int mb = 0; mb < T::MB; ++mb) split_a(0, mb);
   }
 
-  auto mfma = [&](u32x4 a, u32x4 b, f32x4 c) -> f32x4 {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  // The MFMA as assembly, its accumulator tied to its result in the accumulation registers: left to itself the
+  // compiler gives result and addend different registers and moves the eighty accumulators back into place once per
+  // trip (120 moves per 120 MFMAs, in a loop that is bound by the number of instructions the wave can issue: an MFMA
+  // of this shape holds the matrix pipe for 16 cycles, four instructions' worth).  The compiler's hazard handling does
+  // not see such an MFMA: consecutive ones write different accumulators, and the accumulators are read only after the
+  // loop and a pause (below).
+  auto mfma = [&](const u32x4& a, const u32x4& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   };
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef float f32x2v __attribute__((ext_vector_type(2)));
+  // The split of pair e (elements 2 e, 2 e + 1 of a lane's eight) of row block mb in three steps of two VALU
+  // instructions, one step behind each MFMA: {hi pair, hi of the even element as fp32}, {its residual, hi of the odd
+  // element}, {its residual, lo pair}.
+  unsigned hp = 0;
+  float hf = 0.f;
+  auto split_step = [&](int buf, int mb, int e, int t) {
+    const int q = e >> 1, c0 = (2 * e) & 3, c1 = c0 + 1;
+    if (t == 0) {
+      const f32x2v v = {X[mb][q][c0], X[mb][q][c1]};
+      hp = __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2));
+      Ar[buf][mb][0][e] = hp;
+      hf = __builtin_bit_cast(float, hp << 16);
+    } else if (t == 1) {
+      X[mb][q][c0] = X[mb][q][c0] - hf;
+      hf = __builtin_bit_cast(float, hp & 0xFFFF0000u);
+    } else {
+      const f32x2v r = {X[mb][q][c0], X[mb][q][c1] - hf};
+      Ar[buf][mb][1][e] = __builtin_bit_cast(unsigned, __builtin_convertvector(r, bf16x2));
+    }
+  };
+  auto issue_b1 = [&](int i, int buf, int nb, int t) {
+    const int base = i < n_own ? (wave + T::NW * i) * b_step : b_end;
+    Br[buf][nb][t] = __builtin_bit_cast(u32x4, llvm_raw_buffer_load_v4f32(rb, vb + nb * 256, base + t * b_term, 0));
+  };
+#define SLOTN_FENCE() __builtin_amdgcn_sched_barrier(0)
   // Stage i, buffers u = i % 2.  At its top: the eight loads of A's stage i + AHEAD into the ring (that place was
   // last read during stage i - 2), then the wait for A's stage i + 1 -- requested at the top of stage i + 1 - AHEAD,
   // followed since by the ten B loads of that stage, one whole stage and the eight loads just issued: at most
   // 10 + 18 (AHEAD - 2) + 8 loads may still be outstanding -- and the fragment reads of stage i + 1.  Then the
   // twelve MFMAs of each column block (lo.hi, hi.lo, hi.hi over the four row blocks: consecutive MFMAs on different
-  // accumulators); behind column block nb the two slots of block nb - 1 for stage i + 2 (same buffer: free by
-  // then; block 4 is loaded behind block 0 of the next stage... of this buffer's next use, see below) and, nb >= 1,
-  // the split of row block nb - 1 of stage i + 1.
+  // accumulators).  Behind MFMA g of block nb: a step of the split of row block nb of stage i + 1 (nb < 4; the LDS
+  // answers in order, so one wait in front of the block's first step covers its two reads), and behind the first two
+  // MFMAs one of the two slot loads that refill block nb - 1 for stage i + 2 (its last MFMA has been issued);
+  // block 4's follow the stage's last MFMA.
   for (int i0 = 0; i0 < n_own; i0 += 2) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -154,32 +188,39 @@ __global__ __launch_bounds__(SlotN::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
       {
         constexpr int YOUNGER = 2 * T::NB + 18 * (T::AHEAD - 2) + 8;   // 36
         static_assert(YOUNGER <= 63, "the wait counter has six bits");
-        __builtin_amdgcn_sched_barrier(0);
+        SLOTN_FENCE();
         __builtin_amdgcn_s_waitcnt(0x0F70 | (YOUNGER & 0xF) | ((YOUNGER >> 4) << 14));
       }
 #pragma unroll
       for (int mb = 0; mb < T::MB; ++mb) read_a(i + 1, mb);
-      __builtin_amdgcn_sched_barrier(0);
+      SLOTN_FENCE();
 #pragma unroll
       for (int nb = 0; nb < T::NB; ++nb) {
 #pragma unroll
-        for (int mb = 0; mb < T::MB; ++mb) acc[mb][nb] = mfma(Ar[u][mb][1], Br[u][nb][0], acc[mb][nb]);
-#pragma unroll
-        for (int mb = 0; mb < T::MB; ++mb) acc[mb][nb] = mfma(Ar[u][mb][0], Br[u][nb][1], acc[mb][nb]);
-#pragma unroll
-        for (int mb = 0; mb < T::MB; ++mb) acc[mb][nb] = mfma(Ar[u][mb][0], Br[u][nb][0], acc[mb][nb]);
-        issue_b(i + T::D, u, nb);                       // this block's slots are done with: refill them for stage i + 2
-        if (nb < T::MB) split_a(u ^ 1, nb);
-        // six pairs of MFMAs; one of the two loads behind each of the first two
-#pragma unroll
-        for (int x = 0; x < 6; ++x) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-          if (x < 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        for (int g = 0; g < 12; ++g) {
+          const int prod = g >> 2, mb = g & 3;
+          mfma(prod == 0 ? Ar[u][mb][1] : Ar[u][mb][0], prod == 1 ? Br[u][nb][1] : Br[u][nb][0], acc[mb][nb]);
+          SLOTN_FENCE();
+          if (g == 0) {   // lgkmcnt(6 - 2 nb): the reads of the later row blocks may still be on their way
+            if (nb == 0) __builtin_amdgcn_s_waitcnt(0xC67F);
+            if (nb == 1) __builtin_amdgcn_s_waitcnt(0xC47F);
+            if (nb == 2) __builtin_amdgcn_s_waitcnt(0xC27F);
+            if (nb == 3) __builtin_amdgcn_s_waitcnt(0xC07F);
+            SLOTN_FENCE();
+          }
+          if (nb < T::MB) split_step(u ^ 1, nb, g / 3, g % 3);
+          if (nb >= 1 && g < 2) issue_b1(i + T::D, u, nb - 1, g);
+          SLOTN_FENCE();
         }
       }
-      __builtin_amdgcn_sched_barrier(0);
+      issue_b1(i + T::D, u, T::NB - 1, 0);
+      issue_b1(i + T::D, u, T::NB - 1, 1);
+      SLOTN_FENCE();
     }
   }
+#undef SLOTN_FENCE
+  // the passes of the last MFMAs have to drain before the accumulators are read (the compiler does not know)
+  asm volatile("s_nop 7\n s_nop 7" ::: "memory");
 
   // ---- the four partial tiles meet in LDS: every wave puts its twenty blocks at [wave][block] (16 bytes per
   // lane), wave w then adds the four partial sums of blocks w, w + 4, ... in wave order and stores them ----
