@@ -105,10 +105,16 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   // the part ni (0 .. 3) of own stage i's share of its pair's loads: load 4 sp + ni of pair i / 2, sp = i % 2
   // (passed separately: a constant where i is not); past the wave's last pair: the problem's first pair
   // (finite values for the zero slots of B to multiply, whatever lies beyond K)
+  // The four loads of a stage go to consecutive kilobytes of LDS: one M0 and one scalar offset for the four, the
+  // kilobytes as the instruction's immediate offset, which the lane offset takes back out of the memory address
+  // (lda >= 32, so it stays non-negative; the sum the range check sees is the same).
+  int dma_v[4];
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) dma_v[ni] = dma_voff[ni & 1] + ni * (dma_rows8 - 1024);
   auto dma_a = [&](int i, int ni, int sp) {
-    const int q = i >> 1, j = 4 * sp + ni;
-    const int koff = 2 * q < n_own ? stage_of(2 * q) * (T::BK * 4) : 0;
-    wavek_load_lds(rar, ring + (q & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + j * 1024, dma_voff[ni & 1], koff + j * dma_rows8);
+    const int q = i >> 1;
+    const int koff = (2 * q < n_own ? stage_of(2 * q) * (T::BK * 4) : 0) + 4 * sp * dma_rows8;
+    wavek_load_lds_kb(rar, ring + (q & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + sp * 4096, dma_v[ni], koff, ni);
   };
   // fragment of lane (l31, g), row block mi, stage parity s: row 32 mi + l31, chunks 4 s + 2 g and 4 s + 2 g + 1
   // at their rotated places
@@ -343,8 +349,11 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   f32x4 Bq[D][8];   // [ring buffer][k]: columns 4 l31 .. 4 l31 + 3
   float Bs[D][8];   // column 128 + l31
   auto b_base = [&](int i) { return i < n_own ? stage_of(i) * (T::BK * ldb_bytes) : b_bytes; };
-  auto issue_bq = [&](int i, int buf, int e) { Bq[buf][e] = llvm_raw_buffer_load_v4f32(rb, vbq, b_base(i) + e * ldb_bytes, 0); };
-  auto issue_bs = [&](int i, int buf, int e) { Bs[buf][e] = llvm_raw_buffer_load_f32(rb, vbs, b_base(i) + e * ldb_bytes, 0); };
+  // (the stage's place goes into the lane offset, one addition per stage, and the row's into the scalar offset, eight
+  // values that never change: a scalar offset of stage + row would be one more instruction in front of every load, and
+  // this loop is bound by the number of instructions a wave can issue)
+  auto issue_bq = [&](int i, int buf, int e) { Bq[buf][e] = llvm_raw_buffer_load_v4f32(rb, vbq + b_base(i), e * ldb_bytes, 0); };
+  auto issue_bs = [&](int i, int buf, int e) { Bs[buf][e] = llvm_raw_buffer_load_f32(rb, vbs + b_base(i), e * ldb_bytes, 0); };
   u32x4 H[2], L[2];   // the split operand of the current / next block
   auto split_b = [&](int buf, int ni, int dst) {
     float r[8];
@@ -366,10 +375,13 @@ __global__ __launch_bounds__(SlotK::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
   for (int jp = 0; jp < 2; ++jp)
     dma_voff[jp] = (int)(((int64_t)(m0 + (lane >> 3)) * p.lda + (((lane & 7) - (4 * jp + (lane >> 4))) & 7) * 4) * 4);
   const int dma_rows8 = (int)p.lda * 32;
+  int dma_v[4];   // (as in the kernel above: one M0 and one scalar offset for the four loads of a stage)
+#pragma unroll
+  for (int ni = 0; ni < 4; ++ni) dma_v[ni] = dma_voff[ni & 1] + ni * (dma_rows8 - 1024);
   auto dma_a = [&](int i, int ni, int sp) {   // sp = i % 2
-    const int q = i >> 1, j = 4 * sp + ni;
-    const int koff = 2 * q < n_own ? stage_of(2 * q) * (T::BK * 4) : 0;
-    wavek_load_lds(rar, ring + (q & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + j * 1024, dma_voff[ni & 1], koff + j * dma_rows8);
+    const int q = i >> 1;
+    const int koff = (2 * q < n_own ? stage_of(2 * q) * (T::BK * 4) : 0) + 4 * sp * dma_rows8;
+    wavek_load_lds_kb(rar, ring + (q & (T::RA / 2 - 1)) * (2 * T::A_STAGE) + sp * 4096, dma_v[ni], koff, ni);
   };
   int a_frag[2][2];
 #pragma unroll

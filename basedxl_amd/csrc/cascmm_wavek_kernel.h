@@ -41,6 +41,17 @@ typedef __attribute__((address_space(3))) void* wavek_lds_ptr;
 __device__ __forceinline__ void wavek_load_lds(__amdgpu_buffer_rsrc_t rsrc, unsigned char* dst, int voffset, int soffset) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (wavek_lds_ptr)dst, 16, voffset, soffset, 0, 0);
 }
+// The same with the instruction's immediate offset, kb KB (0 .. 3): it is added to the LDS address AND to the memory
+// address, so loads into consecutive kilobytes of LDS can share one M0 (one scalar instruction less per load) if the
+// lane offset makes up for it on the memory side.
+__device__ __forceinline__ void wavek_load_lds_kb(__amdgpu_buffer_rsrc_t rsrc, unsigned char* dst, int voffset, int soffset, int kb) {
+  switch (kb) {
+    case 0: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (wavek_lds_ptr)dst, 16, voffset, soffset, 0, 0); break;
+    case 1: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (wavek_lds_ptr)dst, 16, voffset, soffset, 1024, 0); break;
+    case 2: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (wavek_lds_ptr)dst, 16, voffset, soffset, 2048, 0); break;
+    default: __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (wavek_lds_ptr)dst, 16, voffset, soffset, 3072, 0); break;
+  }
+}
 
 // Host-checked: fp32 operands, two bf16 terms, products hi.hi + hi.lo + lo.hi; K % 32 == 0,
 // N % (32 NB) == 0, lda % 4 == 0 and A 16-byte aligned, NB == 2: ldb % 2 == 0 and B 8-byte aligned;
