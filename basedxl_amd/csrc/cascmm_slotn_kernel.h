@@ -13,8 +13,8 @@
 //   A: raw fp32 rows.  A stage of a row is one 128-byte line; `buffer_load ... lds` brings 64 rows x 128 bytes to
 //      a private ring of the wave (eight loads of 1 KB: eight consecutive lanes fetch the eight 16-byte chunks
 //      of a row, rotated by a function of half the row number so that the sixteen lanes an LDS read serves
-//      together spread over all banks), three stages ahead; the fragments of the next stage are read and split in registers between
-//      the MFMAs of the current one.
+//      together spread over all banks), three stages ahead; the fragments of the next stage are read and split in
+//      registers between the MFMAs of the current one.
 #pragma once
 #include <type_traits>
 
@@ -122,7 +122,12 @@ __global__ __launch_bounds__(SlotN::NT) __attribute__((amdgpu_waves_per_eu(1, 1)
 #pragma unroll
   for (int mb = 0; mb < T::MB; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < T::NB; ++nb) acc[mb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < T::NB; ++nb) {
+      acc[mb][nb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      // (the zeros are made here, a prologue away from the first MFMA: the MFMAs below are assembly, and the compiler
+      // would not keep the distance a register write needs from an MFMA it does not recognise)
+      asm volatile("" : "+a"(acc[mb][nb]));
+    }
   {
     constexpr int LATER = 8 * (T::AHEAD - 1) + 2 * T::NB * T::D;   // 36
     static_assert(LATER <= 63, "the wait counter has six bits");
