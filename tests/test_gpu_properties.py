@@ -104,6 +104,25 @@ def test_prepared_weight_has_the_same_properties(gpu_device, M, K, N):
     assert torch.equal(cascaded_lowp_matmul(a * 4.0, pw), c * 4.0)
 
 
+@pytest.mark.parametrize("M,K,N", [(1024, 1280, 1280), (1024, 5120, 1280), (300, 2560, 200)])
+def test_the_small_tile_of_the_k_over_waves_kernel_has_the_same_properties(gpu_device, M, K, N):
+    """The 64 x 80 tile, forced by name, on the half-latent share's shapes and a ragged one: rows and columns may be
+    permuted, powers of two factor out, and 32 more k of zeros (one more stage, for one of the four waves) change nothing."""
+    print("64 x 80 tile properties", M, K, N, flush=True)
+    from basedxl_amd import _lib
+    v = _lib.variant_names().index("k64x80x32_wk4_bf16x2_tri_bpre")
+    a, b = _operands(M, K, N, 16)
+    g = torch.Generator(device="cuda:0").manual_seed(17)
+    pr, pc = torch.randperm(M, device="cuda:0", generator=g), torch.randperm(N, device="cuda:0", generator=g)
+    c = cascaded_lowp_matmul(a, PreparedWeight(b), variant=v)
+    assert torch.equal(cascaded_lowp_matmul(a[pr].contiguous(), PreparedWeight(b), variant=v), c[pr])
+    assert torch.equal(cascaded_lowp_matmul(a, PreparedWeight(b[:, pc].contiguous()), variant=v), c[:, pc])
+    assert torch.equal(cascaded_lowp_matmul(a * 4.0, PreparedWeight(b * 0.5), variant=v), c * 2.0)
+    a2 = torch.cat([a, torch.zeros(M, 32, device="cuda:0")], dim=1).contiguous()
+    b2 = torch.cat([b, torch.zeros(32, N, device="cuda:0")], dim=0).contiguous()
+    assert torch.equal(cascaded_lowp_matmul(a2, PreparedWeight(b2), variant=v), c)
+
+
 def test_prepared_weight_takes_rows_that_are_not_16_byte_aligned(gpu_device):
     """A view whose rows start at odd element offsets (row stride K + 3, first element shifted by
     one) gives the same bits as its contiguous copy: the wrapper copies what the prepared kernels
